@@ -1,0 +1,106 @@
+"""Oracle for the softmax branch (sparse-KV causal attention over selected chunks).
+
+TEST INFRASTRUCTURE ONLY -- see oracle/__init__.py.
+
+Restates parallel_nats_attn_fwd_kernel, src/nats/ops/attns/attns.py:62-353, as a
+dense masked softmax.  The visibility mask is the closed form of the kernel's
+two phases (whole attention blocks before the query tile :173-217, the tile's
+own keys with causal / same-block rules :271-340); the same recipe is built in
+torch by the reference's debug script at :2041-2062.
+
+Pins: all-attention types => plain causal attention and all-linear types =>
+block-diagonal causal attention, both checked against
+torch.nn.functional.scaled_dot_product_attention (a library routine) in
+tests/test_oracle_branches.py; a brute-force per-row Python loop checks the mask.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+LOG2E = 1.4426950408889634
+
+
+def visibility_mask(attn_types: torch.Tensor, T: int, block: int, same_block_visible: bool = True) -> torch.Tensor:
+    """attn_types [NB] in {0,1} for ONE (batch, selector head) -> bool [T,T] (rows = queries).
+
+    same_block_visible=True  (modes 'all' / 'attn', COMPUTE_INCOMPLETE_CHUNK_SCORES):
+        M(t,s) = s<=t and (blk(s)==blk(t) or a[blk(s)]==1)
+    same_block_visible=False (modes 'gated_delta_net' / 'mamba'):
+        M(t,s) = a[blk(s)]==1 and t >= (blk(s)+1)*block          (attns.py:318-320)
+    """
+    t = torch.arange(T)
+    blk = t // block
+    a = attn_types.reshape(-1)[blk].bool()                       # per key
+    if same_block_visible:
+        causal = t.view(-1, 1) >= t.view(1, -1)
+        same = blk.view(-1, 1) == blk.view(1, -1)
+        return causal & (same | a.view(1, -1))
+    return a.view(1, -1) & (t.view(-1, 1) >= ((blk + 1) * block).view(1, -1))
+
+
+def softmax_branch(q, k, v, types, scale, block, same_block_visible=True, dtype=torch.float32):
+    """q [B,T,HQ,K], k [B,T,HKV,K], v [B,T,HKV,V], types [B,NB,HN,n_ops] -> (o [B,T,HQ,V], lse [B,T,HQ]).
+
+    lse is in log2 units, m + log2(sum) with scores scaled by scale*log2(e)
+    (attns.py:158-159,346-353); rows that see no key give o = 0, lse = 0
+    (attns.py:343-350).  GQA: kv head = hq // (HQ//HKV); selector head =
+    hq // (HQ//HN) (attns.py:99-101).
+    """
+    B, T, HQ, K = q.shape
+    HKV, V = k.shape[2], v.shape[-1]
+    HN = types.shape[2]
+    G, GN = HQ // HKV, HQ // HN
+    o = torch.zeros(B, T, HQ, V, dtype=dtype)
+    lse = torch.zeros(B, T, HQ, dtype=dtype)
+    a = torch.round(types[..., 0].float())
+    for b in range(B):
+        masks = [visibility_mask(a[b, :, hn], T, block, same_block_visible) for hn in range(HN)]
+        for hq in range(HQ):
+            m = masks[hq // GN]
+            s = (q[b, :, hq].to(dtype) @ k[b, :, hq // G].to(dtype).T) * (scale * LOG2E)
+            s = s.masked_fill(~m, float('-inf'))
+            mx = s.max(-1, keepdim=True)[0]
+            valid = torch.isfinite(mx)
+            mx = torch.where(valid, mx, torch.zeros_like(mx))
+            p = torch.exp2(s - mx)
+            den = p.sum(-1, keepdim=True)
+            den_safe = torch.where(valid, den, torch.ones_like(den))
+            o[b, :, hq] = torch.where(valid, (p @ v[b, :, hq // G].to(dtype)) / den_safe, torch.zeros(1, dtype=dtype))
+            lse[b, :, hq] = torch.where(valid, mx + torch.log2(den_safe), torch.zeros_like(mx)).squeeze(-1)
+    return o, lse
+
+
+def softmax_branch_sdpa(q, k, v, types, scale, block, same_block_visible=True):
+    """Same result through F.scaled_dot_product_attention with an explicit mask
+    (used for the CPU baseline timing and as a library cross-check)."""
+    B, T, HQ, K = q.shape
+    HKV = k.shape[2]
+    HN = types.shape[2]
+    G, GN = HQ // HKV, HQ // HN
+    a = torch.round(types[..., 0].float())
+    mask = torch.stack([
+        torch.stack([visibility_mask(a[b, :, hq // GN], T, block, same_block_visible) for hq in range(HQ)])
+        for b in range(B)])
+    kk = k.repeat_interleave(G, 2) if G > 1 else k
+    vv = v.repeat_interleave(G, 2) if G > 1 else v
+    o = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), kk.transpose(1, 2), vv.transpose(1, 2), attn_mask=mask, scale=scale)
+    o = o.transpose(1, 2)
+    empty = ~mask.any(-1)                                        # [B,HQ,T]
+    if empty.any():
+        o = torch.where(empty.transpose(1, 2).unsqueeze(-1), torch.zeros((), dtype=o.dtype), o)
+    return o
+
+
+def flops(types: torch.Tensor, T: int, block: int, K: int, V: int, heads_per_selector: int) -> float:
+    """Algorithmic FLOPs 2(K+V) * sum_t n_keys(t) for the visibility rule 'all'."""
+    a = torch.round(types[..., 0].float())                       # [B,NB,HN]
+    B, NB, HN = a.shape
+    prior = torch.cumsum(a, 1) - a                               # attention blocks before each block
+    tot = 0.0
+    for c in range(NB):
+        n = min(block, T - c * block)
+        tot += float((n * (n + 1) / 2 + n * block * prior[:, c]).sum())
+    return 2.0 * (K + V) * tot * heads_per_selector

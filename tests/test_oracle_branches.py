@@ -1,0 +1,213 @@
+"""Pins the oracle's softmax / GDN / Mamba branches against each other, against library
+routines and against special cases the mathematics fixes (CPU only)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import linear_branch as lb
+from oracle import mixed, norm_gate, routing
+from oracle import softmax_branch as sb
+
+
+def _inputs(B, T, H, K, V, seed=0, HN=None, block=64, p_attn=0.4):
+    g = torch.Generator().manual_seed(seed)
+    HN = HN or H
+    q = torch.randn(B, T, H, K, generator=g, dtype=torch.float64)
+    k = torch.randn(B, T, H, K, generator=g, dtype=torch.float64)
+    v = torch.randn(B, T, H, V, generator=g, dtype=torch.float64)
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g, dtype=torch.float64))
+    gl = -F.softplus(torch.randn(B, T, H, generator=g, dtype=torch.float64))
+    NB = -(-T // block)
+    lin = (torch.rand(B, NB, HN, generator=g) > p_attn).double()
+    types = torch.stack([1 - lin, lin], -1)
+    types = routing.force_last_block(types)
+    return q, k, v, gl, beta, types
+
+
+def _close(a, b, tol=1e-9):
+    assert (a - b).abs().max().item() < tol, (a - b).abs().max().item()
+
+
+@pytest.mark.parametrize("decay", [True, False])
+@pytest.mark.parametrize("block,T", [(64, 256), (64, 200), (128, 384), (256, 512)])
+def test_gdn_chunked_equals_token_recurrence(decay, block, T):
+    q, k, v, g, beta, types = _inputs(2, T, 4, 16, 24, seed=3, HN=2, block=block)
+    h0 = torch.randn(2, 4, 16, 24, dtype=torch.float64, generator=torch.Generator().manual_seed(9))
+    o1, s1 = lb.gdn_token_recurrence(q, k, v, g, beta, types[..., 1], 0.25, h0, block, decay)
+    o2, s2 = lb.gdn_chunked(q, k, v, g, beta, types[..., 1], 0.25, h0, block, decay, dtype=torch.float64)
+    _close(o1, o2)
+    _close(s1, s2)
+
+
+@pytest.mark.parametrize("decay", [True, False])
+def test_gdn_reference_pipeline_equals_token_recurrence(decay):
+    q, k, v, g, beta, types = _inputs(2, 512, 4, 16, 8, seed=5, HN=2, p_attn=0.6)
+    h0 = torch.randn(2, 4, 16, 8, dtype=torch.float64, generator=torch.Generator().manual_seed(2))
+    o1, s1 = lb.gdn_token_recurrence(q, k, v, g, beta, types[..., 1], 0.3, h0, 64, decay)
+    o2, s2 = lb.gdn_chunked_reference(q, k, v, g, beta, types[..., 1], 0.3, h0, decay)
+    _close(o1, o2)
+    _close(s1, s2)
+
+
+def test_gdn_all_linear_is_textbook_gated_delta_rule():
+    q, k, v, g, beta, types = _inputs(1, 128, 2, 8, 8, seed=7)
+    types = torch.zeros_like(types); types[..., 1] = 1
+    o, S = lb.gdn_chunked(q, k, v, g, beta, types[..., 1], 1.0, None, 64, True, dtype=torch.float64)
+    # textbook: S_t = S_{t-1} e^{g_t} (I - beta_t k_t k_t^T) + beta_t k_t v_t^T  (state as [K,V]: S <- e^g (I - beta k k^T) S + beta k v^T)
+    qn, kn = lb.l2norm(q), lb.l2norm(k)
+    for h in range(2):
+        St = torch.zeros(8, 8, dtype=torch.float64)
+        for t in range(128):
+            kt, vt, bt = kn[0, t, h], v[0, t, h], beta[0, t, h]
+            St = math.exp(g[0, t, h]) * (torch.eye(8, dtype=torch.float64) - bt * torch.outer(kt, kt)) @ St + bt * torch.outer(kt, vt)
+            _close(o[0, t, h], St.T @ qn[0, t, h])
+        _close(S[0, h], St)
+
+
+def test_gdn_g0_beta1_is_plain_delta_rule():
+    q, k, v, g, beta, types = _inputs(1, 64, 1, 8, 4, seed=11)
+    types = torch.zeros_like(types); types[..., 1] = 1
+    o, S = lb.gdn_chunked(q, k, v, torch.zeros_like(g), torch.ones_like(beta), types[..., 1], 1.0, None, 64, True,
+                          dtype=torch.float64)
+    kn = lb.l2norm(k)
+    St = torch.zeros(8, 4, dtype=torch.float64)
+    for t in range(64):
+        kt = kn[0, t, 0]
+        St = St + torch.outer(kt, v[0, t, 0] - St.T @ kt)
+    _close(S[0, 0], St)
+
+
+def test_gdn_masked_inputs_identity():
+    """Final state with non-linear chunks == stock gated delta rule on inputs whose k, v, beta are
+    zeroed on the non-linear chunks (decay still applied there)."""
+    q, k, v, g, beta, types = _inputs(2, 384, 2, 8, 8, seed=13)
+    lin_tok = types[..., 1].repeat_interleave(64, 1)                    # [B,T,HN]
+    all_lin = torch.ones_like(types[..., 1])
+    _, S_mixed = lb.gdn_token_recurrence(q, k, v, g, beta, types[..., 1], 1.0, None, 64, True)
+    _, S_stock = lb.gdn_token_recurrence(q, lb.l2norm(k) * lin_tok[..., None], v * lin_tok[..., None], g, beta * lin_tok,
+                                         all_lin, 1.0, None, 64, True, l2norm_qk=False)
+    _close(S_mixed, S_stock)
+
+
+def test_gdn_split_and_chain():
+    q, k, v, g, beta, types = _inputs(1, 512, 2, 8, 8, seed=17)
+    types[:, 3] = torch.tensor([0., 1.])                                 # block before the split is linear
+    o_full, S_full = lb.gdn_chunked(q, k, v, g, beta, types[..., 1], 0.5, None, 64, True, dtype=torch.float64)
+    cut = 256
+    o_a, S_a = lb.gdn_chunked(q[:, :cut], k[:, :cut], v[:, :cut], g[:, :cut], beta[:, :cut], types[:, :4, :, 1], 0.5, None,
+                              64, True, dtype=torch.float64)
+    o_b, S_b = lb.gdn_chunked(q[:, cut:], k[:, cut:], v[:, cut:], g[:, cut:], beta[:, cut:], types[:, 4:, :, 1], 0.5, S_a,
+                              64, True, dtype=torch.float64)
+    _close(torch.cat([o_a, o_b], 1), o_full)
+    _close(S_b, S_full)
+
+
+def test_all_attention_state_is_decayed_initial_state():
+    q, k, v, g, beta, types = _inputs(1, 256, 2, 8, 8, seed=19)
+    types = torch.zeros_like(types); types[..., 0] = 1
+    types = routing.force_last_block(types)
+    h0 = torch.randn(1, 2, 8, 8, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    for decay in (True, False):
+        # state entering the last block: run only the first three blocks
+        _, S3 = lb.gdn_chunked(q[:, :192], k[:, :192], v[:, :192], g[:, :192], beta[:, :192], types[:, :3, :, 1], 1.0, h0,
+                               64, decay, dtype=torch.float64)
+        expect = h0 * torch.exp(g[:, :192].sum(1))[..., None, None] if decay else h0
+        _close(S3, expect)
+
+
+@pytest.mark.parametrize("decay", [True, False])
+@pytest.mark.parametrize("block,T", [(64, 256), (64, 150), (256, 768)])
+def test_mamba_chunked_equals_token_recurrence(decay, block, T):
+    q, k, v, g, _, types = _inputs(2, T, 4, 16, 8, seed=23, HN=2, block=block)
+    h0 = torch.randn(2, 4, 16, 8, dtype=torch.float64, generator=torch.Generator().manual_seed(4))
+    o1, s1 = lb.mamba_token_recurrence(q, k, v, g, types[..., 1], 1.0, h0, block, decay)
+    o2, s2 = lb.mamba_chunked(q, k, v, g, types[..., 1], 1.0, h0, block, decay, dtype=torch.float64)
+    _close(o1, o2)
+    _close(s1, s2)
+
+
+def test_mamba_all_linear_is_decayed_linear_attention():
+    q, k, v, g, _, types = _inputs(1, 128, 1, 8, 4, seed=29)
+    types = torch.zeros_like(types); types[..., 1] = 1
+    o, _ = lb.mamba_chunked(q, k, v, g, types[..., 1], 1.0, None, 64, True, dtype=torch.float64)
+    G = g[0, :, 0].cumsum(0)
+    W = torch.tril(torch.exp(G[:, None] - G[None, :]) * (q[0, :, 0] @ k[0, :, 0].T))
+    _close(o[0, :, 0], W @ v[0, :, 0])
+
+
+def test_softmax_mask_brute_force():
+    a = torch.tensor([1., 0., 1., 0., 0.])
+    T, block = 5 * 8, 8
+    m = sb.visibility_mask(a, T, block, True)
+    m2 = sb.visibility_mask(a, T, block, False)
+    for t in range(T):
+        for s in range(T):
+            same = (s // block) == (t // block)
+            assert bool(m[t, s]) == (s <= t and (same or a[s // block] == 1))
+            assert bool(m2[t, s]) == (a[s // block] == 1 and t >= (s // block + 1) * block)
+
+
+def test_softmax_special_cases_match_sdpa():
+    g = torch.Generator().manual_seed(31)
+    B, T, HQ, HKV, K, V = 2, 192, 4, 2, 16, 8
+    q = torch.randn(B, T, HQ, K, generator=g); k = torch.randn(B, T, HKV, K, generator=g); v = torch.randn(B, T, HKV, V, generator=g)
+    kk, vv = k.repeat_interleave(2, 2), v.repeat_interleave(2, 2)
+    scale = K ** -0.5
+    # all attention -> plain causal
+    types = torch.zeros(B, 3, 2, 2); types[..., 0] = 1
+    o, lse = sb.softmax_branch(q, k, v, types, scale, 64)
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), kk.transpose(1, 2), vv.transpose(1, 2), is_causal=True, scale=scale).transpose(1, 2)
+    _close(o, ref, 1e-5)
+    s = torch.einsum('bthk,bshk->bhts', q, kk) * scale
+    s = s.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float('-inf'))
+    _close(lse, (torch.logsumexp(s, -1) / math.log(2)).transpose(1, 2), 1e-4)
+    # all linear -> block-diagonal causal
+    types = torch.zeros(B, 3, 2, 2); types[..., 1] = 1
+    o, _ = sb.softmax_branch(q, k, v, types, scale, 64)
+    for c in range(3):
+        sl = slice(64 * c, 64 * c + 64)
+        ref = F.scaled_dot_product_attention(q[:, sl].transpose(1, 2), kk[:, sl].transpose(1, 2), vv[:, sl].transpose(1, 2), is_causal=True, scale=scale).transpose(1, 2)
+        _close(o[:, sl], ref, 1e-5)
+    # random types: explicit-mask SDPA path agrees, in both visibility modes
+    types = (torch.rand(B, 3, 2, 2, generator=g) < 0.5).float()
+    for mode in (True, False):
+        o, lse = sb.softmax_branch(q, k, v, types, scale, 64, mode)
+        _close(o, sb.softmax_branch_sdpa(q, k, v, types, scale, 64, mode), 1e-5)
+    # rows with no visible key give exactly 0 / 0
+    types = torch.zeros(B, 3, 2, 2)
+    o, lse = sb.softmax_branch(q, k, v, types, scale, 64, False)
+    assert float(o.abs().max()) == 0.0 and float(lse.abs().max()) == 0.0
+
+
+def test_softmax_flops_formula():
+    types = torch.zeros(1, 4, 1, 2); types[0, [0, 2], 0, 0] = 1
+    T, block, K, V = 256, 64, 8, 8
+    m = sb.visibility_mask(types[0, :, 0, 0], T, block, True)
+    assert sb.flops(types, T, block, K, V, 1) == 2.0 * (K + V) * float(m.sum())
+
+
+def test_mixed_varlen_is_per_sequence():
+    q, k, v, g, beta, _ = _inputs(1, 320, 2, 8, 8, seed=37)
+    cu = [0, 128, 320]
+    types = (torch.rand(1, 5, 2, 2, generator=torch.Generator().manual_seed(3)) < 0.5).double()
+    types[:, 1] = 1; types[:, 4] = 1
+    o_lin, o_attn, S, _ = mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, types, cu_seqlens=cu,
+                                               ops_for_incomplete_chunks='all', output_final_state=True,
+                                               decay_for_non_gdn_blocks=True, dtype=torch.float64)
+    a, b, Sa, _ = mixed.mixed_attn_gdn(q[:, :128], k[:, :128], v[:, :128], q[:, :128], k[:, :128], v[:, :128], None,
+                                       g[:, :128], beta[:, :128], types[:, :2], ops_for_incomplete_chunks='all',
+                                       output_final_state=True, decay_for_non_gdn_blocks=True, dtype=torch.float64)
+    _close(o_lin[:, :128], a); _close(o_attn[:, :128], b); _close(S[0:1], Sa)
+    assert S.shape == (2, 2, 8, 8)
+
+
+def test_norm_gate_closed_form():
+    g = torch.Generator().manual_seed(41)
+    x1, x2, gate = (torch.randn(2, 5, 3, 16, generator=g) for _ in range(3))
+    xw = torch.softmax(torch.randn(2, 5, 3, 2, generator=g), -1)
+    w1, w2 = torch.randn(16, generator=g), torch.randn(16, generator=g)
+    y = norm_gate.two_input_rmsnorm_gated(x1, x2, gate, xw, w1, w2, eps=1e-5)
+    ref = (F.rms_norm(x1, (16,), w1, 1e-5) * xw[..., :1] + F.rms_norm(x2, (16,), w2, 1e-5) * xw[..., 1:]) * F.silu(gate)
+    _close(y, ref, 1e-5)
