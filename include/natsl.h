@@ -1,0 +1,133 @@
+/*
+ * natsl.h -- C ABI of the MI355X (gfx950) implementation of the NAtS-L token-level hybrid
+ * attention forward path.
+ *
+ * Plain pointers and sizes only: every pointer is DEVICE memory owned by the caller unless a
+ * comment says "host"; tensors are dense, token-major [B,T,H,D] as in the reference
+ * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:49-50 makes its inputs contiguous).  Nothing here
+ * allocates, synchronises with the host or keeps state between calls; work is enqueued on
+ * `stream`.  Each function returns NATSL_OK or a negative natsl_status; natsl_last_error()
+ * gives the message for the calling thread.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference repository root).
+ */
+#ifndef NATSL_H
+#define NATSL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* natsl_stream_t; /* a hipStream_t */
+
+enum natsl_dtype { NATSL_F32 = 0, NATSL_BF16 = 1 };
+
+enum natsl_status {
+  NATSL_OK = 0,
+  NATSL_ERR_INVALID = -1,     /* inconsistent shapes / null pointers */
+  NATSL_ERR_UNSUPPORTED = -2, /* a shape or dtype this build has no kernel for */
+  NATSL_ERR_WORKSPACE = -3,   /* workspace too small */
+  NATSL_ERR_LAUNCH = -4       /* the HIP runtime refused the launch */
+};
+
+/* flags for the linear-recurrent branches */
+enum natsl_flags {
+  NATSL_DECAY_NON_LINEAR = 1, /* decay_for_non_gdn_blocks / decay_for_non_mamba_blocks */
+  NATSL_QK_L2NORM = 2,        /* lattn_use_qk_l2norm_in_kernel */
+  NATSL_INTRA_CHUNK = 4       /* the linear op also scores its own incomplete block ('all', 'gated_delta_net', 'mamba') */
+};
+
+/* One row per packed sequence (cu_seqlens / cu_seqlens_nats of the reference, plus prefix
+ * counts the kernels would otherwise have to scan for).  Pass seqs = NULL, n_seqs = 0 for a
+ * regular [B,T,...] batch.  With a table, B must be 1, T is the packed length, TN the packed
+ * number of selector blocks, and `total_units` is the sum over sequences of the entry point's
+ * work unit (ceil(len/64) chunks for the linear branches and the router, ceil(len/256) query
+ * tiles for the softmax branch); it is ignored for regular batches. */
+typedef struct natsl_seq_row {
+  int32_t bos;       /* first token of the sequence (flat token index) */
+  int32_t eos;       /* one past its last token */
+  int32_t bos_nats;  /* first selector block of the sequence (flat block index) */
+  int32_t chunk_off; /* number of 64-token chunks in earlier sequences */
+  int32_t qtile_off; /* number of 256-row softmax query tiles in earlier sequences */
+  int32_t pad[3];
+} natsl_seq_row;
+
+int natsl_version(void);
+const char* natsl_last_error(void);
+
+/* Block mean of hidden [B,T,D] -> pooled [B,ceil(T/block),D] (same dtype), divisor
+ * min(block, T - c*block).
+ * Replaces mean_pooling (src/nats/ops/utils/pooling.py:26-57,190-207) as called by the layer at
+ * src/nats/layers/natsl_attn_gdn.py:412-417. */
+int natsl_mean_pool(const void* hidden, void* pooled, int B, int T, int D, int block, int dtype,
+                    const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
+
+/* Selector: logits [B,TN,HN,2] -> types [B,TN,HN,2] in the same dtype with values exactly {0,1}
+ * (softmax evaluated in fp32, rounded to the logits dtype, first maximum wins), optionally
+ * forcing the last block of every sequence to 1 for both ops, and n_nats_blocks [B,HN,2] int32.
+ * Replaces hard_softmax (src/nats/layers/natsl_attn_gdn.py:47-61) and the two statements at
+ * src/nats/layers/natsl_attn_gdn.py:553-554. n_nats_blocks may be NULL. */
+int natsl_hard_select(const void* logits, void* types, int32_t* n_nats_blocks, int B, int TN, int HN,
+                      int dtype, int force_last, const natsl_seq_row* seqs, int n_seqs,
+                      int total_units, natsl_stream_t stream);
+
+/* Routing tables derived from types [B,TN,HN,2] (values rounded as the reference does at
+ * src/nats/ops/mixed_ops/mixed_attn_gdn.py:88).  Any output may be NULL.
+ *   nats_block_indices   int32 [B,TN,HN,2]   ascending ids of selected blocks, padded with TN
+ *                                            (mixed_attn_gdn.py:93-97)
+ *   n_nats_blocks        int32 [B,HN,2]      (mixed_attn_gdn.py:99-100)
+ *   linear_chunk_offsets int64 [B*HN+1]      prepare_nats_chunk_offsets (src/nats/ops/nats_util.py:35-64)
+ *   chunk_indices_linear int32 [cap,2]       prepare_nats_block_indices (nats_util.py:6-32); cap must be
+ *                                            >= B*HN*TN*(block/64); rows beyond the total are untouched
+ *   starting_h_idx       int64 [B,ceil(T/64),HN]   compute_starting_idx_for_chunks (nats_util.py:124-162)
+ *   attn_n_iters         int64 [B,ceil(T/128),HN]  compute_attn_n_iters_per_block (nats_util.py:67-121)
+ * The last two are defined for regular batches only (seqs == NULL). */
+int natsl_route(const void* types, int types_dtype, int B, int TN, int HN, int T, int block,
+                int32_t* nats_block_indices, int32_t* n_nats_blocks, int64_t* linear_chunk_offsets,
+                int32_t* chunk_indices_linear, int64_t* starting_h_idx, int64_t* attn_n_iters,
+                const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
+
+/* Softmax branch: causal attention in which a query sees its own block and every earlier block
+ * typed "attention" (same_block_visible = 1), or only earlier attention blocks (= 0).
+ * q [B,T,HQ,K], k [B,T,HKV,K], v [B,T,HKV,V] -> o [B,T,HQ,V] (same dtype), lse [B,T,HQ] fp32 in
+ * log2 units; rows that see no key give o = 0, lse = 0.
+ * Replaces parallel_attn_nats_fwd (src/nats/ops/attns/attns.py:1421-1531, kernel :62-353) as
+ * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:111-117. */
+int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                             const void* types, int types_dtype, const int32_t* nats_block_indices,
+                             const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
+                             int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                             const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
+
+/* Bytes of scratch the two linear-branch entry points need for `total_chunks` 64-token chunks
+ * (sum over sequences of ceil(len/64)) and H heads. */
+size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H);
+
+/* Gated DeltaNet branch, chunked forward.
+ * q,k [B,T,H,K], v [B,T,H,V], beta [B,T,H] in `dtype`; g [B,T,H] fp32 log-decay; h0 / ht
+ * [N,H,K,V] fp32 (either may be NULL) -> o [B,T,H,V] in `dtype`.
+ * Replaces l2norm_fwd + chunk_gated_delta_rule_nats_fwd
+ * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:119-164, src/nats/ops/gated_delta_rule/chunk.py:22-167). */
+int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                        const float* h0, void* o, float* ht, const void* types, int types_dtype, int B,
+                        int T, int H, int HN, int K, int V, int TN, int block, float scale, int flags,
+                        void* workspace, size_t workspace_bytes, int dtype, const natsl_seq_row* seqs,
+                        int n_seqs, int total_units, natsl_stream_t stream);
+
+/* Mamba2-style SSD branch, chunked forward (q = C, k = B, v = X*dt, g = A*dt).
+ * Replaces chunk_mamba2_fwd (src/nats/ops/mamba/chunk.py:21-109) as called at
+ * src/nats/ops/mixed_ops/mixed_attn_mamba.py:140-161. */
+int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* h0,
+                          void* o, float* ht, const void* types, int types_dtype, int B, int T, int H,
+                          int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
+                          size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs,
+                          int total_units, natsl_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NATSL_H */
