@@ -1,0 +1,113 @@
+"""Shared host logic of the two mixed operators."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _capi
+from .attns import parallel_attn_nats_fwd
+from .nats_util import CHUNK_SIZE, PackedSeqs, _seq_args, pack_sequences, route
+
+_attn_streams: dict = {}
+
+
+def _get_attn_stream(device: torch.device) -> torch.cuda.Stream:
+    """One cached side stream per device for the softmax branch (default priority), as the
+    reference does at src/nats/ops/mixed_ops/mixed_attn_mamba.py:26-30,114-124."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _attn_streams:
+        _attn_streams[idx] = torch.cuda.Stream(device=idx)
+    return _attn_streams[idx]
+
+
+def _no_backward(*tensors):
+    if torch.is_grad_enabled() and any(t is not None and torch.is_tensor(t) and t.requires_grad for t in tensors):
+        raise NotImplementedError(
+            "only the forward of the mixed operator is built for gfx950; call it under torch.no_grad() "
+            "or with tensors that do not require grad")
+
+
+def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block: int, flags: int,
+                     output_final_state: bool, seqs: Optional[PackedSeqs]):
+    """Launch the chunked linear branch ('gdn' or 'mamba'); returns (o, final_state or None)."""
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    TN, HN = types.shape[1], types.shape[2]
+    dev = q.device
+    n = seqs.n_seqs if seqs is not None else B
+    total_chunks = seqs.total_chunks if seqs is not None else B * (-(-T // CHUNK_SIZE))
+    L = _capi.lib()
+    ws = torch.empty(L.natsl_linear_workspace_bytes(total_chunks, H), dtype=torch.uint8, device=dev)
+    o = torch.empty(B, T, H, V, dtype=q.dtype, device=dev)
+    ht = torch.empty(n, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
+    if h0 is not None:
+        if tuple(h0.shape) != (n, H, K, V):
+            raise ValueError(f"initial state must have shape {(n, H, K, V)}, got {tuple(h0.shape)}")
+        h0 = h0.to(torch.float32).contiguous()
+    sp, ns, tot = _seq_args(seqs, total_chunks)
+    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
+              block, float(scale), flags, _capi.ptr(ws), ws.numel(), _capi.dtype_code(q.dtype), sp, ns, tot,
+              _capi.stream_ptr(dev))
+    if kind == 'gdn':
+        rc = L.natsl_gdn_chunk_fwd(_capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), _capi.ptr(beta), *common)
+        _capi.check(rc, "natsl_gdn_chunk_fwd")
+    else:
+        rc = L.natsl_mamba_chunk_fwd(_capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), *common)
+        _capi.check(rc, "natsl_mamba_chunk_fwd")
+    return o, ht
+
+
+def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
+                  scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size, attn_sw_size,
+                  attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
+                  incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool):
+    if nats_block_size < CHUNK_SIZE:
+        raise AssertionError("nats_block_size must be at least the compute chunk (64)")   # mixed_attn_gdn.py:90
+    if nats_block_size % CHUNK_SIZE:
+        raise NotImplementedError("nats_block_size must be a multiple of 64")
+    if attn_sw_size is not None:
+        raise NotImplementedError("attn_sw_size is not used by the reference layers and is not built")
+    if use_g_for_attn:
+        raise NotImplementedError("use_g_for_attn is disabled in every reference layer and is not built")
+    if lin_intra and not incomplete_block_start_with_ht:
+        raise NotImplementedError("incomplete_block_start_with_ht=False is not built")
+    if not q_lattn.is_cuda:
+        raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
+    _no_backward(q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types)
+
+    io_dtype = q_lattn.dtype
+    if io_dtype not in (torch.bfloat16, torch.float32):
+        raise NotImplementedError(f"dtype {io_dtype} is not supported (bf16, or fp32 which is computed in bf16)")
+
+    def prep(t):
+        return None if t is None else t.detach().to(torch.bfloat16).contiguous()
+
+    q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, beta = map(prep, (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, beta))
+    g = g.detach().to(torch.float32).contiguous()
+    types = nats_block_types.detach()
+    if types.dtype not in (torch.bfloat16, torch.float32):
+        types = types.float()
+    types = types.contiguous()
+    dev = q_lattn.device
+    T = q_lattn.shape[1]
+    seqs = pack_sequences(cu_seqlens, cu_seqlens_nats, nats_block_size, dev)
+
+    r = route(types, T, nats_block_size, seqs)
+    cur = torch.cuda.current_stream(dev)
+    side = _get_attn_stream(dev)
+    side.wait_stream(cur)
+    with torch.cuda.stream(side):
+        o_attn, _lse, _ = parallel_attn_nats_fwd(
+            q_attn, k_attn, v_attn, types, r['nats_block_indices'], None, scale_attn, nats_block_size,
+            compute_incomplete_chunk_scores=attn_same_block, n_nats_blocks=r['n_nats_blocks'], seqs=seqs)
+    flags = (_capi.DECAY_NON_LINEAR if decay_non_linear else 0) | (_capi.QK_L2NORM if qk_l2norm else 0) | \
+            (_capi.INTRA_CHUNK if lin_intra else 0)
+    o_lin, ht = linear_chunk_fwd(kind, q_lattn, k_lattn, v_lattn, g, beta, initial_state, types, scale_lattn,
+                                 nats_block_size, flags, output_final_state, seqs)
+    cur.wait_stream(side)
+    for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
+        t.record_stream(side)
+    if io_dtype != torch.bfloat16:
+        o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
+    return o_lin, o_attn, ht

@@ -1,0 +1,620 @@
+// Linear-recurrent branches (Gated DeltaNet and Mamba2-style SSD), chunked forward for gfx950.
+//
+// Two kernels per call:
+//
+//   linear_prep_kernel   one workgroup per (64-token chunk, head), fully parallel.  Everything
+//                        that does not depend on the running state: row norms of q and k, the
+//                        chunk-local cumulative log-decay gamma, the two 64x64 Gram products
+//                        k k^T and q k^T on the matrix cores, the unit-lower-triangular solve
+//                        Tm = (I + A)^-1 in LDS, and per-token scale vectors.  It leaves, per
+//                        chunk-head, 17 KiB in the workspace:
+//                          TmB  bf16 [64][64]   Tm * diag(beta)                      (delta rule only)
+//                          P    bf16 [64][64]   scale * tril(q^ k^^T * e^{gamma_i-gamma_j})
+//                          sc   f32  [4][64]    se = e^{gamma} rk, sq = scale rq e^{gamma},
+//                                               sk = rk e^{gamma_last-gamma}, {e^{gamma_last}, gamma_last}
+//                        (rq, rk = reciprocal L2 norms, or 1).
+//
+//   linear_scan_kernel   one workgroup per (sequence, head, 32-wide slice of V) walks the chunks
+//                        in order with the state slice S[K][32] in fp32 registers:
+//                          R = k S;  X = v - se*R;  v_new = TmB X               (delta rule)
+//                          o = sq*(q S) + P v_new
+//                          S <- e^{gamma_last} S + (sk*k)^T v_new               (blocks typed linear)
+//                        q, k, TmB, P reach the matrix cores straight from global memory in
+//                        A-operand layout; only what changes layout goes through LDS (S, X, v_new
+//                        written transposed from the accumulator layout, k read back transposed
+//                        with the transposing LDS load).  Raw q, k are used: the 1/norm factors
+//                        are folded into the per-token scale vectors.
+//                        A block that is not typed linear leaves S rolled back at its end (times
+//                        e^{sum g} when decay is on), which is all the reference's carry logic
+//                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
+#include "natsl_device.h"
+#include "natsl_host.h"
+
+namespace natsl {
+
+struct LinearParams {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  const float* g;
+  const bf16_t* beta;
+  const float* h0;
+  bf16_t* o;
+  float* ht;
+  const void* types;
+  int types_dtype;
+  const SeqRow* seqs;
+  int n_seqs;
+  int B, T, H, HN, V, TN, block;
+  int nt;            // chunks per sequence (regular batch)
+  int total_chunks;
+  float scale;
+  int flags;
+  bf16_t* ws_tm;
+  bf16_t* ws_p;
+  float* ws_sc;
+};
+
+constexpr int C = 64;
+constexpr int BV = 32;
+
+NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
+  float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i]
+                               : bf16_to_f32(reinterpret_cast<const bf16_t*>(types)[i]);
+  return rintf(x) == 1.0f;
+}
+
+// =============================================================================================
+// prep
+// =============================================================================================
+template <int DK, bool DELTA>
+__global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) {
+  constexpr int KP = DK + 8;   // bf16 row pitch
+  constexpr int AP = 68;       // fp32 row pitch of the 64x64 fp32 matrices (16-byte multiple)
+  constexpr int KL = DK / 32;  // 16-byte loads per thread per tile
+  // LDS: the q, k tiles are dead once the Gram products are done; the solve reuses their space
+  constexpr int TILE_BYTES = 2 * C * KP * 2, MAT_BYTES = C * AP * 4;
+  constexpr int REGION0 = DELTA ? (TILE_BYTES > 2 * MAT_BYTES ? TILE_BYTES : 2 * MAT_BYTES) : TILE_BYTES;
+  __shared__ __align__(16) unsigned char region0[REGION0];
+  __shared__ __align__(16) float Am[DELTA ? C * AP : 4];
+  __shared__ float gam[C], rq[C], rk[C], bet[C];
+  bf16_t* Qs = reinterpret_cast<bf16_t*>(region0);
+  bf16_t* Ks = Qs + C * KP;
+  float* Xm = reinterpret_cast<float*>(region0);             // (I+A)^-1, block lower triangular
+  float* Mm = reinterpret_cast<float*>(region0 + MAT_BYTES);  // inner sums of the block merge
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
+  int bos, len, c;
+  if (p.seqs == nullptr) {
+    const int n = gc / p.nt;
+    c = gc - n * p.nt;
+    bos = n * p.T;
+    len = p.T;
+  } else {
+    int n = 0;
+    for (int i = 1; i < p.n_seqs; ++i)
+      if (p.seqs[i].chunk_off <= gc) n = i;
+    c = gc - p.seqs[n].chunk_off;
+    bos = p.seqs[n].bos;
+    len = p.seqs[n].eos - bos;
+  }
+  const int t0 = c * C;
+  const bool l2 = (p.flags & NATSL_QK_L2NORM) != 0;
+
+  // ---- load q, k tiles; row sums of squares from the registers just loaded -----------------
+  {
+    const int row = tid >> 2, seg = tid & 3;
+    const bool ok = t0 + row < len;
+    const size_t off = ((size_t)(bos + t0 + row) * p.H + h) * DK;
+    const u32x4* qr = reinterpret_cast<const u32x4*>(p.q + off);
+    const u32x4* kr = reinterpret_cast<const u32x4*>(p.k + off);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    float sq = 0.f, sk = 0.f;
+#pragma unroll
+    for (int i = 0; i < KL; ++i) {
+      const u32x4 a = ok ? qr[seg + 4 * i] : z, b = ok ? kr[seg + 4 * i] : z;
+      *reinterpret_cast<u32x4*>(Qs + row * KP + (seg + 4 * i) * 8) = a;
+      *reinterpret_cast<u32x4*>(Ks + row * KP + (seg + 4 * i) * 8) = b;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a0 = __uint_as_float(a[j] << 16), a1 = __uint_as_float(a[j] & 0xffff0000u);
+        const float b0 = __uint_as_float(b[j] << 16), b1 = __uint_as_float(b[j] & 0xffff0000u);
+        sq += a0 * a0 + a1 * a1;
+        sk += b0 * b0 + b1 * b1;
+      }
+    }
+    sq += __shfl_xor(sq, 1); sq += __shfl_xor(sq, 2);
+    sk += __shfl_xor(sk, 1); sk += __shfl_xor(sk, 2);
+    if (seg == 0) {
+      rq[row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
+      rk[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
+    }
+  }
+  // ---- gamma = inclusive cumsum of g over the chunk (wave 0), beta -------------------------
+  if (wave == 0) {
+    const bool ok = t0 + lane < len;
+    const size_t gi = (size_t)(bos + t0 + lane) * p.H + h;
+    float x = ok ? p.g[gi] : 0.f;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float y = __shfl_up(x, d);
+      if (lane >= d) x += y;
+    }
+    gam[lane] = x;
+    if (DELTA) bet[lane] = ok ? bf16_to_f32(p.beta[gi]) : 0.f;
+  }
+  __syncthreads();
+
+  const size_t unit = (size_t)gc * p.H + h;
+  bf16_t* Pout = p.ws_p + unit * (C * C);
+  bf16_t* Tout = p.ws_tm + unit * (C * C);
+  float* Sout = p.ws_sc + unit * (4 * C);
+
+  // ---- Gram products on the matrix cores: wave w owns the 32x32 tile (w/2, w%2) ------------
+  {
+    const int ti = wave >> 1, tj = wave & 1, l32 = lane & 31, hf = lane >> 5;
+    if (ti >= tj) {
+      f32x16 gk, gq;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) gk[r] = gq[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < DK / 16; ++s) {
+        const bf16x8 kb = ld8(Ks + (32 * tj + l32) * KP + 16 * s + 8 * hf);
+        const bf16x8 qa = ld8(Qs + (32 * ti + l32) * KP + 16 * s + 8 * hf);
+        gq = mfma32(qa, kb, gq);
+        if (DELTA) {
+          const bf16x8 ka = ld8(Ks + (32 * ti + l32) * KP + 16 * s + 8 * hf);
+          gk = mfma32(ka, kb, gk);
+        }
+      }
+      const int j = 32 * tj + l32;
+      const float gj = gam[j], rkj = rk[j];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 32 * ti + 8 * (r >> 2) + 4 * hf + (r & 3);
+        const float dec = i >= j ? __expf(gam[i] - gj) : 0.f;
+        Pout[i * C + j] = f32_to_bf16(p.scale * rq[i] * rkj * gq[r] * dec);
+        if (DELTA) Am[i * AP + j] = i > j ? bet[i] * rk[i] * rkj * gk[r] * dec : 0.f;
+      }
+    } else {
+      // the strictly upper 32x32 tile is zero
+      const int l32 = lane & 31, hf = lane >> 5;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r >> 2) + 4 * hf + (r & 3), j = 32 + l32;
+        Pout[i * C + j] = 0;
+        if (DELTA) Am[i * AP + j] = 0.f;
+      }
+    }
+  }
+  // ---- per-token scale vectors -------------------------------------------------------------
+  if (wave == 1) {
+    const float gl = gam[C - 1], gt = gam[lane], eg = __expf(gt);
+    float dk = gl - gt;
+    if (!DELTA) dk = fminf(dk, 0.f);  // src/nats/ops/mamba/chunk_h.py:177
+    Sout[lane] = eg * rk[lane];
+    Sout[C + lane] = p.scale * rq[lane] * eg;
+    Sout[2 * C + lane] = rk[lane] * __expf(dk);
+    if (lane == 0) Sout[3 * C] = __expf(gl);
+    if (lane == 1) Sout[3 * C + 1] = gl;
+  }
+  if (!DELTA) return;
+  __syncthreads();
+
+  // ---- Tm = (I + A)^-1, fp32, blocked 4x4 with 16x16 blocks ----------------------------------
+  // diagonal blocks: forward substitution, one (block, column) per lane of wave 0
+  if (wave == 0) {
+    const int b0 = 16 * (lane >> 4), col = lane & 15;
+    float x[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float acc = r == col ? 1.f : 0.f;
+#pragma unroll
+      for (int j4 = 0; j4 < (r + 3) / 4; ++j4) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(Am + (b0 + r) * AP + b0 + 4 * j4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (4 * j4 + e < r) acc -= a[e] * x[4 * j4 + e];
+      }
+      x[r] = acc;
+      Xm[(b0 + r) * AP + b0 + col] = acc;
+    }
+  }
+  __syncthreads();
+  // off-diagonal blocks by block forward substitution, one block diagonal at a time:
+  //   X_ik = -X_ii * sum_{j=k}^{i-1} A_ij X_jk        (i = k + d)
+  {
+    const int r = tid >> 4, cc = tid & 15;
+#pragma unroll
+    for (int d = 1; d < 4; ++d) {
+#pragma unroll
+      for (int k = 0; k + d < 4; ++k) {
+        const int i = k + d;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = k; j < i; ++j)
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(Am + (16 * i + r) * AP + 16 * j + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc += a[e] * Xm[(16 * j + 4 * e4 + e) * AP + 16 * k + cc];
+          }
+        Mm[(16 * i + r) * AP + 16 * k + cc] = acc;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k + d < 4; ++k) {
+        const int i = k + d;
+        float acc = 0.f;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+          const f32x4 a = *reinterpret_cast<const f32x4*>(Xm + (16 * i + r) * AP + 16 * i + 4 * e4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc -= a[e] * Mm[(16 * i + 4 * e4 + e) * AP + 16 * k + cc];
+        }
+        Xm[(16 * i + r) * AP + 16 * k + cc] = acc;
+      }
+      __syncthreads();
+    }
+  }
+  // TmB = Tm * diag(beta), bf16, rows of 16 contiguous elements per thread
+  {
+    const int row = tid >> 2, cb = tid & 3;
+    u32x4 w[2];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = 16 * cb + 2 * e;
+      const float x0 = cb <= (row >> 4) ? Xm[row * AP + j] * bet[j] : 0.f;
+      const float x1 = cb <= (row >> 4) ? Xm[row * AP + j + 1] * bet[j + 1] : 0.f;
+      w[e >> 2][e & 3] = pack_bf16x2(x0, x1);
+    }
+    u32x4* dst = reinterpret_cast<u32x4*>(Tout + row * C + 16 * cb);
+    dst[0] = w[0];
+    dst[1] = w[1];
+  }
+}
+
+// =============================================================================================
+// scan
+// =============================================================================================
+NATSL_DEVICE u32x2 pack4(f32x4 v) {
+  u32x2 w;
+  w[0] = pack_bf16x2(v[0], v[1]);
+  w[1] = pack_bf16x2(v[2], v[3]);
+  return w;
+}
+
+template <int DK, bool DELTA>
+__global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) {
+  constexpr int KS = DK / 32;   // MFMA k-steps over the key dimension
+  constexpr int MT = DK / 64;   // 16-row state tiles per wave
+  constexpr int KP = DK + 8;    // kbuf / ST row pitch (elements)
+  constexpr int VP = BV + 8;    // vbuf row pitch
+  constexpr int XP = C + 8;     // XT / VNT / VTT row pitch
+  __shared__ __align__(16) bf16_t kbuf[2][C * KP];
+  __shared__ __align__(16) bf16_t vbuf[2][C * VP];
+  __shared__ __align__(16) bf16_t ST[BV * KP];
+  __shared__ __align__(16) bf16_t XT[BV * XP];
+  __shared__ __align__(16) bf16_t VNT[BV * XP];
+  __shared__ __align__(16) bf16_t VTT[BV * XP];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int i16 = lane & 15, g4 = lane >> 4;
+
+  // ---- which (sequence, head, V slice): the slices of one chain sit on one XCD --------------
+  const int nsplit = p.V / BV;
+  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int split = slot % nsplit;
+  const int chain = (slot / nsplit) * 8 + xcd;
+  if (chain >= n_chains) return;
+  const int n = chain / p.H, h = chain % p.H, hn = h / (p.H / p.HN);
+  int bos, len, bos_nats, chunk_off;
+  if (p.seqs == nullptr) {
+    bos = n * p.T; len = p.T; bos_nats = n * p.TN; chunk_off = n * p.nt;
+  } else {
+    bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; bos_nats = p.seqs[n].bos_nats; chunk_off = p.seqs[n].chunk_off;
+  }
+  const int NT = (len + C - 1) / C;
+  const int per_blk = p.block / C;
+  const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0;
+  const bool intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
+  const int vcol0 = split * BV;
+
+  const size_t qk_row = (size_t)p.H * DK, v_row = (size_t)p.H * p.V;
+  const bf16_t* qp = p.q + ((size_t)bos * p.H + h) * DK;
+  const bf16_t* kp = p.k + ((size_t)bos * p.H + h) * DK;
+  const bf16_t* vp = p.v + ((size_t)bos * p.H + h) * p.V + vcol0;
+  bf16_t* op = p.o + ((size_t)bos * p.H + h) * p.V + vcol0;
+
+  // ---- state slice in accumulator layout: tile (mi, nn) = rows 16(wave*MT+mi).., cols 16nn.. ---
+  f32x4 S[MT][2], Ssave[MT][2];
+#pragma unroll
+  for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
+        S[mi][nn][r] = p.h0 ? p.h0[((size_t)chain * DK + kd) * p.V + vc] : 0.f;
+        Ssave[mi][nn][r] = 0.f;
+      }
+  auto write_ST = [&]() {
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+      for (int nn = 0; nn < 2; ++nn)
+        *reinterpret_cast<u32x2*>(ST + (16 * nn + i16) * KP + 16 * (wave * MT + mi) + 4 * g4) = pack4(S[mi][nn]);
+  };
+
+  // ---- operand staging ------------------------------------------------------------------------
+  bf16x8 kA[KS], qA[KS], TA[2], PA[2];
+  f32x4 se, sq, sk;
+  float dec = 1.f, glast = 0.f;
+  u32x4 vld;
+  const int a_row = 16 * wave + i16;          // this lane's A-operand row (token within the chunk)
+  const int v_ld_row = tid >> 2, v_ld_seg = tid & 3;
+  auto gload = [&](int c) {
+    const int tok = c * C + a_row;
+    const bool ok = tok < len;
+    const bf16_t* kr = kp + (size_t)tok * qk_row + 8 * g4;
+    const bf16_t* qr = qp + (size_t)tok * qk_row + 8 * g4;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      kA[s] = ok ? ld8(kr + 32 * s) : zero8();
+      qA[s] = ok ? ld8(qr + 32 * s) : zero8();
+    }
+    const size_t unit = (size_t)(chunk_off + c) * p.H + h;
+    const bf16_t* Pm = p.ws_p + unit * (C * C) + a_row * C + 8 * g4;
+    PA[0] = ld8(Pm);
+    PA[1] = ld8(Pm + 32);
+    if (DELTA) {
+      const bf16_t* Tm = p.ws_tm + unit * (C * C) + a_row * C + 8 * g4;
+      TA[0] = ld8(Tm);
+      TA[1] = ld8(Tm + 32);
+    }
+    const float* sc = p.ws_sc + unit * (4 * C);
+    const int r0 = 16 * wave + 4 * g4;
+    se = *reinterpret_cast<const f32x4*>(sc + r0);
+    sq = *reinterpret_cast<const f32x4*>(sc + C + r0);
+    sk = *reinterpret_cast<const f32x4*>(sc + 2 * C + r0);
+    dec = sc[3 * C];
+    glast = sc[3 * C + 1];
+    const int vt = c * C + v_ld_row;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    vld = vt < len ? *reinterpret_cast<const u32x4*>(vp + (size_t)vt * v_row + 8 * v_ld_seg) : z;
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]) = kA[s];
+    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = vld;
+  };
+
+  if (NT > 0) {
+    gload(0);
+    lstore(0);
+  }
+  write_ST();
+  float gsum = 0.f;
+
+  for (int c = 0; c < NT; ++c) {
+    const int buf = c & 1;
+    __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
+
+    // operands of this step, kept while the next step's loads are in flight
+    bf16x8 kC[KS], qC[KS], TC[2], PC[2];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) { kC[s] = kA[s]; qC[s] = qA[s]; }
+    PC[0] = PA[0]; PC[1] = PA[1];
+    if (DELTA) { TC[0] = TA[0]; TC[1] = TA[1]; }
+    const f32x4 seC = se, sqC = sq, skC = sk;
+    const float decC = dec, glC = glast;
+    (void)seC; (void)TC;
+    if (c + 1 < NT) gload(c + 1);
+
+    if (c % per_blk == 0) {
+#pragma unroll
+      for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+        for (int nn = 0; nn < 2; ++nn) Ssave[mi][nn] = S[mi][nn];
+      gsum = 0.f;
+    }
+
+    // (1) R = k S, O1 = q S
+    f32x4 R[2], O1[2];
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) { R[nn] = (f32x4){0.f, 0.f, 0.f, 0.f}; O1[nn] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const bf16x8 sb0 = ld8(ST + i16 * KP + 32 * s + 8 * g4);
+      const bf16x8 sb1 = ld8(ST + (16 + i16) * KP + 32 * s + 8 * g4);
+      if (DELTA) {
+        R[0] = mfma16(kC[s], sb0, R[0]);
+        R[1] = mfma16(kC[s], sb1, R[1]);
+      }
+      O1[0] = mfma16(qC[s], sb0, O1[0]);
+      O1[1] = mfma16(qC[s], sb1, O1[1]);
+    }
+    // (2) v in accumulator layout via the transposing read; X = v - se * R
+    f32x4 VN[2];
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+      const s16x4 vv = lds_tr4(&vbuf[buf][(16 * wave + 4 * g4 + (i16 >> 2)) * VP + 16 * nn + 4 * (i16 & 3)]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) VN[nn][r] = bf16_to_f32((bf16_t)vv[r]);
+    }
+    if (DELTA) {
+#pragma unroll
+      for (int nn = 0; nn < 2; ++nn) {
+        f32x4 X;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - seC[r] * R[nn][r];
+        *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(X);
+      }
+      __syncthreads();
+      // (3) v_new = TmB X
+#pragma unroll
+      for (int nn = 0; nn < 2; ++nn) {
+        VN[nn] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 2; ++s) VN[nn] = mfma16(TC[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
+      }
+    }
+    // (4) v_new and sk * v_new, transposed, for the two products that reduce over tokens
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+      f32x4 vt;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) vt[r] = VN[nn][r] * skC[r];
+      *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(VN[nn]);
+      *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
+    }
+    __syncthreads();
+    // (5) o = sq * O1 + P v_new
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+      f32x4 O;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[r] = O1[nn][r] * sqC[r];
+      if (intra) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) O = mfma16(PC[s], ld8(VNT + (16 * nn + i16) * XP + 32 * s + 8 * g4), O);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int tok = c * C + 16 * wave + 4 * g4 + r;
+        if (tok < len) op[(size_t)tok * v_row + 16 * nn + i16] = f32_to_bf16(O[r]);
+      }
+    }
+    // (6) state update / roll-back
+    const int blk = (c * C) / p.block;
+    const bool is_lin = lin_type(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2 + 1);
+    const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
+    gsum += glC;
+    if (is_lin || !last_of_block) {
+#pragma unroll
+      for (int mi = 0; mi < MT; ++mi) {
+        const int m = wave * MT + mi;
+        bf16x8 kt[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const bf16_t* kb = &kbuf[buf][(32 * s + 8 * g4 + (i16 >> 2)) * KP + 16 * m + 4 * (i16 & 3)];
+          kt[s] = join4(lds_tr4(kb), lds_tr4(kb + 4 * KP));
+        }
+#pragma unroll
+        for (int nn = 0; nn < 2; ++nn) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= decC;
+#pragma unroll
+          for (int s = 0; s < 2; ++s) S[mi][nn] = mfma16(kt[s], ld8(VTT + (16 * nn + i16) * XP + 32 * s + 8 * g4), S[mi][nn]);
+        }
+      }
+    } else {
+      const float f = decay ? __expf(gsum) : 1.f;
+#pragma unroll
+      for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+        for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) S[mi][nn][r] = Ssave[mi][nn][r] * f;
+    }
+    // (7) bf16 copy of the state and the staged k, v tiles for the next step
+    write_ST();
+    if (c + 1 < NT) lstore(buf ^ 1);
+  }
+
+  if (p.ht) {
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+      for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
+          p.ht[((size_t)chain * DK + kd) * p.V + vc] = S[mi][nn][r];
+        }
+  }
+}
+
+constexpr size_t WS_UNIT_BYTES = (size_t)C * C * 2 * 2 + 4 * C * 4;
+
+template <int DK, bool DELTA>
+static int launch_linear(const LinearParams& p, hipStream_t stream, const char* what) {
+  const long long units = (long long)p.total_chunks * p.H;
+  if (units <= 0) return NATSL_OK;
+  hipLaunchKernelGGL((linear_prep_kernel<DK, DELTA>), dim3((unsigned)units), dim3(256), 0, stream, p);
+  int rc = check_launch(what);
+  if (rc != NATSL_OK) return rc;
+  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+  const int grid = 8 * cdiv(n_chains, 8) * (p.V / BV);
+  hipLaunchKernelGGL((linear_scan_kernel<DK, DELTA>), dim3(grid), dim3(256), 0, stream, p);
+  return check_launch(what);
+}
+
+static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
+                      const float* h0, void* o, float* ht, const void* types, int types_dtype, int B, int T, int H, int HN,
+                      int K, int V, int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
+                      int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream) {
+  const char* what = delta ? "natsl_gdn_chunk_fwd" : "natsl_mamba_chunk_fwd";
+  if (!q || !k || !v || !g || !o || !types || (delta && !beta)) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
+  if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
+  if (B <= 0 || T <= 0 || H <= 0 || HN <= 0 || TN <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
+  if (H % HN) return fail(NATSL_ERR_INVALID, "%s: H=%d must be a multiple of HN=%d", what, H, HN);
+  if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
+  if (V % BV || V <= 0) return fail(NATSL_ERR_UNSUPPORTED, "%s: V=%d must be a multiple of %d", what, V, BV);
+  if (seqs ? (B != 1 || n_seqs <= 0 || total_units <= 0) : (TN != cdiv(T, block)))
+    return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
+  LinearParams p;
+  p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.g = g; p.beta = (const bf16_t*)beta;
+  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.types = types; p.types_dtype = types_dtype;
+  p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0;
+  p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block;
+  p.nt = cdiv(T, C);
+  p.total_chunks = seqs ? total_units : B * p.nt;
+  p.scale = scale; p.flags = flags;
+  const size_t units = (size_t)p.total_chunks * H;
+  const size_t need = natsl_linear_workspace_bytes(p.total_chunks, H);
+  if (!workspace || workspace_bytes < need) return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255) return fail(NATSL_ERR_INVALID, "%s: workspace must be 256-byte aligned", what);
+  p.ws_tm = reinterpret_cast<bf16_t*>(workspace);
+  p.ws_p = p.ws_tm + units * (C * C);
+  p.ws_sc = reinterpret_cast<float*>(p.ws_p + units * (C * C));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (delta) {
+    if (K == 128) return launch_linear<128, true>(p, s, what);
+    if (K == 64) return launch_linear<64, true>(p, s, what);
+  } else {
+    if (K == 128) return launch_linear<128, false>(p, s, what);
+    if (K == 64) return launch_linear<64, false>(p, s, what);
+  }
+  return fail(NATSL_ERR_UNSUPPORTED, "%s: key dim K=%d not built (supported: 64, 128)", what, K);
+}
+
+}  // namespace natsl
+
+using namespace natsl;
+
+extern "C" size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H) {
+  if (total_chunks <= 0 || H <= 0) return 0;
+  return (size_t)total_chunks * (size_t)H * WS_UNIT_BYTES;
+}
+
+extern "C" int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                                   const float* h0, void* o, float* ht, const void* types, int types_dtype, int B, int T,
+                                   int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
+                                   size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
+                                   natsl_stream_t stream) {
+  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
+                    workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
+}
+
+extern "C" int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* h0, void* o,
+                                     float* ht, const void* types, int types_dtype, int B, int T, int H, int HN, int K, int V,
+                                     int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
+                                     int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
+                                     natsl_stream_t stream) {
+  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
+                    flags & ~NATSL_QK_L2NORM, workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
+}

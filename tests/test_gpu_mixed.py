@@ -1,0 +1,137 @@
+"""GPU parity: the mixed operators (drop-in API) vs the oracle, at the configurations the path is
+specified on (reduced sizes where the fp32 oracle would take minutes) and through
+size-independent properties at full size."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import mixed, routing as R
+from tests._util import assert_close, make_gates, make_qkv, make_types
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+def _to(*ts):
+    return [None if t is None else t.to(DEV) for t in ts]
+
+
+def _gdn_case(B, T, H, K, V, p_attn, seed, dtype=torch.bfloat16, mode='all', block=64, HN=None, h0=False, cu=None):
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    HN = HN or H
+    q, k, v = make_qkv(B, T, H, K, V, seed, dtype)
+    g, beta = make_gates(B, T, H, seed + 1, dtype)
+    if cu is None:
+        ty = make_types(B, -(-T // block), HN, p_attn, seed + 2, dtype)
+    else:
+        parts = [make_types(1, -(-(b - a) // block), HN, p_attn, seed + 2 + i, dtype) for i, (a, b) in enumerate(zip(cu[:-1], cu[1:]))]
+        ty = torch.cat(parts, 1)
+    n = B if cu is None else len(cu) - 1
+    init = torch.randn(n, H, K, V, generator=torch.Generator().manual_seed(seed + 9)) * 0.5 if h0 else None
+    nb = R.n_blocks(ty.float())
+    qr, kr, vr, br = (x.to(torch.bfloat16) for x in (q, k, v, beta))      # the kernels compute on bf16 operands
+    o_lin_ref, o_attn_ref, S_ref, _ = mixed.mixed_attn_gdn(
+        qr if dtype == torch.bfloat16 else q, kr if dtype == torch.bfloat16 else k, vr if dtype == torch.bfloat16 else v,
+        qr if dtype == torch.bfloat16 else q, kr if dtype == torch.bfloat16 else k, vr if dtype == torch.bfloat16 else v,
+        init, g, br if dtype == torch.bfloat16 else beta, ty, cu_seqlens=cu, nats_block_size=block,
+        ops_for_incomplete_chunks=mode, output_final_state=True, decay_for_non_gdn_blocks=True)
+    qd, kd, vd, gd, bd, tyd, initd, nbd = _to(q, k, v, g, beta, ty, init, nb)
+    cud = None if cu is None else torch.tensor(cu, dtype=torch.int64, device=DEV)
+    with torch.no_grad():
+        o_lin, o_attn, S = nats_mixed_attn_gdn(qd, kd, vd, qd, kd, vd, initd, gd, bd, tyd, nbd, cu_seqlens=cud,
+                                               nats_block_size=block, ops_for_incomplete_chunks=mode,
+                                               output_final_state_gated_delta=True, decay_for_non_gdn_blocks=True)
+    torch.cuda.synchronize()
+    assert o_lin.dtype == dtype and o_attn.dtype == dtype and S.dtype == torch.float32
+    assert_close(o_lin.float(), o_lin_ref, "o_gdn")
+    assert_close(o_attn.float(), o_attn_ref, "o_attn")
+    assert_close(S, S_ref, "final_state")
+
+
+def test_config0_plumbing_fp32():
+    """B=1, T=256, H=2, d_k=d_v=64, chunk 64, fp32 tensors, hard-selected N(0,1) logits, seed 0."""
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    torch.manual_seed(0)
+    B, T, H, D = 1, 256, 2, 64
+    q, k, v = torch.randn(B, T, H, D), torch.randn(B, T, H, D), torch.randn(B, T, H, D)
+    beta = torch.sigmoid(torch.randn(B, T, H))
+    g = -F.softplus(torch.randn(B, T, H))
+    logits = torch.randn(B, T // 64, H, 2)
+    ty_ref = R.force_last_block(R.hard_select(logits))
+    ty, nb = nats_util.hard_select(logits.to(DEV), force_last_block=True)
+    assert torch.equal(ty.cpu(), ty_ref) and torch.equal(nb.cpu(), R.n_blocks(ty_ref))
+    o_lin_ref, o_attn_ref, S_ref, _ = mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty_ref, ops_for_incomplete_chunks='all',
+                                                           output_final_state=True, decay_for_non_gdn_blocks=True)
+    with torch.no_grad():
+        o_lin, o_attn, S = nats_mixed_attn_gdn(*_to(q, k, v, q, k, v), None, g.to(DEV), beta.to(DEV), ty, nb,
+                                               ops_for_incomplete_chunks='all', output_final_state_gated_delta=True,
+                                               decay_for_non_gdn_blocks=True)
+    assert o_lin.dtype == torch.float32
+    assert_close(o_lin, o_lin_ref, "o_gdn"); assert_close(o_attn, o_attn_ref, "o_attn"); assert_close(S, S_ref, "final_state")
+
+
+def test_config1_gdn_only_reduced():
+    """all chunks linear, K=V=128, H=16 (T reduced from 4096 to 1024 for the fp32 oracle)."""
+    _gdn_case(2, 1024, 16, 128, 128, 0.0, seed=1)
+
+
+def test_config2_hybrid_reduced():
+    """25% softmax chunks, K=V=128, H=16 (B, T reduced from 8 x 8192)."""
+    _gdn_case(1, 2048, 16, 128, 128, 0.25, seed=2)
+
+
+@pytest.mark.parametrize("mode", ['attn', 'gated_delta_net'])
+def test_modes(mode):
+    _gdn_case(1, 512, 4, 128, 128, 0.4, seed=3, mode=mode)
+
+
+def test_selector_head_groups_and_initial_state():
+    _gdn_case(2, 512, 8, 64, 64, 0.4, seed=4, HN=2, h0=True)
+
+
+def test_packed_sequences_reset_state():
+    """config 3's packed batch shape (lengths 8192/16384/16384/24576) scaled by 1/64."""
+    _gdn_case(1, 1024, 4, 128, 128, 0.1, seed=5, cu=[0, 128, 384, 640, 1024], h0=True)
+    _gdn_case(1, 700, 2, 64, 64, 0.3, seed=6, cu=[0, 100, 357, 700])          # ragged sequence lengths
+
+
+def test_mamba_config4_reduced():
+    """Mamba2 hybrid: heads of dim 64, state 128, selector block 256, one B/C group shared by the heads."""
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
+    torch.manual_seed(0)
+    B, T, H, P, N, block = 2, 2048, 8, 64, 128, 256
+    X = torch.randn(B, T, H, P)
+    dt = F.softplus(torch.randn(B, T, H) - 4)
+    A = -torch.exp(torch.rand(H) * torch.log(torch.tensor(16.0)))
+    Bm = F.normalize(torch.randn(B, T, 1, N), dim=-1).expand(B, T, H, N)
+    Cm = F.normalize(torch.randn(B, T, 1, N), dim=-1).expand(B, T, H, N)
+    g = A * dt
+    v_attn = X.bfloat16()
+    v = (X * dt[..., None]).bfloat16()
+    q, k = Cm.bfloat16().contiguous(), Bm.bfloat16().contiguous()
+    ty = make_types(B, T // block, H, 0.25, 7, torch.bfloat16)
+    nb = R.n_blocks(ty.float())
+    o_ref, oa_ref, S_ref, _ = mixed.mixed_attn_mamba(q, k, v_attn, q, k, v, None, g, ty, scale_lattn=1, nats_block_size=block,
+                                                     ops_for_incomplete_chunks='all', output_final_state=True,
+                                                     decay_for_non_mamba_blocks=True)
+    with torch.no_grad():
+        o, oa, S = nats_mixed_attn_mamba(*_to(q, k, v_attn, q, k, v), None, g.to(DEV), ty.to(DEV), nb.to(DEV), scale_lattn=1,
+                                         nats_block_size=block, ops_for_incomplete_chunks='all', output_final_state_mamba=True,
+                                         decay_for_non_mamba_blocks=True)
+    assert_close(o.float(), o_ref, "o_mamba"); assert_close(oa.float(), oa_ref, "o_attn"); assert_close(S, S_ref, "final_state")
+
+
+def test_errors_mirror_reference():
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    q, k, v = (t.to(DEV) for t in make_qkv(1, 128, 2, 64, 64, 0))
+    g, beta = (t.to(DEV) for t in make_gates(1, 128, 2, 1))
+    ty = make_types(1, 2, 2, 0.5, 2, torch.bfloat16).to(DEV)
+    with pytest.raises(KeyError):
+        nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, ops_for_incomplete_chunks='nope')
+    with pytest.raises(AssertionError):
+        nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, nats_block_size=32)
+    with pytest.raises(NotImplementedError):
+        nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, attn_sw_size=128)
+    with pytest.raises(NotImplementedError):
+        nats_mixed_attn_gdn(q.requires_grad_(), k, v, q, k, v, None, g, beta, ty, None)
