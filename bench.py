@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the NAtS-L hybrid-layer forward (selector + routing + softmax branch + Gated DeltaNet
+branch) on one MI355X.  A step is one pass of that path over one synthetic batch resident in HBM.
+
+Prints ONE JSON line: tokens/s of the whole step, the roofline of the dominant kernel (the sparse
+softmax kernel, MFMA-bound) from HIP events recorded on the stream it is launched on, and a
+host-CPU baseline (the fp32 oracle on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: B, T, H, K, V, attention rate, selector block
+    "hybrid_gdn_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
+    "gdn_only_B4_T4096_H16_d128": dict(B=4, T=4096, H=16, K=128, V=128, p_attn=0.0, block=64),
+    "hybrid_gdn_B1_T65536_H32_d128_p10": dict(B=1, T=65536, H=32, K=128, V=128, p_attn=0.10, block=64),
+}
+PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
+PEAK_HBM_GBS = 8000.0
+
+
+def selector_bias(p_attn):
+    """bias on the linear op's logit so that P(attention) = p_attn for N(0,1) logit pairs: b = -sqrt(2)*Phi^-1(p)."""
+    if p_attn <= 0.0:
+        return 30.0
+    if p_attn >= 1.0:
+        return -30.0
+    from statistics import NormalDist
+    return -math.sqrt(2.0) * NormalDist().inv_cdf(p_attn)
+
+
+def make_inputs(w, torch, device):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(0)
+    B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
+    q = torch.randn(B, T, H, K, generator=g).bfloat16()
+    k = torch.randn(B, T, H, K, generator=g).bfloat16()
+    v = torch.randn(B, T, H, V, generator=g).bfloat16()
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g)).bfloat16()
+    gl = -F.softplus(torch.randn(B, T, H, generator=g))
+    logits = torch.randn(B, T // w["block"], H, 2, generator=g)
+    logits[..., 1] += selector_bias(w["p_attn"])
+    logits = logits.bfloat16()
+    host = dict(q=q, k=k, v=v, beta=beta, g=gl, logits=logits)
+    dev = {n: t.to(device) for n, t in host.items()}
+    return host, dev
+
+
+def softmax_flops(types, T, block, K, V):
+    """2(K+V) * sum over queries of visible keys, mode 'all': own block causally + earlier attention blocks."""
+    a = types[..., 0].float().round()                     # [B,NB,HN]
+    prior = a.cumsum(1) - a
+    n = float(block)
+    return 2.0 * (K + V) * float((n * (n + 1) / 2 + n * block * prior).sum())
+
+
+def gdn_flops(types, K, V, C=64):
+    lin = types[..., 1].float().round()
+    n_all, n_lin = float(lin.numel()), float(lin.sum())
+    per = 2 * C * C * (3 * K + 2 * V) + 6 * C * K * V + (2.0 / 3.0) * C ** 3
+    return per * n_all - 2 * C * K * V * (n_all - n_lin)
+
+
+def cpu_baseline(host, w, types_host, torch, max_heads=None):
+    """fp32 oracle on the B=1 slice of the workload (all heads unless max_heads), on the host cores."""
+    from oracle import mixed
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(threads)
+    H = w["H"] if max_heads is None else min(w["H"], max_heads)
+    sl = lambda t: t[:1, :, :H].contiguous()
+    q, k, v, beta, g = (sl(host[n]) for n in ("q", "k", "v", "beta", "g"))
+    ty = types_host[:1, :, :H].contiguous()
+    t0 = time.perf_counter()
+    mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, ops_for_incomplete_chunks='all', output_final_state=True,
+                         decay_for_non_gdn_blocks=True, nats_block_size=w["block"])
+    dt = time.perf_counter() - t0
+    tok_s = w["T"] / dt * (H / w["H"])
+    sample = f"B=1 slice (of {w['B']}), {H} of {w['H']} heads, full T={w['T']}; {dt:.1f} s of fp32 torch-CPU oracle, scaled per head"
+    return dict(value=tok_s, unit="tokens/s", cores=threads, kind="port", sample=sample)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-heads", type=int, default=4, help="heads of the B=1 slice timed on the CPU")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path shards over (batch, head) with no communication and every box has one "
+              "GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    device = torch.device("cuda:0")
+    w = WORKLOADS[args.workload]
+    host, dev = make_inputs(w, torch, device)
+
+    events = []
+
+    def hook(name, stream):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(stream)
+        events.append((name, ev))
+
+    def step():
+        ty, nb = nats_util.hard_select(dev["logits"], force_last_block=True)
+        return nats_mixed_attn_gdn(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v"], None, dev["g"], dev["beta"], ty,
+                                   nb, nats_block_size=w["block"], ops_for_incomplete_chunks="all",
+                                   output_final_state_gated_delta=True, decay_for_non_gdn_blocks=True), ty
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        _mixed_common.TIMING_HOOK = hook
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out, ty = step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        _mixed_common.TIMING_HOOK = None
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    tokens = w["B"] * w["T"]
+    value = tokens / (ms_per_step * 1e-3)
+
+    def avg_ms(tag):
+        starts = [e for n, e in events if n == tag + ":start"]
+        ends = [e for n, e in events if n == tag + ":end"]
+        return sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / max(1, len(starts))
+
+    sm_ms, lin_ms = avg_ms("softmax"), avg_ms("linear")
+    types_host = ty.cpu()
+    f_attn = softmax_flops(types_host, w["T"], w["block"], w["K"], w["V"])
+    f_gdn = gdn_flops(types_host, w["K"], w["V"])
+    if f_attn >= f_gdn:
+        achieved = f_attn / (sm_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", kernel="softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
+                    unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=None, launch_ms=sm_ms,
+                    algorithmic_flops=f_attn)
+    else:
+        # GDN-only workload: HBM-bound; algorithmic bytes = q,k,v read + o written + g,beta + final state
+        B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
+        nbytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * 6 + B * H * K * V * 4
+        achieved = nbytes / (lin_ms * 1e-3) / 1e9
+        roof = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=achieved, peak=PEAK_HBM_GBS,
+                    unit="GB/s", frac=achieved / PEAK_HBM_GBS, traffic=None, launch_ms=lin_ms, algorithmic_bytes=nbytes)
+
+    rec = dict(
+        metric="hybrid-layer fwd tokens/sec @T=8192,H=16,d=128 bf16; % of MFMA/HBM roofline",
+        value=value, unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step,
+        higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+        config=dict(workload=args.workload, **w, attn_fraction=float(types_host[..., 0].float().mean()),
+                    softmax_ms=sm_ms, linear_ms=lin_ms, step_flops=f_attn + f_gdn,
+                    step_frac_of_mfma_peak=(f_attn + f_gdn) / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS),
+        roofline=roof,
+    )
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(host, w, types_host, torch, max_heads=args.cpu_heads)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

@@ -127,6 +127,15 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
                           size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs,
                           int total_units, natsl_stream_t stream);
 
+/* Layer tail: y = (rms(x1)*w1*xw[...,0] + rms(x2)*w2*xw[...,1]) * gate*sigmoid(gate) with
+ * rms(x) = x*rsqrt(mean(x^2)+eps); x1, x2, gate, y [rows, D] and x_weights [rows, 2] in `dtype`,
+ * w1, w2 [D] in `w_dtype`.
+ * Replaces the forward of FusedMultiInputRMSNormGated (src/nats/modules/fused_norm_gate.py:38-182)
+ * as called at src/nats/layers/natsl_attn_gdn.py:652-661. */
+int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const void* x_weights, const void* w1,
+                        const void* w2, void* y, int64_t rows, int D, int dtype, float eps, int w_dtype,
+                        natsl_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

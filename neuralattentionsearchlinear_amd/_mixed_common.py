@@ -11,6 +11,16 @@ from .nats_util import CHUNK_SIZE, PackedSeqs, _seq_args, pack_sequences, route
 
 _attn_streams: dict = {}
 
+# Optional timing hook: when set to a callable(name, stream) it is invoked right before and right
+# after each branch is enqueued ("softmax:start", "softmax:end", "linear:start", "linear:end") so a
+# caller can record events on the stream the kernels were launched on.
+TIMING_HOOK = None
+
+
+def _mark(name, stream):
+    if TIMING_HOOK is not None:
+        TIMING_HOOK(name, stream)
+
 
 def _get_attn_stream(device: torch.device) -> torch.cuda.Stream:
     """One cached side stream per device for the softmax branch (default priority), as the
@@ -98,13 +108,17 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
     side = _get_attn_stream(dev)
     side.wait_stream(cur)
     with torch.cuda.stream(side):
+        _mark("softmax:start", side)
         o_attn, _lse, _ = parallel_attn_nats_fwd(
             q_attn, k_attn, v_attn, types, r['nats_block_indices'], None, scale_attn, nats_block_size,
             compute_incomplete_chunk_scores=attn_same_block, n_nats_blocks=r['n_nats_blocks'], seqs=seqs)
+        _mark("softmax:end", side)
     flags = (_capi.DECAY_NON_LINEAR if decay_non_linear else 0) | (_capi.QK_L2NORM if qk_l2norm else 0) | \
             (_capi.INTRA_CHUNK if lin_intra else 0)
+    _mark("linear:start", cur)
     o_lin, ht = linear_chunk_fwd(kind, q_lattn, k_lattn, v_lattn, g, beta, initial_state, types, scale_lattn,
                                  nats_block_size, flags, output_final_state, seqs)
+    _mark("linear:end", cur)
     cur.wait_stream(side)
     for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
         t.record_stream(side)

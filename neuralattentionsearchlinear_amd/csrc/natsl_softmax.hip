@@ -9,6 +9,7 @@
 // O^T = V^T P^T.  V^T is read from the row-major V tile with the transposing LDS load.
 #include "natsl_device.h"
 #include "natsl_host.h"
+#include <stdlib.h>
 
 namespace natsl {
 
@@ -29,6 +30,7 @@ struct SoftmaxParams {
   int total_tiles;
   float scale_log2;
   int same_block;
+  int variant;
 };
 
 NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
@@ -38,14 +40,135 @@ NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
 }
 
 constexpr int QTILE = 256;
+constexpr int VT_PITCH = 68;          // elements per row of the transposed V tile (64 keys + 4): conflict-free operand reads
+constexpr float RESCALE_SLACK = 8.f;  // log2 units: probabilities may reach 2^8 before the reference maximum moves
+constexpr int MAX_LDS_LIST = 2048;    // prior attention blocks whose ids are kept in LDS (more are re-read from memory)
 
-template <int DK, int DV>
-__global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
-  constexpr int KP = DK + 8, VP = DV + 8;  // LDS row pitch in elements (16-byte multiple)
-  constexpr int KSTEPS = DK / 16, VT = DV / 32, KL = DK / 32, VL = DV / 32;
+// One 64-key chunk for one wave owning NQ column tiles of 32 queries, in three pieces:
+//   scores      S^T = K Q^T (key tile kt x query tile qt) and the scaled row maxima
+//   rescale     move the reference maximum m_ref and rescale the accumulators.  It is needed only
+//               when some row's maximum has grown by more than RESCALE_SLACK since m_ref was set,
+//               so the hot loop never touches the accumulators with vector ALU instructions.
+//   exp_pv      P = exp2(S*c - m_ref), row sums, O^T += V^T P^T, 16 keys per step.
+//               Accumulator register r of key tile kt is key 32kt + 8(r/4) + 4hf + r%4; the same
+//               order is used for the k-slots of the V^T operand, so P needs no data movement.
+//               V is staged TRANSPOSED in LDS (VT[v][key]): that operand is two 8-byte reads.
+template <int DK, int NQ, bool CAUSAL>
+NATSL_DEVICE void scores(const bf16_t* Kb, const bf16x8 (&QB)[NQ][DK / 16], f32x16 (&s)[2][NQ], float (&mx)[NQ], const float c,
+                         const int lane, const int qloc0) {
+  constexpr int KP = DK + 8, KSTEPS = DK / 16;
+  const int l32 = lane & 31, hf = lane >> 5;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[kt][qt][r] = 0.f;
+#pragma unroll
+  for (int st = 0; st < KSTEPS; ++st) {
+    const bf16x8 ka0 = ld8(Kb + l32 * KP + 16 * st + 8 * hf);
+    const bf16x8 ka1 = ld8(Kb + (32 + l32) * KP + 16 * st + 8 * hf);
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+      s[0][qt] = mfma32(ka0, QB[qt][st], s[0][qt]);
+      s[1][qt] = mfma32(ka1, QB[qt][st], s[1][qt]);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if (CAUSAL) {
+          const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3), qloc = qloc0 + 32 * qt + l32;
+          if (kloc > qloc) s[kt][qt][r] = -INFINITY;
+        }
+        m = fmaxf(m, s[kt][qt][r]);
+      }
+    mx[qt] = xhalf_max(m) * c;
+  }
+}
+
+template <int NQ>
+NATSL_DEVICE bool needs_rescale(const float (&mx)[NQ], const float (&m_ref)[NQ]) {
+  bool need = false;
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) need = need || mx[qt] > m_ref[qt] + RESCALE_SLACK;
+  return __any(need) != 0;
+}
+
+template <int DV, int NQ>
+NATSL_DEVICE void rescale(f32x16 (&acc)[DV / 32][NQ], float (&m_ref)[NQ], float (&l_run)[NQ], const float (&mx)[NQ]) {
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    const float m_new = fmaxf(m_ref[qt], mx[qt]);
+    const float alpha = __builtin_amdgcn_exp2f(m_ref[qt] - (m_new == -INFINITY ? 0.f : m_new));
+    m_ref[qt] = m_new;
+    l_run[qt] *= alpha;
+#pragma unroll
+    for (int vt = 0; vt < DV / 32; ++vt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[vt][qt][r] *= alpha;
+  }
+}
+
+template <int DV, int NQ>
+NATSL_DEVICE void exp_pv(const bf16_t* VTb, f32x16 (&s)[2][NQ], f32x16 (&acc)[DV / 32][NQ], const float (&m_ref)[NQ],
+                         float (&l_run)[NQ], const float c, const int lane) {
+  constexpr int TP = VT_PITCH, VT = DV / 32;
+  const int l32 = lane & 31, hf = lane >> 5;
+  float neg[NQ], rs[NQ];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    neg[qt] = m_ref[qt] == -INFINITY ? 0.f : -m_ref[qt];
+    rs[qt] = 0.f;
+  }
+#pragma unroll
+  for (int sidx = 0; sidx < 4; ++sidx) {
+    const int kt = sidx >> 1, ss = sidx & 1;
+    bf16x8 PB[NQ];
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+      float e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        e[j] = __builtin_amdgcn_exp2f(fmaf(s[kt][qt][8 * ss + j], c, neg[qt]));
+        rs[qt] += e[j];
+      }
+      u32x4 w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(e[2 * j], e[2 * j + 1]);
+      PB[qt] = __builtin_bit_cast(bf16x8, w);
+    }
+    const int kbase = 32 * kt + 16 * ss + 4 * hf;  // this lane's keys: kbase..kbase+3 and kbase+8..kbase+11
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+      const bf16_t* vr = VTb + (32 * vt + l32) * TP + kbase;
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
+      const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+      const bf16x8 va = __builtin_bit_cast(bf16x8, w);
+#pragma unroll
+      for (int qt = 0; qt < NQ; ++qt) acc[vt][qt] = mfma32(va, PB[qt], acc[vt][qt]);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) l_run[qt] += rs[qt];  // partial over this lane's keys; halves are joined in the epilogue
+}
+
+// NQ = 32-query column tiles per wave; the workgroup has 8/NQ waves and always owns 256 queries.
+template <int DK, int DV, int NQ>
+__global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
+  constexpr int NWAVES = 8 / NQ, NTHREADS = 64 * NWAVES, QW = 32 * NQ;  // queries per wave
+  constexpr int KP = DK + 8, VP = DV + 8;  // row pitch (elements) of the K tile and of the epilogue tile
+  constexpr int TP = VT_PITCH;
+  constexpr int KSTEPS = DK / 16, VT = DV / 32;
   extern __shared__ __align__(16) unsigned char smem[];
-  bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);  // [2][64][KP]
-  bf16_t* Vs = Ks + 2 * 64 * KP;                 // [2][64][VP]
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);  // [2][64][KP]   keys, row-major
+  bf16_t* Vs = Ks + 2 * 64 * KP;                 // [2][DV][TP]   values, transposed
+  __shared__ int lds_list[MAX_LDS_LIST];
+  __shared__ int lds_count;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l32 = lane & 31, hf = lane >> 5;
@@ -53,11 +176,15 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   // ---- which (sequence, head, tile) ------------------------------------------------------
   int n, tile, hq, bos, len, bos_nats;
   if (p.seqs == nullptr) {
-    const int per = p.B * p.HQ;
-    tile = p.nq_tiles - 1 - (int)blockIdx.x / per;  // heaviest tiles first
-    const int rem = (int)blockIdx.x % per;
-    n = rem / p.HQ;
-    hq = rem % p.HQ;
+    // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD whole (batch, head) pairs,
+    // heaviest tile first, so the tiles that share one pair's K/V run together on one L2.
+    const int n_pairs = p.B * p.HQ;
+    const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
+    const int pair = (j / p.nq_tiles) * 8 + xcd;
+    if (pair >= n_pairs) return;
+    tile = p.nq_tiles - 1 - j % p.nq_tiles;
+    n = pair / p.HQ;
+    hq = pair % p.HQ;
     bos = n * p.T;
     len = p.T;
     bos_nats = n * p.TN;
@@ -75,7 +202,9 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   const int Bs = p.block, per_blk = Bs >> 6;
   const int hkv = hq / (p.HQ / p.HKV), hn = hq / (p.HQ / p.HN);
   const int tile_start = tile * QTILE;
-  const int q0 = tile_start + wave * 64;
+  const int q0 = tile_start + wave * QW;      // this wave's first query
+  const int my_chunk = (wave * QW) >> 6;      // which of the tile's four 64-key chunks holds them
+  const int qloc0 = (wave * QW) & 63;         // ... and where in that chunk
   const bool wave_valid = q0 < len;
 
   const bf16_t* qp = p.q + ((size_t)bos * p.HQ + hq) * DK;
@@ -86,24 +215,41 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   const size_t list_stride = (size_t)p.HN * 2;
   const int n_attn = p.nblk[((size_t)n * p.HN + hn) * 2];
 
-  // number of attention blocks that end at or before the tile's first query
-  int n_prior;
-  {
-    int lo = 0, hi = n_attn;
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if ((list[mid * list_stride] + 1) * Bs <= tile_start) lo = mid + 1; else hi = mid;
-    }
-    n_prior = lo;
+  // ---- Q as the B operand of S^T = K Q^T: lane = query column ----------------------------
+  bf16x8 QB[NQ][KSTEPS];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    const int qi = min(q0 + 32 * qt + l32, len - 1);  // rows past the end are computed on a copy and never stored
+    const bf16_t* qr = qp + (size_t)qi * p.HQ * DK + 8 * hf;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) QB[qt][s] = ld8(qr + 16 * s);
   }
-  const int n_prior_chunks = n_prior * per_blk;
+
+  // ---- attention blocks that end at or before the tile's first query: ids into LDS, count ----
+  // (the list is sorted, so the qualifying entries are a prefix of it)
+  if (tid == 0) lds_count = 0;
+  __syncthreads();
+  {
+    int cnt = 0;
+    for (int j = tid; j < n_attn; j += NTHREADS) {
+      const int e = list[j * list_stride];
+      if ((e + 1) * Bs <= tile_start) {
+        ++cnt;
+        if (j < MAX_LDS_LIST) lds_list[j] = e;
+      }
+    }
+    if (cnt) atomicAdd(&lds_count, cnt);
+  }
+  __syncthreads();
+  const int n_prior_chunks = lds_count * per_blk;
   const int n_diag = min(4, (len - tile_start + 63) >> 6);
   const int n_iters = n_prior_chunks + n_diag;
 
   auto key_start = [&](int it) -> int {
     if (it < n_prior_chunks) {
       const int j = it / per_blk;
-      return list[j * list_stride] * Bs + (it - j * per_blk) * 64;
+      const int e = j < MAX_LDS_LIST ? lds_list[j] : list[j * list_stride];
+      return e * Bs + (it - j * per_blk) * 64;
     }
     return tile_start + (it - n_prior_chunks) * 64;
   };
@@ -111,46 +257,71 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
     return type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2);
   };
 
-  // ---- Q as the B operand of S^T = K Q^T: lane = query column ----------------------------
-  bf16x8 QB[2][KSTEPS];
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    const int qi = q0 + 32 * qt + l32;
-    const bf16_t* qr = qp + (size_t)qi * p.HQ * DK + 8 * hf;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) QB[qt][s] = qi < len ? ld8(qr + 16 * s) : zero8();
-  }
-
-  f32x16 acc[VT][2];
+  f32x16 acc[VT][NQ];
 #pragma unroll
   for (int vt = 0; vt < VT; ++vt)
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
+    for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[vt][qt][r] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+  float m_ref[NQ], l_run[NQ];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    m_ref[qt] = -INFINITY;
+    l_run[qt] = 0.f;
+  }
 
   // ---- global -> register -> LDS staging of one 64-key chunk -----------------------------
-  u32x4 kreg[KL], vreg[VL];
-  const int ld_row = tid >> 2, ld_seg = tid & 3;
+  // 256 threads stage K (thread = row, 16-byte segments; stored row-major), 256 threads stage V
+  // (thread = group of 4 keys x 8 value columns; the 4x8 block is transposed in registers and
+  // stored as 8 rows of 4 keys).  With 4 waves every thread does both.
+  constexpr bool SPLIT = NTHREADS == 512;
+  constexpr int KL = DK / 32;
+  const int st = SPLIT ? (tid & 255) : tid;
+  const bool do_k = !SPLIT || tid < 256, do_v_role = !SPLIT || tid >= 256;
+  u32x4 kreg[KL], vreg[4];
+  const int ld_row = st >> 2, ld_seg = st & 3;
+  constexpr int VSEGS = DV / 8;                    // 8-column segments per V row
+  const int v_seg = (st & 3) + 4 * (st >> 6);      // 64 contiguous bytes per row per wave
+  const int v_kg = (st >> 2) & 15;                 // keys 4*v_kg .. 4*v_kg+3
+  const bool v_on = do_v_role && v_seg < VSEGS;
   auto gload = [&](int ks) {
-    const int tok = ks + ld_row;
-    const bool ok = tok < len;
-    const u32x4* kr = reinterpret_cast<const u32x4*>(kp + (size_t)tok * krow);
-    const u32x4* vr = reinterpret_cast<const u32x4*>(vp + (size_t)tok * vrow);
-    const u32x4 z = {0u, 0u, 0u, 0u};
+    // Rows past the end of the sequence are clamped to its last row: such keys are always hidden
+    // by the causal rule (a valid query precedes them), so only finite values are needed there.
+    if (do_k) {
+      const int tok = min(ks + ld_row, len - 1);
+      const u32x4* kr = reinterpret_cast<const u32x4*>(kp + (size_t)tok * krow);
 #pragma unroll
-    for (int i = 0; i < KL; ++i) kreg[i] = ok ? kr[ld_seg + 4 * i] : z;
+      for (int i = 0; i < KL; ++i) kreg[i] = kr[ld_seg + 4 * i];
+    }
+    if (v_on) {
 #pragma unroll
-    for (int i = 0; i < VL; ++i) vreg[i] = ok ? vr[ld_seg + 4 * i] : z;
+      for (int j = 0; j < 4; ++j) {
+        const int vt_ = min(ks + 4 * v_kg + j, len - 1);
+        vreg[j] = *reinterpret_cast<const u32x4*>(vp + (size_t)vt_ * vrow + 8 * v_seg);
+      }
+    }
   };
   auto lstore = [&](int buf) {
-    bf16_t* kd = Ks + (buf * 64 + ld_row) * KP;
-    bf16_t* vd = Vs + (buf * 64 + ld_row) * VP;
+    if (do_k) {
+      bf16_t* kd = Ks + (buf * 64 + ld_row) * KP;
 #pragma unroll
-    for (int i = 0; i < KL; ++i) *reinterpret_cast<u32x4*>(kd + (ld_seg + 4 * i) * 8) = kreg[i];
+      for (int i = 0; i < KL; ++i) *reinterpret_cast<u32x4*>(kd + (ld_seg + 4 * i) * 8) = kreg[i];
+    }
+    if (v_on) {
+      bf16_t* vd = Vs + (buf * DV + 8 * v_seg) * TP + 4 * v_kg;
 #pragma unroll
-    for (int i = 0; i < VL; ++i) *reinterpret_cast<u32x4*>(vd + (ld_seg + 4 * i) * 8) = vreg[i];
+      for (int d = 0; d < 4; ++d) {
+        // value columns 2d (low halves) and 2d+1 (high halves) of the four keys
+        u32x2 lo, hi;
+        lo[0] = __builtin_amdgcn_perm(vreg[1][d], vreg[0][d], 0x05040100u);
+        lo[1] = __builtin_amdgcn_perm(vreg[3][d], vreg[2][d], 0x05040100u);
+        hi[0] = __builtin_amdgcn_perm(vreg[1][d], vreg[0][d], 0x07060302u);
+        hi[1] = __builtin_amdgcn_perm(vreg[3][d], vreg[2][d], 0x07060302u);
+        *reinterpret_cast<u32x2*>(vd + (2 * d) * TP) = lo;
+        *reinterpret_cast<u32x2*>(vd + (2 * d + 1) * TP) = hi;
+      }
+    }
   };
 
   if (n_iters > 0) {
@@ -159,118 +330,73 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   }
   __syncthreads();
 
+  const float c = p.scale_log2;
+  f32x16 s[2][NQ];
+  float mx[NQ];
+  // ---- phase A: whole attention blocks before the tile; every wave, no masks.  The inner loop is
+  // the fast path; an iteration whose maxima outgrow the reference leaves it, rescales, finishes
+  // and re-enters.
+  int it = 0;
+  while (it < n_prior_chunks) {
+    bool pending = false;
+    for (; it < n_prior_chunks; ++it) {
+      const int buf = it & 1;
+      if (it + 1 < n_iters) gload(key_start(it + 1));
+      if (wave_valid) {
+        scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
+        if (needs_rescale<NQ>(mx, m_ref)) {
+          pending = true;
+          break;
+        }
+        exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
+      }
+      if (it + 1 < n_iters) lstore(buf ^ 1);
+      __syncthreads();
+    }
+    if (pending) {
+      const int buf = it & 1;
+      rescale<DV, NQ>(acc, m_ref, l_run, mx);
+      exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
+      if (it + 1 < n_iters) lstore(buf ^ 1);
+      __syncthreads();
+      ++it;
+    }
+  }
+  // ---- phase B: the tile's own four chunks
   const int my_blk = q0 / Bs;
-  for (int it = 0; it < n_iters; ++it) {
+  for (; it < n_iters; ++it) {
     const int buf = it & 1;
     if (it + 1 < n_iters) gload(key_start(it + 1));
-
+    const int jc = it - n_prior_chunks;
+    const int kblk = (tile_start + jc * 64) / Bs;
     bool active = wave_valid, causal = false;
-    if (it >= n_prior_chunks) {
-      const int jc = it - n_prior_chunks;
-      const int kblk = (tile_start + jc * 64) / Bs;
-      if (p.same_block) {
-        if (jc > wave) active = false;
-        else if (jc == wave) causal = true;
-        else active = active && (kblk == my_blk || attn_block(kblk));
-      } else {
-        active = active && jc < wave && kblk < my_blk && attn_block(kblk);
-      }
+    if (p.same_block) {
+      if (jc > my_chunk) active = false;
+      else if (jc == my_chunk) causal = true;
+      else active = active && (kblk == my_blk || attn_block(kblk));
+    } else {
+      active = active && jc < my_chunk && kblk < my_blk && attn_block(kblk);
     }
-
     if (active) {
-      const bf16_t* Kb = Ks + buf * 64 * KP;
-      const bf16_t* Vb = Vs + buf * 64 * VP;
-      f32x16 s[2][2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[kt][qt][r] = 0.f;
-#pragma unroll
-      for (int st = 0; st < KSTEPS; ++st) {
-        const bf16x8 ka0 = ld8(Kb + l32 * KP + 16 * st + 8 * hf);
-        const bf16x8 ka1 = ld8(Kb + (32 + l32) * KP + 16 * st + 8 * hf);
-        s[0][0] = mfma32(ka0, QB[0][st], s[0][0]);
-        s[0][1] = mfma32(ka0, QB[1][st], s[0][1]);
-        s[1][0] = mfma32(ka1, QB[0][st], s[1][0]);
-        s[1][1] = mfma32(ka1, QB[1][st], s[1][1]);
-      }
-      // online softmax; acc register r of key tile kt is key 32kt + 8(r/4) + 4hf + r%4
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        const int qloc = 32 * qt + l32;
-        float mx = -INFINITY;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float x = s[kt][qt][r] * p.scale_log2;
-            if (causal) {
-              const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3);
-              if (kloc > qloc) x = -INFINITY;
-            }
-            s[kt][qt][r] = x;
-            mx = fmaxf(mx, x);
-          }
-        mx = xhalf_max(mx);
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);
-        float rs = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float e = __builtin_amdgcn_exp2f(s[kt][qt][r] - m_safe);
-            s[kt][qt][r] = e;
-            rs += e;
-          }
-        l_run[qt] = l_run[qt] * alpha + rs;  // partial over this lane's keys; halves are joined at the end
-        m_run[qt] = m_new;
-#pragma unroll
-        for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[vt][qt][r] *= alpha;
-      }
-      // O^T += V^T P^T, 16 keys per step; MFMA k-slot (hf, j) <-> key base + 8(j/4) + 4hf + j%4
-      const int i16 = lane & 15, colsel = 16 * ((lane >> 4) & 1);
-#pragma unroll
-      for (int sidx = 0; sidx < 4; ++sidx) {
-        const int kt = sidx >> 1, ss = sidx & 1;
-        bf16x8 PB[2];
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-          u32x4 w;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(s[kt][qt][8 * ss + 2 * j], s[kt][qt][8 * ss + 2 * j + 1]);
-          PB[qt] = __builtin_bit_cast(bf16x8, w);
-        }
-        const int base = 32 * kt + 16 * ss + 4 * hf;
-        const bf16_t* vrow0 = Vb + (base + (i16 >> 2)) * VP + colsel + 4 * (i16 & 3);
-#pragma unroll
-        for (int vt = 0; vt < VT; ++vt) {
-          const bf16x8 va = join4(lds_tr4(vrow0 + 32 * vt), lds_tr4(vrow0 + 8 * VP + 32 * vt));
-          acc[vt][0] = mfma32(va, PB[0], acc[vt][0]);
-          acc[vt][1] = mfma32(va, PB[1], acc[vt][1]);
-        }
-      }
+      if (causal) scores<DK, NQ, true>(Ks + buf * 64 * KP, QB, s, mx, c, lane, qloc0);
+      else scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
+      if (needs_rescale<NQ>(mx, m_ref)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
+      exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
     }
-
     if (it + 1 < n_iters) lstore(buf ^ 1);
     __syncthreads();
   }
 
   // ---- epilogue: normalise, transpose through LDS, coalesced stores ------------------------
-  bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + wave * 64 * VP;  // this wave's [64][VP]
+  bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + wave * QW * VP;  // this wave's [QW][VP]
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     const float l_tot = xhalf_sum(l_run[qt]);
     const bool has = l_tot > 0.f;
     const float inv = has ? 1.f / l_tot : 0.f;
     const int qi = q0 + 32 * qt + l32;
     if (hf == 0 && qi < len)
-      p.lse[((size_t)(bos + qi)) * p.HQ + hq] = has ? m_run[qt] + __builtin_amdgcn_logf(l_tot) : 0.f;
+      p.lse[((size_t)(bos + qi)) * p.HQ + hq] = has ? m_ref[qt] + __builtin_amdgcn_logf(l_tot) : 0.f;
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt)
 #pragma unroll
@@ -286,7 +412,7 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   constexpr int SEGS = DV / 8;           // 16-byte segments per row
   constexpr int ROWS_PER_PASS = 64 / SEGS;
 #pragma unroll
-  for (int pass = 0; pass < 64 / ROWS_PER_PASS; ++pass) {
+  for (int pass = 0; pass < QW / ROWS_PER_PASS; ++pass) {
     const int row = pass * ROWS_PER_PASS + lane / SEGS, seg = lane % SEGS;
     const int qi = q0 + row;
     if (qi < len) {
@@ -296,18 +422,18 @@ __global__ __launch_bounds__(256, 1) void softmax_sparse_fwd_kernel(const Softma
   }
 }
 
-template <int DK, int DV>
+template <int DK, int DV, int NQ>
 static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   constexpr int KP = DK + 8, VP = DV + 8;
-  size_t lds = (size_t)2 * 64 * (KP + VP) * sizeof(bf16_t);
+  size_t lds = (size_t)2 * (64 * KP + DV * VT_PITCH) * sizeof(bf16_t);
   const size_t epi = (size_t)QTILE * VP * sizeof(bf16_t);
   if (epi > lds) lds = epi;
-  auto kern = softmax_sparse_fwd_kernel<DK, DV>;
+  auto kern = softmax_sparse_fwd_kernel<DK, DV, NQ>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-  const long long grid = (long long)p.total_tiles * p.HQ;
+  const long long grid = p.seqs ? (long long)p.total_tiles * p.HQ : (long long)8 * ((p.B * p.HQ + 7) / 8) * p.nq_tiles;
   if (grid <= 0) return NATSL_OK;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512 / NQ), lds, stream, p);
   return check_launch("natsl_softmax_sparse_fwd");
 }
 
@@ -340,10 +466,15 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.total_tiles = seqs ? total_units : B * p.nq_tiles;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.same_block = same_block_visible ? 1 : 0;
+  p.variant = getenv("NATSL_SOFTMAX_WAVES") ? atoi(getenv("NATSL_SOFTMAX_WAVES")) : 8;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (K == 128 && V == 128) return launch_softmax<128, 128>(p, s);
-  if (K == 64 && V == 64) return launch_softmax<64, 64>(p, s);
-  if (K == 64 && V == 128) return launch_softmax<64, 128>(p, s);
-  if (K == 128 && V == 64) return launch_softmax<128, 64>(p, s);
+#define NATSL_SM(KK, VV)                                              \
+  if (K == KK && V == VV)                                             \
+    return p.variant == 4 ? launch_softmax<KK, VV, 2>(p, s) : launch_softmax<KK, VV, 1>(p, s);
+  NATSL_SM(128, 128)
+  NATSL_SM(64, 64)
+  NATSL_SM(64, 128)
+  NATSL_SM(128, 64)
+#undef NATSL_SM
   return fail(NATSL_ERR_UNSUPPORTED, "softmax: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", K, V);
 }
