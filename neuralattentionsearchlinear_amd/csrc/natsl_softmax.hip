@@ -31,6 +31,7 @@ struct SoftmaxParams {
   float scale_log2;
   int same_block;
   int variant;
+  int dbg;
 };
 
 NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
@@ -39,7 +40,7 @@ NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
   return rintf(x) == 1.0f;
 }
 
-constexpr int QTILE = 256;
+constexpr int QTILE_TABLE = 256;  // query tile the packed-sequence table counts in
 constexpr int VT_PITCH = 68;          // elements per row of the transposed V tile (64 keys + 4): conflict-free operand reads
 constexpr float RESCALE_SLACK = 8.f;  // log2 units: probabilities may reach 2^8 before the reference maximum moves
 constexpr int MAX_LDS_LIST = 2048;    // prior attention blocks whose ids are kept in LDS (more are re-read from memory)
@@ -157,10 +158,10 @@ NATSL_DEVICE void exp_pv(const bf16_t* VTb, f32x16 (&s)[2][NQ], f32x16 (&acc)[DV
   for (int qt = 0; qt < NQ; ++qt) l_run[qt] += rs[qt];  // partial over this lane's keys; halves are joined in the epilogue
 }
 
-// NQ = 32-query column tiles per wave; the workgroup has 8/NQ waves and always owns 256 queries.
-template <int DK, int DV, int NQ>
-__global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
-  constexpr int NWAVES = 8 / NQ, NTHREADS = 64 * NWAVES, QW = 32 * NQ;  // queries per wave
+// NQ = 32-query column tiles per wave, NWAVES waves: the workgroup owns QTILE = 32*NQ*NWAVES queries.
+template <int DK, int DV, int NQ, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
+  constexpr int NTHREADS = 64 * NWAVES, QW = 32 * NQ, QTILE = QW * NWAVES;  // QW = queries per wave
   constexpr int KP = DK + 8, VP = DV + 8;  // row pitch (elements) of the K tile and of the epilogue tile
   constexpr int TP = VT_PITCH;
   constexpr int KSTEPS = DK / 16, VT = DV / 32;
@@ -180,21 +181,23 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
     // heaviest tile first, so the tiles that share one pair's K/V run together on one L2.
     const int n_pairs = p.B * p.HQ;
     const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
-    const int pair = (j / p.nq_tiles) * 8 + xcd;
+    const int nq_tiles = (p.T + QTILE - 1) / QTILE;
+    const int pair = (j / nq_tiles) * 8 + xcd;
     if (pair >= n_pairs) return;
-    tile = p.nq_tiles - 1 - j % p.nq_tiles;
+    tile = nq_tiles - 1 - j % nq_tiles;
     n = pair / p.HQ;
     hq = pair % p.HQ;
     bos = n * p.T;
     len = p.T;
     bos_nats = n * p.TN;
   } else {
-    const int gt = p.total_tiles - 1 - (int)blockIdx.x / p.HQ;
+    const int tiles_per_256 = QTILE_TABLE / QTILE;
+    const int gt = p.total_tiles * tiles_per_256 - 1 - (int)blockIdx.x / p.HQ;
     hq = (int)blockIdx.x % p.HQ;
     n = 0;
     for (int i = 1; i < p.n_seqs; ++i)
-      if (p.seqs[i].qtile_off <= gt) n = i;
-    tile = gt - p.seqs[n].qtile_off;
+      if (p.seqs[i].qtile_off * tiles_per_256 <= gt) n = i;
+    tile = gt - p.seqs[n].qtile_off * tiles_per_256;
     bos = p.seqs[n].bos;
     len = p.seqs[n].eos - bos;
     bos_nats = p.seqs[n].bos_nats;
@@ -203,8 +206,11 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
   const int hkv = hq / (p.HQ / p.HKV), hn = hq / (p.HQ / p.HN);
   const int tile_start = tile * QTILE;
   const int q0 = tile_start + wave * QW;      // this wave's first query
-  const int my_chunk = (wave * QW) >> 6;      // which of the tile's four 64-key chunks holds them
-  const int qloc0 = (wave * QW) & 63;         // ... and where in that chunk
+  const int my_chunk = q0 >> 6;               // the 64-key chunk of the sequence that holds them
+  const int qloc0 = q0 & 63;                  // ... and where in that chunk
+  // keys from here on are handled chunk by chunk with the same-block / causal rules: the start of
+  // the tile, or of the selector block it falls into when blocks are larger than the tile
+  const int dstart = (tile_start / p.block) * p.block;
   const bool wave_valid = q0 < len;
 
   const bf16_t* qp = p.q + ((size_t)bos * p.HQ + hq) * DK;
@@ -225,15 +231,16 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
     for (int s = 0; s < KSTEPS; ++s) QB[qt][s] = ld8(qr + 16 * s);
   }
 
-  // ---- attention blocks that end at or before the tile's first query: ids into LDS, count ----
+  // ---- attention blocks that end at or before dstart: ids into LDS, count ----
   // (the list is sorted, so the qualifying entries are a prefix of it)
+  if (tile_start >= len) return;  // packed input: a sequence's last 256-row table slot may hold no tile of this size
   if (tid == 0) lds_count = 0;
   __syncthreads();
   {
     int cnt = 0;
     for (int j = tid; j < n_attn; j += NTHREADS) {
       const int e = list[j * list_stride];
-      if ((e + 1) * Bs <= tile_start) {
+      if ((e + 1) * Bs <= dstart) {
         ++cnt;
         if (j < MAX_LDS_LIST) lds_list[j] = e;
       }
@@ -242,7 +249,7 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
   }
   __syncthreads();
   const int n_prior_chunks = lds_count * per_blk;
-  const int n_diag = min(4, (len - tile_start + 63) >> 6);
+  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;
   const int n_iters = n_prior_chunks + n_diag;
 
   auto key_start = [&](int it) -> int {
@@ -251,7 +258,7 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
       const int e = j < MAX_LDS_LIST ? lds_list[j] : list[j * list_stride];
       return e * Bs + (it - j * per_blk) * 64;
     }
-    return tile_start + (it - n_prior_chunks) * 64;
+    return dstart + (it - n_prior_chunks) * 64;
   };
   auto attn_block = [&](int blk) -> bool {
     return type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2);
@@ -275,6 +282,7 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
   // 256 threads stage K (thread = row, 16-byte segments; stored row-major), 256 threads stage V
   // (thread = group of 4 keys x 8 value columns; the 4x8 block is transposed in registers and
   // stored as 8 rows of 4 keys).  With 4 waves every thread does both.
+  static_assert(NTHREADS == 256 || NTHREADS == 512, "staging is written for 4 or 8 waves");
   constexpr bool SPLIT = NTHREADS == 512;
   constexpr int KL = DK / 32;
   const int st = SPLIT ? (tid & 255) : tid;
@@ -341,8 +349,8 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
     bool pending = false;
     for (; it < n_prior_chunks; ++it) {
       const int buf = it & 1;
-      if (it + 1 < n_iters) gload(key_start(it + 1));
-      if (wave_valid) {
+      if (it + 1 < n_iters && !(p.dbg & 1)) gload(key_start(it + 1));
+      if (wave_valid && !(p.dbg & 2)) {
         scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
         if (needs_rescale<NQ>(mx, m_ref)) {
           pending = true;
@@ -350,7 +358,7 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
         }
         exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
       }
-      if (it + 1 < n_iters) lstore(buf ^ 1);
+      if (it + 1 < n_iters && !(p.dbg & 1)) lstore(buf ^ 1);
       __syncthreads();
     }
     if (pending) {
@@ -362,13 +370,13 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
       ++it;
     }
   }
-  // ---- phase B: the tile's own four chunks
+  // ---- phase B: the chunks from dstart to the end of the tile
   const int my_blk = q0 / Bs;
   for (; it < n_iters; ++it) {
     const int buf = it & 1;
     if (it + 1 < n_iters) gload(key_start(it + 1));
-    const int jc = it - n_prior_chunks;
-    const int kblk = (tile_start + jc * 64) / Bs;
+    const int jc = (dstart >> 6) + it - n_prior_chunks;  // absolute chunk index of the keys
+    const int kblk = (jc * 64) / Bs;
     bool active = wave_valid, causal = false;
     if (p.same_block) {
       if (jc > my_chunk) active = false;
@@ -377,7 +385,7 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
     } else {
       active = active && jc < my_chunk && kblk < my_blk && attn_block(kblk);
     }
-    if (active) {
+    if (active && !(p.dbg & 8)) {
       if (causal) scores<DK, NQ, true>(Ks + buf * 64 * KP, QB, s, mx, c, lane, qloc0);
       else scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
       if (needs_rescale<NQ>(mx, m_ref)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
@@ -422,18 +430,19 @@ __global__ __launch_bounds__(512 / NQ) void softmax_sparse_fwd_kernel(const Soft
   }
 }
 
-template <int DK, int DV, int NQ>
+template <int DK, int DV, int NQ, int NWAVES>
 static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
-  constexpr int KP = DK + 8, VP = DV + 8;
+  constexpr int KP = DK + 8, VP = DV + 8, QTILE = 32 * NQ * NWAVES;
   size_t lds = (size_t)2 * (64 * KP + DV * VT_PITCH) * sizeof(bf16_t);
   const size_t epi = (size_t)QTILE * VP * sizeof(bf16_t);
   if (epi > lds) lds = epi;
-  auto kern = softmax_sparse_fwd_kernel<DK, DV, NQ>;
+  auto kern = softmax_sparse_fwd_kernel<DK, DV, NQ, NWAVES>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-  const long long grid = p.seqs ? (long long)p.total_tiles * p.HQ : (long long)8 * ((p.B * p.HQ + 7) / 8) * p.nq_tiles;
+  const long long grid = p.seqs ? (long long)p.total_tiles * (QTILE_TABLE / QTILE) * p.HQ
+                                : (long long)8 * ((p.B * p.HQ + 7) / 8) * ((p.T + QTILE - 1) / QTILE);
   if (grid <= 0) return NATSL_OK;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512 / NQ), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NWAVES), lds, stream, p);
   return check_launch("natsl_softmax_sparse_fwd");
 }
 
@@ -462,15 +471,16 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.types = types; p.types_dtype = types_dtype; p.idx = nats_block_indices; p.nblk = n_nats_blocks;
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0;
   p.B = B; p.T = T; p.HQ = HQ; p.HKV = HKV; p.HN = HN; p.TN = TN; p.block = block;
-  p.nq_tiles = cdiv(T, QTILE);
+  p.nq_tiles = cdiv(T, QTILE_TABLE);
   p.total_tiles = seqs ? total_units : B * p.nq_tiles;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.same_block = same_block_visible ? 1 : 0;
-  p.variant = getenv("NATSL_SOFTMAX_WAVES") ? atoi(getenv("NATSL_SOFTMAX_WAVES")) : 8;
+  p.dbg = getenv("NATSL_DBG") ? atoi(getenv("NATSL_DBG")) : 0;
+  p.variant = getenv("NATSL_SOFTMAX_WAVES") ? atoi(getenv("NATSL_SOFTMAX_WAVES")) : 1;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define NATSL_SM(KK, VV)                                              \
   if (K == KK && V == VV)                                             \
-    return p.variant == 4 ? launch_softmax<KK, VV, 2>(p, s) : launch_softmax<KK, VV, 1>(p, s);
+    return p.variant == 4 ? launch_softmax<KK, VV, 2, 4>(p, s) : p.variant == 8 ? launch_softmax<KK, VV, 1, 8>(p, s) : launch_softmax<KK, VV, 1, 4>(p, s);
   NATSL_SM(128, 128)
   NATSL_SM(64, 64)
   NATSL_SM(64, 128)

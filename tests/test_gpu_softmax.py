@@ -43,7 +43,7 @@ def test_softmax_ragged_length():
     _run(1, 100, 2, 2, 2, 64, 64, 64, 0.5, True, seed=6)
 
 
-@pytest.mark.parametrize("block", [128, 256])
+@pytest.mark.parametrize("block", [128, 256, 512])
 def test_softmax_large_blocks(block):
     _run(1, 1024, 2, 2, 2, 128, 64, block, 0.5, True, seed=7)
     _run(1, 1024, 2, 2, 2, 128, 64, block, 0.5, False, seed=8)
