@@ -11,7 +11,7 @@
 //                          TmB  bf16 [64][64]   Tm * diag(beta)                      (delta rule only)
 //                          P    bf16 [64][64]   scale * tril(q^ k^^T * e^{gamma_i-gamma_j})
 //                          sc   f32  [4][64]    se = e^{gamma} rk, sq = scale rq e^{gamma},
-//                                               sk = rk e^{gamma_last-gamma}, {e^{gamma_last}, gamma_last}
+//                                               sk = rk e^{gamma_last-gamma}, {e^{gamma_last}, gamma_last, is_linear}
 //                        (rq, rk = reciprocal L2 norms, or 1).
 //
 //   linear_scan_kernel   one workgroup per (sequence, head, 32-wide slice of V) walks the chunks
@@ -29,6 +29,7 @@
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
 #include "natsl_device.h"
 #include "natsl_host.h"
+#include <stdlib.h>
 
 namespace natsl {
 
@@ -85,12 +86,13 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
-  int bos, len, c;
+  int bos, len, c, bos_nats;
   if (p.seqs == nullptr) {
     const int n = gc / p.nt;
     c = gc - n * p.nt;
     bos = n * p.T;
     len = p.T;
+    bos_nats = n * p.TN;
   } else {
     int n = 0;
     for (int i = 1; i < p.n_seqs; ++i)
@@ -98,6 +100,7 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     c = gc - p.seqs[n].chunk_off;
     bos = p.seqs[n].bos;
     len = p.seqs[n].eos - bos;
+    bos_nats = p.seqs[n].bos_nats;
   }
   const int t0 = c * C;
   const bool l2 = (p.flags & NATSL_QK_L2NORM) != 0;
@@ -198,6 +201,12 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     Sout[2 * C + lane] = rk[lane] * __expf(dk);
     if (lane == 0) Sout[3 * C] = __expf(gl);
     if (lane == 1) Sout[3 * C + 1] = gl;
+    if (lane == 2) {
+      // is this chunk's selector block typed linear?  (kept next to the decay so the scan finds it
+      // in the cache line it prefetches anyway)
+      const int hn = h / (p.H / p.HN);
+      Sout[3 * C + 2] = lin_type(p.types, p.types_dtype, ((size_t)(bos_nats + (c * C) / p.block) * p.HN + hn) * 2 + 1) ? 1.f : 0.f;
+    }
   }
   if (!DELTA) return;
   __syncthreads();
@@ -286,7 +295,7 @@ NATSL_DEVICE u32x2 pack4(f32x4 v) {
 }
 
 template <int DK, bool DELTA>
-__global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) {
+__global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams p) {
   constexpr int KS = DK / 32;   // MFMA k-steps over the key dimension
   constexpr int MT = DK / 64;   // 16-row state tiles per wave
   constexpr int KP = DK + 8;    // kbuf / ST row pitch (elements)
@@ -298,6 +307,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
   __shared__ __align__(16) bf16_t XT[BV * XP];
   __shared__ __align__(16) bf16_t VNT[BV * XP];
   __shared__ __align__(16) bf16_t VTT[BV * XP];
+  __shared__ __align__(16) bf16_t Os[C * VP];  // output tile, row-major, for 16-byte stores
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int i16 = lane & 15, g4 = lane >> 4;
@@ -309,12 +319,12 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
   const int split = slot % nsplit;
   const int chain = (slot / nsplit) * 8 + xcd;
   if (chain >= n_chains) return;
-  const int n = chain / p.H, h = chain % p.H, hn = h / (p.H / p.HN);
-  int bos, len, bos_nats, chunk_off;
+  const int n = chain / p.H, h = chain % p.H;
+  int bos, len, chunk_off;
   if (p.seqs == nullptr) {
-    bos = n * p.T; len = p.T; bos_nats = n * p.TN; chunk_off = n * p.nt;
+    bos = n * p.T; len = p.T; chunk_off = n * p.nt;
   } else {
-    bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; bos_nats = p.seqs[n].bos_nats; chunk_off = p.seqs[n].chunk_off;
+    bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; chunk_off = p.seqs[n].chunk_off;
   }
   const int NT = (len + C - 1) / C;
   const int per_blk = p.block / C;
@@ -349,69 +359,69 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
   };
 
   // ---- operand staging ------------------------------------------------------------------------
-  bf16x8 kA[KS], qA[KS], TA[2], PA[2];
-  f32x4 se, sq, sk;
-  float dec = 1.f, glast = 0.f;
-  u32x4 vld;
+  // Two register sets, used alternately by the two halves of the (unrolled-by-2) chunk loop: while
+  // one set feeds the matrix cores the other receives the next chunk's loads.
+  struct Operands {
+    bf16x8 kA[KS], qA[KS], TA[2], PA[2];
+    f32x4 se, sq, sk;
+    float dec, glast, linf;
+    u32x4 vld;
+  };
   const int a_row = 16 * wave + i16;          // this lane's A-operand row (token within the chunk)
   const int v_ld_row = tid >> 2, v_ld_seg = tid & 3;
-  auto gload = [&](int c) {
-    const int tok = c * C + a_row;
-    const bool ok = tok < len;
-    const bf16_t* kr = kp + (size_t)tok * qk_row + 8 * g4;
-    const bf16_t* qr = qp + (size_t)tok * qk_row + 8 * g4;
+  const int r0 = 16 * wave + 4 * g4;          // first of this lane's four accumulator rows
+  // running pointers, advanced by one chunk per load; rows past the end of the sequence are clamped
+  // (beta = 0 there makes their v_new exactly 0, and their outputs are never stored)
+  const bf16_t* k_ptr = kp + 8 * g4;
+  const bf16_t* q_ptr = qp + 8 * g4;
+  const bf16_t* v_ptr = vp + 8 * v_ld_seg;
+  const size_t unit0 = (size_t)chunk_off * p.H + h;
+  const bf16_t* P_ptr = p.ws_p + unit0 * (C * C) + a_row * C + 8 * g4;
+  const bf16_t* T_ptr = p.ws_tm + unit0 * (C * C) + a_row * C + 8 * g4;
+  const float* sc_ptr = p.ws_sc + unit0 * (4 * C);
+  const size_t unit_step = (size_t)p.H * (C * C), sc_step = (size_t)p.H * (4 * C);
+  int next_c = 0;
+  auto gload = [&](Operands& A) {
+    const int tok = min(next_c * C + a_row, len - 1);
+    const bf16_t* kr = k_ptr + (size_t)tok * qk_row;
+    const bf16_t* qr = q_ptr + (size_t)tok * qk_row;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      kA[s] = ok ? ld8(kr + 32 * s) : zero8();
-      qA[s] = ok ? ld8(qr + 32 * s) : zero8();
+      A.kA[s] = ld8(kr + 32 * s);
+      A.qA[s] = ld8(qr + 32 * s);
     }
-    const size_t unit = (size_t)(chunk_off + c) * p.H + h;
-    const bf16_t* Pm = p.ws_p + unit * (C * C) + a_row * C + 8 * g4;
-    PA[0] = ld8(Pm);
-    PA[1] = ld8(Pm + 32);
+    A.PA[0] = ld8(P_ptr);
+    A.PA[1] = ld8(P_ptr + 32);
     if (DELTA) {
-      const bf16_t* Tm = p.ws_tm + unit * (C * C) + a_row * C + 8 * g4;
-      TA[0] = ld8(Tm);
-      TA[1] = ld8(Tm + 32);
+      A.TA[0] = ld8(T_ptr);
+      A.TA[1] = ld8(T_ptr + 32);
     }
-    const float* sc = p.ws_sc + unit * (4 * C);
-    const int r0 = 16 * wave + 4 * g4;
-    se = *reinterpret_cast<const f32x4*>(sc + r0);
-    sq = *reinterpret_cast<const f32x4*>(sc + C + r0);
-    sk = *reinterpret_cast<const f32x4*>(sc + 2 * C + r0);
-    dec = sc[3 * C];
-    glast = sc[3 * C + 1];
-    const int vt = c * C + v_ld_row;
+    A.se = *reinterpret_cast<const f32x4*>(sc_ptr + r0);
+    A.sq = *reinterpret_cast<const f32x4*>(sc_ptr + C + r0);
+    A.sk = *reinterpret_cast<const f32x4*>(sc_ptr + 2 * C + r0);
+    A.dec = sc_ptr[3 * C];
+    A.glast = sc_ptr[3 * C + 1];
+    A.linf = sc_ptr[3 * C + 2];
+    const int vt = next_c * C + v_ld_row;
     const u32x4 z = {0u, 0u, 0u, 0u};
-    vld = vt < len ? *reinterpret_cast<const u32x4*>(vp + (size_t)vt * v_row + 8 * v_ld_seg) : z;
+    A.vld = vt < len ? *reinterpret_cast<const u32x4*>(v_ptr + (size_t)vt * v_row) : z;  // v must be 0 past the end
+    P_ptr += unit_step;
+    T_ptr += unit_step;
+    sc_ptr += sc_step;
+    ++next_c;
   };
-  auto lstore = [&](int buf) {
+  auto lstore = [&](const Operands& A, int buf) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]) = kA[s];
-    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = vld;
+    for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]) = A.kA[s];
+    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = A.vld;
   };
 
-  if (NT > 0) {
-    gload(0);
-    lstore(0);
-  }
-  write_ST();
   float gsum = 0.f;
-
-  for (int c = 0; c < NT; ++c) {
-    const int buf = c & 1;
+  // one chunk: CUR holds its operands (already staged in kbuf/vbuf[buf]); NXT receives the next chunk's
+  auto step = [&](const int c, const int buf, const Operands& CUR, Operands& NXT) {
     __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
-
-    // operands of this step, kept while the next step's loads are in flight
-    bf16x8 kC[KS], qC[KS], TC[2], PC[2];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) { kC[s] = kA[s]; qC[s] = qA[s]; }
-    PC[0] = PA[0]; PC[1] = PA[1];
-    if (DELTA) { TC[0] = TA[0]; TC[1] = TA[1]; }
-    const f32x4 seC = se, sqC = sq, skC = sk;
-    const float decC = dec, glC = glast;
-    (void)seC; (void)TC;
-    if (c + 1 < NT) gload(c + 1);
+    const bool more = c + 1 < NT;
+    if (more) gload(NXT);
 
     if (c % per_blk == 0) {
 #pragma unroll
@@ -430,11 +440,11 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
       const bf16x8 sb0 = ld8(ST + i16 * KP + 32 * s + 8 * g4);
       const bf16x8 sb1 = ld8(ST + (16 + i16) * KP + 32 * s + 8 * g4);
       if (DELTA) {
-        R[0] = mfma16(kC[s], sb0, R[0]);
-        R[1] = mfma16(kC[s], sb1, R[1]);
+        R[0] = mfma16(CUR.kA[s], sb0, R[0]);
+        R[1] = mfma16(CUR.kA[s], sb1, R[1]);
       }
-      O1[0] = mfma16(qC[s], sb0, O1[0]);
-      O1[1] = mfma16(qC[s], sb1, O1[1]);
+      O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
+      O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
     }
     // (2) v in accumulator layout via the transposing read; X = v - se * R
     f32x4 VN[2];
@@ -449,7 +459,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
       for (int nn = 0; nn < 2; ++nn) {
         f32x4 X;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - seC[r] * R[nn][r];
+        for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - CUR.se[r] * R[nn][r];
         *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(X);
       }
       __syncthreads();
@@ -458,7 +468,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
       for (int nn = 0; nn < 2; ++nn) {
         VN[nn] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < 2; ++s) VN[nn] = mfma16(TC[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
+        for (int s = 0; s < 2; ++s) VN[nn] = mfma16(CUR.TA[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
       }
     }
     // (4) v_new and sk * v_new, transposed, for the two products that reduce over tokens
@@ -466,7 +476,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
     for (int nn = 0; nn < 2; ++nn) {
       f32x4 vt;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) vt[r] = VN[nn][r] * skC[r];
+      for (int r = 0; r < 4; ++r) vt[r] = VN[nn][r] * CUR.sk[r];
       *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(VN[nn]);
       *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
     }
@@ -476,23 +486,26 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
     for (int nn = 0; nn < 2; ++nn) {
       f32x4 O;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) O[r] = O1[nn][r] * sqC[r];
+      for (int r = 0; r < 4; ++r) O[r] = O1[nn][r] * CUR.sq[r];
       if (intra) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) O = mfma16(PC[s], ld8(VNT + (16 * nn + i16) * XP + 32 * s + 8 * g4), O);
+        for (int s = 0; s < 2; ++s) O = mfma16(CUR.PA[s], ld8(VNT + (16 * nn + i16) * XP + 32 * s + 8 * g4), O);
       }
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int tok = c * C + 16 * wave + 4 * g4 + r;
-        if (tok < len) op[(size_t)tok * v_row + 16 * nn + i16] = f32_to_bf16(O[r]);
-      }
+      for (int r = 0; r < 4; ++r) Os[(r0 + r) * VP + 16 * nn + i16] = f32_to_bf16(O[r]);
+    }
+    {
+      // each wave stores the 16 rows it owns: 4 lanes x 16 bytes per row
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+      const int row = 16 * wave + (lane >> 2), tok = c * C + row;
+      if (tok < len)
+        *reinterpret_cast<u32x4*>(op + (size_t)tok * v_row + 8 * (lane & 3)) = *reinterpret_cast<const u32x4*>(Os + row * VP + 8 * (lane & 3));
     }
     // (6) state update / roll-back
-    const int blk = (c * C) / p.block;
-    const bool is_lin = lin_type(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2 + 1);
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
-    gsum += glC;
-    if (is_lin || !last_of_block) {
+    gsum += CUR.glast;
+    if (CUR.linf != 0.f || !last_of_block) {
 #pragma unroll
       for (int mi = 0; mi < MT; ++mi) {
         const int m = wave * MT + mi;
@@ -505,7 +518,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
 #pragma unroll
         for (int nn = 0; nn < 2; ++nn) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= decC;
+          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= CUR.dec;
 #pragma unroll
           for (int s = 0; s < 2; ++s) S[mi][nn] = mfma16(kt[s], ld8(VTT + (16 * nn + i16) * XP + 32 * s + 8 * g4), S[mi][nn]);
         }
@@ -521,7 +534,18 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const LinearParams p) 
     }
     // (7) bf16 copy of the state and the staged k, v tiles for the next step
     write_ST();
-    if (c + 1 < NT) lstore(buf ^ 1);
+    if (more) lstore(NXT, buf ^ 1);
+  };
+
+  Operands A0, A1;
+  if (NT > 0) {
+    gload(A0);
+    lstore(A0, 0);
+  }
+  write_ST();
+  for (int c = 0; c < NT; c += 2) {
+    step(c, 0, A0, A1);
+    if (c + 1 < NT) step(c + 1, 1, A1, A0);
   }
 
   if (p.ht) {
