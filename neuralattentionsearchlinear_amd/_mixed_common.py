@@ -39,8 +39,9 @@ def _no_backward(*tensors):
 
 
 def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block: int, flags: int,
-                     output_final_state: bool, seqs: Optional[PackedSeqs]):
-    """Launch the chunked linear branch ('gdn' or 'mamba'); returns (o, final_state or None)."""
+                     output_final_state: bool, seqs: Optional[PackedSeqs], block_start_state: bool = False):
+    """Launch the chunked linear branch ('gdn' or 'mamba'); returns (o, final_state or None), or with
+    block_start_state (o, final_state, state entering the last block, sum of g over the last block)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     TN, HN = types.shape[1], types.shape[2]
@@ -51,12 +52,14 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
     ws = torch.empty(L.natsl_linear_workspace_bytes(total_chunks, H), dtype=torch.uint8, device=dev)
     o = torch.empty(B, T, H, V, dtype=q.dtype, device=dev)
     ht = torch.empty(n, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
+    hs = torch.empty(n, H, K, V, dtype=torch.float32, device=dev) if block_start_state else None
+    gs = torch.empty(n, H, dtype=torch.float32, device=dev) if block_start_state else None
     if h0 is not None:
         if tuple(h0.shape) != (n, H, K, V):
             raise ValueError(f"initial state must have shape {(n, H, K, V)}, got {tuple(h0.shape)}")
         h0 = h0.to(torch.float32).contiguous()
     sp, ns, tot = _seq_args(seqs, total_chunks)
-    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
+    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(hs), _capi.ptr(gs), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
               block, float(scale), flags, _capi.ptr(ws), ws.numel(), _capi.dtype_code(q.dtype), sp, ns, tot,
               _capi.stream_ptr(dev))
     if kind == 'gdn':
@@ -65,13 +68,18 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
     else:
         rc = L.natsl_mamba_chunk_fwd(_capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), *common)
         _capi.check(rc, "natsl_mamba_chunk_fwd")
+    if block_start_state:
+        return o, ht, hs, gs
     return o, ht
 
 
 def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
                   scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size, attn_sw_size,
                   attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
-                  incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool):
+                  incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
+                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0):
+    """Shared forward of the mixed operators.  With inference=True it also returns the state at the
+    start of the current selector block (4-tuple), as the reference's *_chunk_inference operators do."""
     if nats_block_size < CHUNK_SIZE:
         raise AssertionError("nats_block_size must be at least the compute chunk (64)")   # mixed_attn_gdn.py:90
     if nats_block_size % CHUNK_SIZE:
@@ -82,6 +90,10 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
         raise NotImplementedError("use_g_for_attn is disabled in every reference layer and is not built")
     if lin_intra and not incomplete_block_start_with_ht:
         raise NotImplementedError("incomplete_block_start_with_ht=False is not built")
+    if n_tokens_in_current_block != 0:
+        raise NotImplementedError("n_tokens_in_current_block != 0 is never passed by the reference layers and is not built")
+    if inference and (cu_seqlens is not None):
+        raise NotImplementedError("packed sequences are not supported by the prefill hand-off")
     if not q_lattn.is_cuda:
         raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
     _no_backward(q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types)
@@ -116,12 +128,33 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
     flags = (_capi.DECAY_NON_LINEAR if decay_non_linear else 0) | (_capi.QK_L2NORM if qk_l2norm else 0) | \
             (_capi.INTRA_CHUNK if lin_intra else 0)
     _mark("linear:start", cur)
-    o_lin, ht = linear_chunk_fwd(kind, q_lattn, k_lattn, v_lattn, g, beta, initial_state, types, scale_lattn,
-                                 nats_block_size, flags, output_final_state, seqs)
+    want_start = inference and output_final_state
+    res = linear_chunk_fwd(kind, q_lattn, k_lattn, v_lattn, g, beta, initial_state, types, scale_lattn,
+                           nats_block_size, flags, output_final_state, seqs, block_start_state=want_start)
+    o_lin, ht = res[0], res[1]
     _mark("linear:end", cur)
     cur.wait_stream(side)
     for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
         t.record_stream(side)
     if io_dtype != torch.bfloat16:
         o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
-    return o_lin, o_attn, ht
+    if not inference:
+        return o_lin, o_attn, ht
+    h_start = None
+    if want_start:
+        # State at the start of the current block (src/nats/ops/gated_delta_rule/chunk_fwd.py:178-206):
+        # with an incomplete last block it is the state that entered that block; when the input ends on
+        # a block boundary it is the state after the last block under its TRUE type -- the final state
+        # if that type is linear, otherwise the entering state rolled forward by the block's decay.
+        hs, gs = res[2], res[3]
+        if T % nats_block_size != 0:
+            h_start = hs
+        else:
+            if op_type_last_chunk is None:
+                raise AssertionError("op_type_last_chunk is required when the input ends on a block boundary")
+            H = ht.shape[1]
+            lin = (op_type_last_chunk[..., 1] > 0)
+            lin = lin.repeat_interleave(H // lin.shape[1], dim=1).view(ht.shape[0], H, 1, 1)
+            rolled = hs * torch.exp(gs).view(ht.shape[0], H, 1, 1) if decay_non_linear else hs
+            h_start = torch.where(lin, ht, rolled)
+    return o_lin, o_attn, ht, h_start

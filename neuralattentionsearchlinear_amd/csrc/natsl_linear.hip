@@ -42,6 +42,8 @@ struct LinearParams {
   const float* h0;
   bf16_t* o;
   float* ht;
+  float* hs;      // state entering each sequence's last selector block (optional)
+  float* gs;      // sum of g over that block, [N,H] (optional)
   const void* types;
   int types_dtype;
   const SeqRow* seqs;
@@ -548,6 +550,19 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     if (c + 1 < NT) step(c + 1, 1, A1, A0);
   }
 
+  if (p.hs) {
+    // Ssave / gsum still belong to the last block: the state that entered it and its total log-decay
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+      for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
+          p.hs[((size_t)chain * DK + kd) * p.V + vc] = Ssave[mi][nn][r];
+        }
+    if (p.gs && split == 0 && tid == 0) p.gs[chain] = gsum;
+  }
   if (p.ht) {
 #pragma unroll
     for (int mi = 0; mi < MT; ++mi)
@@ -577,8 +592,8 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
-                      const float* h0, void* o, float* ht, const void* types, int types_dtype, int B, int T, int H, int HN,
-                      int K, int V, int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
+                      const float* h0, void* o, float* ht, float* hs, float* gs, const void* types, int types_dtype, int B, int T,
+                      int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                       int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream) {
   const char* what = delta ? "natsl_gdn_chunk_fwd" : "natsl_mamba_chunk_fwd";
   if (!q || !k || !v || !g || !o || !types || (delta && !beta)) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
@@ -592,7 +607,7 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
     return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   LinearParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.g = g; p.beta = (const bf16_t*)beta;
-  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.types = types; p.types_dtype = types_dtype;
+  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.hs = hs; p.gs = gs; p.types = types; p.types_dtype = types_dtype;
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block;
   p.nt = cdiv(T, C);
@@ -626,19 +641,20 @@ extern "C" size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H) {
 }
 
 extern "C" int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
-                                   const float* h0, void* o, float* ht, const void* types, int types_dtype, int B, int T,
+                                   const float* h0, void* o, float* ht, float* h_block_start, float* g_block_sum,
+                                   const void* types, int types_dtype, int B, int T,
                                    int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
                                    size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                    natsl_stream_t stream) {
-  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
+  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, h_block_start, g_block_sum, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
                     workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }
 
 extern "C" int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* h0, void* o,
-                                     float* ht, const void* types, int types_dtype, int B, int T, int H, int HN, int K, int V,
+                                     float* ht, float* h_block_start, float* g_block_sum, const void* types, int types_dtype, int B, int T, int H, int HN, int K, int V,
                                      int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                                      int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                      natsl_stream_t stream) {
-  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
+  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, h_block_start, g_block_sum, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
                     flags & ~NATSL_QK_L2NORM, workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }

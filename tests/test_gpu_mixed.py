@@ -135,3 +135,48 @@ def test_errors_mirror_reference():
         nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, attn_sw_size=128)
     with pytest.raises(NotImplementedError):
         nats_mixed_attn_gdn(q.requires_grad_(), k, v, q, k, v, None, g, beta, ty, None)
+
+
+@pytest.mark.parametrize("decay", [True, False])
+@pytest.mark.parametrize("T", [512, 480])       # ends on a block boundary / inside a block
+def test_gdn_chunk_inference_block_start_state(T, decay):
+    """The prefill hand-off.  Pinned by the token-level recurrence under the TRUE block types: the state at
+    the start of the current block is the final state of the recurrence over the complete blocks."""
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn_chunk_inference
+    from oracle import linear_branch as lb
+    B, H, K, V, block = 2, 4, 64, 64, 64
+    q, k, v = make_qkv(B, T, H, K, V, 21)
+    g, beta = make_gates(B, T, H, 22)
+    NB = -(-T // block)
+    true_ty = make_types(B, NB, H, 0.5, 23, torch.bfloat16, force_last=False)
+    forced = true_ty.clone(); forced[:, -1] = 1
+    init = torch.randn(B, H, K, V, generator=torch.Generator().manual_seed(24)) * 0.5
+    n_complete = T // block
+    Tc = n_complete * block
+    _, S_start_ref = lb.gdn_token_recurrence(q[:, :Tc], k[:, :Tc], v[:, :Tc], g[:, :Tc], beta[:, :Tc], true_ty[:, :n_complete, :, 1],
+                                             K ** -0.5, init, block, decay, dtype=torch.float64)
+    o_ref, S_ref = lb.gdn_token_recurrence(q, k, v, g, beta, forced[..., 1], K ** -0.5, init, block, decay, dtype=torch.float64)
+    op_last = true_ty[:, -1].clone() if T % block == 0 else None
+    with torch.no_grad():
+        o, o_attn, S, S_start = nats_mixed_attn_gdn_chunk_inference(
+            *_to(q, k, v, q, k, v, init), g.to(DEV), beta.to(DEV), forced.to(DEV), None if op_last is None else op_last.to(DEV), None,
+            nats_block_size=block, ops_for_incomplete_chunks='all', output_final_state_gated_delta=True,
+            decay_for_non_gdn_blocks=decay)
+    assert_close(o.float(), o_ref, "o_gdn"); assert_close(S, S_ref, "final_state"); assert_close(S_start, S_start_ref, "block_start_state")
+
+
+def test_mamba_chunk_inference_block_start_state():
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba_chunk_inference
+    from oracle import linear_branch as lb
+    torch.manual_seed(3)
+    B, T, H, K, V, block = 1, 640, 4, 128, 64, 128
+    q = F.normalize(torch.randn(B, T, H, K), dim=-1).bfloat16(); k = F.normalize(torch.randn(B, T, H, K), dim=-1).bfloat16()
+    dt = F.softplus(torch.randn(B, T, H) - 3); v = (torch.randn(B, T, H, V) * dt[..., None]).bfloat16(); g = -2.0 * dt
+    true_ty = make_types(B, T // block, H, 0.5, 31, torch.bfloat16, force_last=False)
+    forced = true_ty.clone(); forced[:, -1] = 1
+    _, S_start_ref = lb.mamba_token_recurrence(q, k, v, g, true_ty[..., 1], 1.0, None, block, True)
+    o_ref, S_ref = lb.mamba_token_recurrence(q, k, v, g, forced[..., 1], 1.0, None, block, True)
+    with torch.no_grad():
+        o, _, S, S_start = nats_mixed_attn_mamba_chunk_inference(*_to(q, k, v, q, k, v), None, g.to(DEV), forced.to(DEV), true_ty[:, -1].to(DEV),
+                                                                 None, scale_lattn=1, nats_block_size=block)
+    assert_close(o.float(), o_ref, "o_mamba"); assert_close(S, S_ref, "final_state"); assert_close(S_start, S_start_ref, "block_start_state")
