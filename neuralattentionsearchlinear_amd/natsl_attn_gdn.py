@@ -1,0 +1,182 @@
+"""Gated-DeltaNet / softmax hybrid token mixer with the forward signature, returns and parameter
+names of the reference layer (src/nats/layers/natsl_attn_gdn.py:64-666).
+
+Projections, short convolutions and norms are torch; block pooling, the selector, the mixed operator
+and the output norm-gate are the HIP kernels of this package.  Forward only: there is no backward, no
+decode (q_len < 64) path and no NAtSCache -- those raise NotImplementedError.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import nats_util
+from .mixed_attn_gdn import nats_mixed_attn_gdn, nats_mixed_attn_gdn_chunk_inference
+from .modules import FusedMultiInputRMSNormGated, RMSNorm, ShortConvolution
+
+
+class NeuralAttentionSearchLinearAttnGDN(nn.Module):
+    def __init__(self, hidden_size: int = 2048, expand_v: float = 2, head_dim: int = 256, num_heads: int = 6,
+                 num_attn_heads: int = 24, num_v_heads: int = None, n_ops: int = 2, num_nats_head: Optional[int] = None,
+                 nats_block_size: int = 64, nats_block_agg_type: str = 'mean', nats_sample_strategy: str = 'argmax',
+                 ops_for_incomplete_chunks: str = 'all', mode: str = 'chunk', use_gate: bool = True,
+                 use_short_conv: bool = True, allow_neg_eigval: bool = False, conv_size: int = 4, conv_bias: bool = False,
+                 conv_activation: Optional[str] = 'silu', outputs_are_weighted: bool = True, attn_qk_norm: bool = True,
+                 attn_with_short_conv: bool = True, compute_dnats_for_invalid_blocks_attn: bool = False,
+                 compute_dnats_for_invalid_blocks_linear_att: bool = False, decay_for_non_gdn_blocks: bool = True,
+                 incomplete_block_start_with_ht: bool = True, attn_apply_pos_encoding: bool = False,
+                 attn_rope_theta: Optional[float] = 10000., attn_max_position_embeddings: Optional[int] = None,
+                 layer_idx: int = None, norm_eps: float = 1e-5, **kwargs):
+        super().__init__()
+        if n_ops != 2:
+            raise NotImplementedError("two ops (softmax, linear) are built")
+        if nats_block_agg_type != 'mean':
+            raise NotImplementedError(f"Pooling system {nats_block_agg_type} is not supported!")
+        if nats_sample_strategy != 'argmax':
+            raise NotImplementedError("only the hard (argmax) selector is built")
+        if attn_apply_pos_encoding:
+            raise NotImplementedError("rotary position encoding for the attention view is not built")
+        if not use_gate or not outputs_are_weighted:
+            raise NotImplementedError("only use_gate=True with weighted outputs (the published configuration) is built")
+        assert mode in ['chunk', 'fused_recurrent'], f"Not supported mode `{mode}`."
+        self.mode, self.hidden_size, self.expand_v = mode, hidden_size, expand_v
+        self.allow_neg_eigval, self.use_gate, self.use_short_conv = allow_neg_eigval, use_gate, use_short_conv
+        self.conv_size, self.conv_bias = conv_size, conv_bias
+        self.head_dim, self.num_heads = head_dim, num_heads
+        self.num_v_heads = num_v_heads if num_v_heads is not None else num_heads
+        self.n_ops = n_ops
+        self.head_k_dim = head_dim
+        self.head_v_dim = int(head_dim * expand_v)
+        self.key_dim = int(num_heads * self.head_k_dim)
+        self.value_dim = int(self.num_v_heads * self.head_v_dim)
+        self.layer_idx = layer_idx
+        self.attn_qk_norm, self.num_attn_heads = attn_qk_norm, num_attn_heads
+        self.head_attn_k_dim = self.key_dim // num_attn_heads
+        self.head_attn_v_dim = self.value_dim // num_attn_heads
+        self.attn_with_short_conv = attn_with_short_conv
+        self.incomplete_block_start_with_ht = incomplete_block_start_with_ht
+        self.decay_for_non_gdn_blocks = decay_for_non_gdn_blocks
+        self.compute_dnats_for_invalid_blocks_attn = compute_dnats_for_invalid_blocks_attn
+        self.compute_dnats_for_invalid_blocks_linear_att = compute_dnats_for_invalid_blocks_linear_att
+        self.nats_block_size = nats_block_size
+        self.num_nats_head = num_heads if num_nats_head is None else num_nats_head
+        self.ops_for_incomplete_chunks = ops_for_incomplete_chunks
+        self.outputs_are_weighted = outputs_are_weighted
+        if not math.isclose(self.num_v_heads * head_dim * expand_v, self.value_dim, rel_tol=1e-5):
+            raise ValueError(f"expand_v={expand_v} does not produce an integer value_dim")
+        if self.num_v_heads > num_heads and self.num_v_heads % num_heads != 0:
+            raise ValueError(f"num_v_heads={self.num_v_heads} must be divisible by num_heads={num_heads}.")
+        if num_attn_heads > num_heads and num_attn_heads % num_heads != 0:
+            raise ValueError(f"num_attn_heads={num_attn_heads} must be divisible by num_heads={num_heads}.")
+
+        if attn_qk_norm:
+            self.q_norm = RMSNorm(self.head_attn_k_dim, eps=norm_eps)
+            self.k_norm = RMSNorm(self.head_attn_k_dim, eps=norm_eps)
+        self.q_proj = nn.Linear(hidden_size, self.key_dim, bias=False)
+        self.k_proj = nn.Linear(hidden_size, self.key_dim, bias=False)
+        self.v_proj = nn.Linear(hidden_size, self.value_dim, bias=False)
+        self.a_proj = nn.Linear(hidden_size, self.num_v_heads, bias=False)
+        self.b_proj = nn.Linear(hidden_size, self.num_v_heads, bias=False)
+        self.nats_layer = nn.Linear(hidden_size, n_ops * self.num_nats_head, bias=False)
+        A = torch.empty(self.num_v_heads, dtype=torch.float32).uniform_(0, 16)
+        self.A_log = nn.Parameter(torch.log(A))
+        dt = torch.exp(torch.rand(self.num_v_heads) * (math.log(0.1) - math.log(0.001)) + math.log(0.001)).clamp(min=1e-4)
+        self.dt_bias = nn.Parameter(dt + torch.log(-torch.expm1(-dt)))
+        self.nats_out_weights_layer = nn.Linear(self.key_dim, n_ops * num_attn_heads, bias=False)
+        if use_short_conv:
+            self.q_conv1d = ShortConvolution(self.key_dim, conv_size, conv_bias, conv_activation)
+            self.k_conv1d = ShortConvolution(self.key_dim, conv_size, conv_bias, conv_activation)
+            self.v_conv1d = ShortConvolution(self.value_dim, conv_size, conv_bias, conv_activation)
+        self.g_proj = nn.Linear(hidden_size, self.value_dim, bias=False)
+        self.o_norm = FusedMultiInputRMSNormGated(self.head_attn_v_dim, eps=norm_eps)
+        self.o_proj = nn.Linear(self.value_dim, hidden_size, bias=False)
+        self.attn_fraction = torch.zeros(1)
+
+    # -- pieces of the forward, also used by the parity test ---------------------------------------
+    def select_ops(self, hidden_states: torch.Tensor, cu_seqlens=None):
+        """Selector: block means -> nats_layer -> hard selection with the last block forced to both ops
+        (reference :411-420, :553-555, :579-583).  Returns (types [B,TN,HN,2], n_nats_blocks int32 [B,HN,2],
+        the last block's type before forcing [B,HN,2])."""
+        B, _, dim = hidden_states.shape
+        pooled = nats_util.mean_pooling(hidden_states.unsqueeze(-2), self.nats_block_size, cu_seqlens=cu_seqlens)
+        pooled = pooled.view(B, pooled.shape[1], dim)
+        logits = self.nats_layer(pooled).unflatten(-1, (self.num_nats_head, self.n_ops))
+        types, n_blocks = nats_util.hard_select(logits, force_last_block=False)
+        last = types[:, -1].clone()
+        n_blocks = n_blocks + (1 - last.to(torch.int32))      # counts after forcing the last block to 1
+        types[:, -1] = 1
+        return types, n_blocks, last
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_values=None,
+                use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False, **kwargs):
+        if attention_mask is not None:
+            assert len(attention_mask.shape) == 2, "Expected attention_mask as a 0-1 matrix with shape [batch_size, seq_len]"
+            if len(attention_mask) > 1:
+                raise NotImplementedError("Attention with variable length is not supported yet!")
+        if past_key_values is not None:
+            raise NotImplementedError("the NAtS KV/state cache (decode and chunked prefill continuation) is not built")
+        B, q_len, _ = hidden_states.shape
+        if q_len < 64:
+            raise NotImplementedError("the token-recurrent decode path (q_len < 64) is not built")
+        cu_seqlens = kwargs.get('cu_seqlens', None)
+
+        types, n_nats_blocks, last_type = self.select_ops(hidden_states, cu_seqlens)
+
+        def conv_or_act(x, conv):
+            if self.use_short_conv:
+                return conv(x=x, cache=None, output_final_state=False, cu_seqlens=cu_seqlens)[0]
+            return F.silu(x)
+
+        if self.attn_with_short_conv:
+            q = conv_or_act(self.q_proj(hidden_states), getattr(self, 'q_conv1d', None))
+            k = conv_or_act(self.k_proj(hidden_states), getattr(self, 'k_conv1d', None))
+            v = conv_or_act(self.v_proj(hidden_states), getattr(self, 'v_conv1d', None))
+            q_attn, k_attn, v_attn = q, k, v
+        else:
+            q_attn, k_attn, v_attn = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+            q = conv_or_act(q_attn, getattr(self, 'q_conv1d', None))
+            k = conv_or_act(k_attn, getattr(self, 'k_conv1d', None))
+            v = conv_or_act(v_attn, getattr(self, 'v_conv1d', None))
+        o_weights = self.nats_out_weights_layer(q).unflatten(-1, (self.num_attn_heads, self.n_ops)).softmax(-1)
+
+        q, k = (x.unflatten(-1, (-1, self.head_k_dim)) for x in (q, k))
+        v = v.unflatten(-1, (-1, self.head_v_dim))
+        q_attn, k_attn = (x.unflatten(-1, (-1, self.head_attn_k_dim)) for x in (q_attn, k_attn))
+        v_attn = v_attn.unflatten(-1, (-1, self.head_attn_v_dim))
+        if self.num_v_heads > self.num_heads:
+            q, k = (x.repeat_interleave(self.num_v_heads // self.num_heads, dim=-2) for x in (q, k))
+        if self.attn_qk_norm:
+            q_attn, k_attn = self.q_norm(q_attn), self.k_norm(k_attn)
+
+        beta = self.b_proj(hidden_states).sigmoid()
+        if self.allow_neg_eigval:
+            beta = beta * 2.
+        g = -self.A_log.float().exp() * F.softplus(self.a_proj(hidden_states).float() + self.dt_bias)
+
+        self.attn_fraction = (n_nats_blocks.float()[..., 0] / types.shape[1]).mean(0).detach()
+        common = dict(q_attn=q_attn, k_attn=k_attn, v_attn=v_attn, q_lattn=q, k_lattn=k, v_lattn=v, g=g, beta=beta,
+                      nats_block_types=types, n_nats_blocks=n_nats_blocks, scale_attn=k_attn.shape[-1] ** -0.5,
+                      scale_lattn=k.shape[-1] ** -0.5, cu_seqlens=cu_seqlens, cu_seqlens_nats=None,
+                      nats_block_size=self.nats_block_size, ops_for_incomplete_chunks=self.ops_for_incomplete_chunks,
+                      output_final_state_gated_delta=bool(use_cache),
+                      incomplete_block_start_with_ht=self.incomplete_block_start_with_ht,
+                      decay_for_non_gdn_blocks=self.decay_for_non_gdn_blocks, use_g_for_attn=False,
+                      lattn_use_qk_l2norm_in_kernel=True)
+        if self.training:
+            o_lin, o_attn, self.last_recurrent_state = nats_mixed_attn_gdn(
+                initial_state_gated_delta=None,
+                compute_dnats_for_invalid_blocks_attn=self.compute_dnats_for_invalid_blocks_attn,
+                compute_dnats_for_invalid_blocks_linear_att=self.compute_dnats_for_invalid_blocks_linear_att, **common)
+        else:
+            o_lin, o_attn, self.last_recurrent_state, self.last_block_start_state = nats_mixed_attn_gdn_chunk_inference(
+                initial_state_gated_delta_chunk_start=None,
+                op_type_last_chunk=last_type if q_len % self.nats_block_size == 0 else None, **common)
+
+        gate = self.g_proj(hidden_states).unflatten(-1, (-1, self.head_v_dim))
+        o = self.o_norm(o_lin.reshape(o_attn.shape), o_attn, gate.reshape(o_attn.shape), o_weights)
+        o = self.o_proj(o.flatten(-2))
+        return o, None, past_key_values
