@@ -1,0 +1,70 @@
+"""CPU-only: the C-ABI library builds, loads, and exports every function include/natsl.h declares;
+argument validation runs on the host before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "natsl.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(natsl_[a-z_0-9]+)\s*\(", text)))
+
+
+def _lib():
+    from neuralattentionsearchlinear_amd import _capi
+    if not os.path.exists(_capi.LIB_PATH):
+        from neuralattentionsearchlinear_amd import _build
+        _build.build()
+    return _capi.lib()
+
+
+def test_header_symbols_are_exported():
+    names = _declared()
+    assert len(names) >= 10
+    L = _lib()
+    missing = [n for n in names if not hasattr(L, n)]
+    assert not missing, missing
+    from neuralattentionsearchlinear_amd import _capi
+    assert sorted(_capi.exported_symbols()) == names          # the ctypes table covers the whole header
+    assert L.natsl_version() >= 100
+
+
+def test_argument_validation_needs_no_gpu():
+    L = _lib()
+    # null pointers / bad shapes are rejected on the host, before any launch
+    assert L.natsl_hard_select(None, None, None, 1, 4, 2, 1, 0, None, 0, 0, None) == -1
+    assert b"null" in L.natsl_last_error()
+    assert L.natsl_route(ctypes.c_void_p(16), 1, 1, 4, 2, 256, 32, None, None, None, None, None, None, None, 0, 0, None) == -2
+    assert b"multiple of 64" in L.natsl_last_error()
+    assert L.natsl_linear_workspace_bytes(16384, 16) == 16384 * 16 * (2 * 64 * 64 * 2 + 4 * 64 * 4)
+    p = ctypes.c_void_p(256)
+    rc = L.natsl_softmax_sparse_fwd(p, p, p, p, p, p, 1, p, p, 1, 256, 4, 4, 4, 96, 96, 4, 64, 0.1, 1, 1, None, 0, 0, None)
+    assert rc == -2 and b"head dims" in L.natsl_last_error()
+    rc = L.natsl_gdn_chunk_fwd(p, p, p, p, p, None, p, None, None, None, p, 1, 1, 256, 4, 4, 128, 128, 4, 64, 0.1, 7, p, 16, 1,
+                               None, 0, 0, None)
+    assert rc == -3 and b"workspace" in L.natsl_last_error()
+
+
+def test_no_cpu_fallback():
+    import torch
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    x = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16)
+    g = torch.zeros(1, 64, 1)
+    ty = torch.ones(1, 1, 1, 2)
+    with pytest.raises(_capi.NatslError):
+        nats_mixed_attn_gdn(x, x, x, x, x, x, None, g, g.bfloat16(), ty, None)
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "neuralattentionsearchlinear_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src.replace("no CPU fallback", ""), f"{f} mentions the oracle"
