@@ -53,6 +53,11 @@ def make_inputs(w, torch, device):
     return host, dev
 
 
+# HBM bytes per launch of the dominant kernel (read + written), from FETCH_SIZE / WRITE_SIZE counter runs of this
+# script scaled by a 1 GiB copy in the same run; the counter summaries are kept under profiles/.
+MEASURED_TRAFFIC = {"hybrid_gdn_B8_T8192_H16_d128_p25": 809.0e6 + 302.3e6}
+
+
 def softmax_flops(types, T, block, K, V):
     """2(K+V) * sum over queries of visible keys, mode 'all': own block causally + earlier attention blocks."""
     a = types[..., 0].float().round()                     # [B,NB,HN]
@@ -68,21 +73,23 @@ def gdn_flops(types, K, V, C=64):
     return per * n_all - 2 * C * K * V * (n_all - n_lin)
 
 
-def cpu_baseline(host, w, types_host, torch, max_heads=None):
-    """fp32 oracle on the B=1 slice of the workload (all heads unless max_heads), on the host cores."""
+def cpu_baseline(host, w, types_host, torch, max_heads=None, max_batch=None):
+    """fp32 oracle on a batch/head slice of the workload (full sequence length), on the host cores."""
     from oracle import mixed
     threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     torch.set_num_threads(threads)
     H = w["H"] if max_heads is None else min(w["H"], max_heads)
-    sl = lambda t: t[:1, :, :H].contiguous()
+    Bs = w["B"] if max_batch is None else min(w["B"], max_batch)
+    sl = lambda t: t[:Bs, :, :H].contiguous()
     q, k, v, beta, g = (sl(host[n]) for n in ("q", "k", "v", "beta", "g"))
-    ty = types_host[:1, :, :H].contiguous()
+    ty = types_host[:Bs, :, :H].contiguous()
     t0 = time.perf_counter()
     mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, ops_for_incomplete_chunks='all', output_final_state=True,
                          decay_for_non_gdn_blocks=True, nats_block_size=w["block"])
     dt = time.perf_counter() - t0
-    tok_s = w["T"] / dt * (H / w["H"])
-    sample = f"B=1 slice (of {w['B']}), {H} of {w['H']} heads, full T={w['T']}; {dt:.1f} s of fp32 torch-CPU oracle, scaled per head"
+    tok_s = Bs * w["T"] / dt * (H / w["H"])
+    sample = (f"{Bs} of {w['B']} sequences, {H} of {w['H']} heads, full T={w['T']}; {dt:.1f} s of the fp32 torch-CPU oracle, "
+              f"tokens/s scaled by heads")
     return dict(value=tok_s, unit="tokens/s", cores=threads, kind="port", sample=sample)
 
 
@@ -93,7 +100,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-heads", type=int, default=4, help="heads of the B=1 slice timed on the CPU")
+    ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
+    ap.add_argument("--cpu-batch", type=int, default=4, help="sequences of the slice timed on the CPU")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB device copy after the timed steps, so that a counter run of this "
+                         "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path shards over (batch, head) with no communication and every box has one "
@@ -135,6 +146,12 @@ def main():
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         _mixed_common.TIMING_HOOK = None
+        if args.calibrate_copy:
+            src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+            dst = torch.empty_like(src)
+            dst.copy_(src)  # 1 GiB read + 1 GiB written
+            torch.cuda.synchronize()
+            del src, dst
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     tokens = w["B"] * w["T"]
@@ -152,7 +169,7 @@ def main():
     if f_attn >= f_gdn:
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", kernel="softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
-                    unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=None, launch_ms=sm_ms,
+                    unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=MEASURED_TRAFFIC.get(args.workload), launch_ms=sm_ms,
                     algorithmic_flops=f_attn)
     else:
         # GDN-only workload: HBM-bound; algorithmic bytes = q,k,v read + o written + g,beta + final state
@@ -172,7 +189,7 @@ def main():
         roofline=roof,
     )
     if not args.no_cpu_baseline:
-        rec["cpu_baseline"] = cpu_baseline(host, w, types_host, torch, max_heads=args.cpu_heads)
+        rec["cpu_baseline"] = cpu_baseline(host, w, types_host, torch, max_heads=args.cpu_heads, max_batch=args.cpu_batch)
     print(json.dumps(rec))
 
 

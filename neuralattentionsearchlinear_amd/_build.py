@@ -14,6 +14,7 @@ FLAGS = [
     # keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    *os.environ.get("NATSL_HIPCC_EXTRA", "").split(),  # e.g. -DNATSL_ABLATE for a development build
 ]
 
 

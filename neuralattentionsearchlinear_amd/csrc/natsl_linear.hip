@@ -29,7 +29,9 @@
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
 #include "natsl_device.h"
 #include "natsl_host.h"
-#include <stdlib.h>
+#ifdef NATSL_ABLATE
+#include <stdlib.h>  // development build only: getenv for the ablation switch
+#endif
 
 namespace natsl {
 
@@ -56,6 +58,7 @@ struct LinearParams {
   bf16_t* ws_tm;
   bf16_t* ws_p;
   float* ws_sc;
+  int dbg;
 };
 
 constexpr int C = 64;
@@ -424,6 +427,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
     const bool more = c + 1 < NT;
     if (more) gload(NXT);
+    if (NATSL_ABL(p.dbg & 4)) { __syncthreads(); __syncthreads(); if (more) lstore(NXT, buf ^ 1); return; }
 
     if (c % per_blk == 0) {
 #pragma unroll
@@ -613,6 +617,10 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
   p.nt = cdiv(T, C);
   p.total_chunks = seqs ? total_units : B * p.nt;
   p.scale = scale; p.flags = flags;
+  p.dbg = 0;
+#ifdef NATSL_ABLATE
+  if (getenv("NATSL_DBG")) p.dbg = atoi(getenv("NATSL_DBG"));
+#endif
   const size_t units = (size_t)p.total_chunks * H;
   const size_t need = natsl_linear_workspace_bytes(p.total_chunks, H);
   if (!workspace || workspace_bytes < need) return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);

@@ -9,7 +9,9 @@
 // O^T = V^T P^T.  V^T is read from the row-major V tile with the transposing LDS load.
 #include "natsl_device.h"
 #include "natsl_host.h"
-#include <stdlib.h>
+#ifdef NATSL_ABLATE
+#include <stdlib.h>  // development build only: getenv for the ablation switches
+#endif
 
 namespace natsl {
 
@@ -30,8 +32,8 @@ struct SoftmaxParams {
   int total_tiles;
   float scale_log2;
   int same_block;
-  int variant;
-  int dbg;
+  int variant;  // 1: 128-query tile on 4 waves, 8: 256-query tile on 8 waves, 4: 256-query tile, 64 queries per wave
+  int dbg;      // ablation bits, always 0 unless built with NATSL_ABLATE
 };
 
 NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
@@ -349,8 +351,8 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     bool pending = false;
     for (; it < n_prior_chunks; ++it) {
       const int buf = it & 1;
-      if (it + 1 < n_iters && !(p.dbg & 1)) gload(key_start(it + 1));
-      if (wave_valid && !(p.dbg & 2)) {
+      if (it + 1 < n_iters && !NATSL_ABL(p.dbg & 1)) gload(key_start(it + 1));
+      if (wave_valid && !NATSL_ABL(p.dbg & 2)) {
         scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
         if (needs_rescale<NQ>(mx, m_ref)) {
           pending = true;
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
         }
         exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
       }
-      if (it + 1 < n_iters && !(p.dbg & 1)) lstore(buf ^ 1);
+      if (it + 1 < n_iters && !NATSL_ABL(p.dbg & 1)) lstore(buf ^ 1);
       __syncthreads();
     }
     if (pending) {
@@ -385,7 +387,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     } else {
       active = active && jc < my_chunk && kblk < my_blk && attn_block(kblk);
     }
-    if (active && !(p.dbg & 8)) {
+    if (active && !NATSL_ABL(p.dbg & 8)) {
       if (causal) scores<DK, NQ, true>(Ks + buf * 64 * KP, QB, s, mx, c, lane, qloc0);
       else scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
       if (needs_rescale<NQ>(mx, m_ref)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
@@ -475,8 +477,12 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.total_tiles = seqs ? total_units : B * p.nq_tiles;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.same_block = same_block_visible ? 1 : 0;
-  p.dbg = getenv("NATSL_DBG") ? atoi(getenv("NATSL_DBG")) : 0;
-  p.variant = getenv("NATSL_SOFTMAX_WAVES") ? atoi(getenv("NATSL_SOFTMAX_WAVES")) : 1;
+  p.dbg = 0;
+  p.variant = 1;
+#ifdef NATSL_ABLATE
+  if (getenv("NATSL_DBG")) p.dbg = atoi(getenv("NATSL_DBG"));
+  if (getenv("NATSL_SOFTMAX_WAVES")) p.variant = atoi(getenv("NATSL_SOFTMAX_WAVES"));
+#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define NATSL_SM(KK, VV)                                              \
   if (K == KK && V == VV)                                             \
