@@ -139,6 +139,7 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
       rk[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
     }
   }
+  if (NATSL_ABL(p.dbg & 32)) return;  // loads only
   // ---- gamma = inclusive cumsum of g over the chunk (wave 0), beta -------------------------
   if (wave == 0) {
     const bool ok = t0 + lane < len;
@@ -214,6 +215,7 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     }
   }
   if (!DELTA) return;
+  if (NATSL_ABL(p.dbg & 64)) return;  // no solve, no Tm store
   __syncthreads();
 
   // ---- Tm = (I + A)^-1, fp32, blocked 4x4 with 16x16 blocks ----------------------------------
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     }
   }
   // TmB = Tm * diag(beta), bf16, rows of 16 contiguous elements per thread
-  {
+  if (!NATSL_ABL(p.dbg & 128)) {
     const int row = tid >> 2, cb = tid & 3;
     u32x4 w[2];
 #pragma unroll
@@ -387,6 +389,20 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
   const size_t unit_step = (size_t)p.H * (C * C), sc_step = (size_t)p.H * (4 * C);
   int next_c = 0;
   auto gload = [&](Operands& A) {
+    if (NATSL_ABL(p.dbg & 16)) {
+      // timing experiment: the same bytes with row-contiguous (fully coalesced) lane addressing
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int tok = min(next_c * C + 16 * wave + 4 * s + g4, len - 1);
+        A.kA[s] = ld8(kp + (size_t)tok * qk_row + 8 * i16);
+        A.qA[s] = ld8(qp + (size_t)tok * qk_row + 8 * i16);
+      }
+      const bf16_t* Pb = P_ptr - (a_row * C + 8 * g4), *Tb = T_ptr - (a_row * C + 8 * g4);
+      A.PA[0] = ld8(Pb + (16 * wave + (lane >> 3)) * C + 8 * (lane & 7));
+      A.PA[1] = ld8(Pb + (16 * wave + 8 + (lane >> 3)) * C + 8 * (lane & 7));
+      A.TA[0] = ld8(Tb + (16 * wave + (lane >> 3)) * C + 8 * (lane & 7));
+      A.TA[1] = ld8(Tb + (16 * wave + 8 + (lane >> 3)) * C + 8 * (lane & 7));
+    } else {
     const int tok = min(next_c * C + a_row, len - 1);
     const bf16_t* kr = k_ptr + (size_t)tok * qk_row;
     const bf16_t* qr = q_ptr + (size_t)tok * qk_row;
@@ -400,6 +416,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     if (DELTA) {
       A.TA[0] = ld8(T_ptr);
       A.TA[1] = ld8(T_ptr + 32);
+    }
     }
     A.se = *reinterpret_cast<const f32x4*>(sc_ptr + r0);
     A.sq = *reinterpret_cast<const f32x4*>(sc_ptr + C + r0);

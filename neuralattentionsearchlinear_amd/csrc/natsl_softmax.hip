@@ -67,16 +67,34 @@ NATSL_DEVICE void scores(const bf16_t* Kb, const bf16x8 (&QB)[NQ][DK / 16], f32x
     for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[kt][qt][r] = 0.f;
+  // K operand reads run two k-steps ahead of the matrix instructions that consume them
+  constexpr int AHEAD = 2;
+  bf16x8 ka[KSTEPS][2];
+#pragma unroll
+  for (int st = 0; st < AHEAD; ++st) {
+    ka[st][0] = ld8(Kb + l32 * KP + 16 * st + 8 * hf);
+    ka[st][1] = ld8(Kb + (32 + l32) * KP + 16 * st + 8 * hf);
+  }
 #pragma unroll
   for (int st = 0; st < KSTEPS; ++st) {
-    const bf16x8 ka0 = ld8(Kb + l32 * KP + 16 * st + 8 * hf);
-    const bf16x8 ka1 = ld8(Kb + (32 + l32) * KP + 16 * st + 8 * hf);
+    if (st + AHEAD < KSTEPS) {
+      ka[st + AHEAD][0] = ld8(Kb + l32 * KP + 16 * (st + AHEAD) + 8 * hf);
+      ka[st + AHEAD][1] = ld8(Kb + (32 + l32) * KP + 16 * (st + AHEAD) + 8 * hf);
+    }
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
-      s[0][qt] = mfma32(ka0, QB[qt][st], s[0][qt]);
-      s[1][qt] = mfma32(ka1, QB[qt][st], s[1][qt]);
+      s[0][qt] = mfma32(ka[st][0], QB[qt][st], s[0][qt]);
+      s[1][qt] = mfma32(ka[st][1], QB[qt][st], s[1][qt]);
     }
   }
+  // pin that order: 2*AHEAD reads, then {2 NQ matrix instructions, 2 reads} per k-step
+  __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+  for (int st = 0; st < KSTEPS - AHEAD; ++st) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 2 * NQ, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 2 * NQ * AHEAD, 0);
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     float m = -INFINITY;
@@ -173,7 +191,8 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   __shared__ int lds_list[MAX_LDS_LIST];
   __shared__ int lds_count;
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, so everything derived from it stays scalar
   const int l32 = lane & 31, hf = lane >> 5;
 
   // ---- which (sequence, head, tile) ------------------------------------------------------
@@ -250,17 +269,29 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     if (cnt) atomicAdd(&lds_count, cnt);
   }
   __syncthreads();
-  const int n_prior_chunks = lds_count * per_blk;
+  const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
   const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;
   const int n_iters = n_prior_chunks + n_diag;
 
-  auto key_start = [&](int it) -> int {
-    if (it < n_prior_chunks) {
-      const int j = it / per_blk;
-      const int e = j < MAX_LDS_LIST ? lds_list[j] : list[j * list_stride];
-      return e * Bs + (it - j * per_blk) * 64;
+  // Chunk iterator, all wave-uniform (scalar registers): first the 64-key chunks of the prior
+  // attention blocks in list order, then the chunks from dstart on.
+  int nx_it = 0, nx_j = 0, nx_sub = 0;
+  auto next_key_start = [&]() -> int {
+    int ks;
+    if (nx_it < n_prior_chunks) {
+      int e;
+      if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+      else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
+      ks = e * Bs + nx_sub * 64;
+      if (++nx_sub == per_blk) {
+        nx_sub = 0;
+        ++nx_j;
+      }
+    } else {
+      ks = dstart + (nx_it - n_prior_chunks) * 64;
     }
-    return dstart + (it - n_prior_chunks) * 64;
+    ++nx_it;
+    return ks;
   };
   auto attn_block = [&](int blk) -> bool {
     return type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2);
@@ -295,7 +326,23 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   const int v_seg = (st & 3) + 4 * (st >> 6);      // 64 contiguous bytes per row per wave
   const int v_kg = (st >> 2) & 15;                 // keys 4*v_kg .. 4*v_kg+3
   const bool v_on = do_v_role && v_seg < VSEGS;
-  auto gload = [&](int ks) {
+  // per-thread byte offsets inside a chunk; the chunk's base address is wave-uniform
+  const unsigned k_off = (unsigned)(((size_t)ld_row * krow + ld_seg * 8) * sizeof(bf16_t));
+  const unsigned v_off = (unsigned)(((size_t)(4 * v_kg) * vrow + 8 * v_seg) * sizeof(bf16_t));
+  auto gload_full = [&](int ks) {
+    // a chunk that lies wholly inside the sequence (every prior attention block): scalar base + lane offset
+    if (do_k) {
+      const char* kb = reinterpret_cast<const char*>(kp + (size_t)ks * krow) + k_off;
+#pragma unroll
+      for (int i = 0; i < KL; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(kb + 64 * i);
+    }
+    if (v_on) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        vreg[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(vp + ((size_t)ks + j) * vrow) + v_off);
+    }
+  };
+  auto gload_clamped = [&](int ks) {
     // Rows past the end of the sequence are clamped to its last row: such keys are always hidden
     // by the causal rule (a valid query precedes them), so only finite values are needed there.
     if (do_k) {
@@ -311,6 +358,10 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
         vreg[j] = *reinterpret_cast<const u32x4*>(vp + (size_t)vt_ * vrow + 8 * v_seg);
       }
     }
+  };
+  auto gload = [&](int ks) {
+    if (ks + 64 <= len) gload_full(ks);
+    else gload_clamped(ks);
   };
   auto lstore = [&](int buf) {
     if (do_k) {
@@ -334,9 +385,11 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     }
   };
 
+  int ks_fetch = 0;  // key start of the chunk the next gload brings in (known one iteration ahead)
   if (n_iters > 0) {
-    gload(key_start(0));
+    gload(next_key_start());
     lstore(0);
+    if (n_iters > 1) ks_fetch = next_key_start();
   }
   __syncthreads();
 
@@ -351,7 +404,8 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     bool pending = false;
     for (; it < n_prior_chunks; ++it) {
       const int buf = it & 1;
-      if (it + 1 < n_iters && !NATSL_ABL(p.dbg & 1)) gload(key_start(it + 1));
+      const bool more = it + 1 < n_iters;
+      if (more && !NATSL_ABL(p.dbg & 1)) gload(ks_fetch);
       if (wave_valid && !NATSL_ABL(p.dbg & 2)) {
         scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
         if (needs_rescale<NQ>(mx, m_ref)) {
@@ -360,7 +414,8 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
         }
         exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
       }
-      if (it + 1 < n_iters && !NATSL_ABL(p.dbg & 1)) lstore(buf ^ 1);
+      if (more && !NATSL_ABL(p.dbg & 1) && !NATSL_ABL(p.dbg & 32)) lstore(buf ^ 1);
+      if (it + 2 < n_iters) ks_fetch = next_key_start();
       __syncthreads();
     }
     if (pending) {
@@ -368,6 +423,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
       rescale<DV, NQ>(acc, m_ref, l_run, mx);
       exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
       if (it + 1 < n_iters) lstore(buf ^ 1);
+      if (it + 2 < n_iters) ks_fetch = next_key_start();
       __syncthreads();
       ++it;
     }
@@ -376,7 +432,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   const int my_blk = q0 / Bs;
   for (; it < n_iters; ++it) {
     const int buf = it & 1;
-    if (it + 1 < n_iters) gload(key_start(it + 1));
+    if (it + 1 < n_iters) gload(ks_fetch);
     const int jc = (dstart >> 6) + it - n_prior_chunks;  // absolute chunk index of the keys
     const int kblk = (jc * 64) / Bs;
     bool active = wave_valid, causal = false;
@@ -394,6 +450,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
       exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
     }
     if (it + 1 < n_iters) lstore(buf ^ 1);
+    if (it + 2 < n_iters) ks_fetch = next_key_start();
     __syncthreads();
   }
 
