@@ -178,6 +178,75 @@ NATSL_DEVICE void exp_pv(const bf16_t* VTb, f32x16 (&s)[2][NQ], f32x16 (&acc)[DV
   for (int qt = 0; qt < NQ; ++qt) l_run[qt] += rs[qt];  // partial over this lane's keys; halves are joined in the epilogue
 }
 
+// ---- the same work in halves of 32 keys, for the software-pipelined hot loop (one 32-query tile per wave) ----
+// qk_half    S^T tile of key half kt (8 matrix instructions on one accumulator), K reads two steps ahead
+// half_max   scaled row maximum of one half (both lane halves joined)
+// probs_half P = exp2(S*c - m_ref) for one half, packed to bf16 in the B-operand order; adds the row sums
+// pv_half    O^T += V^T P^T for one half
+template <int DK>
+NATSL_DEVICE void qk_half(const bf16_t* Kb, const int kt, const bf16x8 (&QB)[DK / 16], f32x16& s, const int lane) {
+  constexpr int KP = DK + 8, KSTEPS = DK / 16, AHEAD = 2;
+  const bf16_t* kr = Kb + (32 * kt + (lane & 31)) * KP + 8 * (lane >> 5);
+  bf16x8 ka[KSTEPS];
+#pragma unroll
+  for (int st = 0; st < AHEAD; ++st) ka[st] = ld8(kr + 16 * st);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+  for (int st = 0; st < KSTEPS; ++st) {
+    if (st + AHEAD < KSTEPS) ka[st + AHEAD] = ld8(kr + 16 * (st + AHEAD));
+    s = mfma32(ka[st], QB[st], s);
+  }
+}
+
+template <bool CAUSAL>
+NATSL_DEVICE float half_max(f32x16& s, const int kt, const float c, const int lane, const int qloc0) {
+  const int l32 = lane & 31, hf = lane >> 5;
+  float m = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    if (CAUSAL) {
+      const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3), qloc = qloc0 + l32;
+      if (kloc > qloc) s[r] = -INFINITY;
+    }
+    m = fmaxf(m, s[r]);
+  }
+  return xhalf_max(m) * c;
+}
+
+NATSL_DEVICE void probs_half(const f32x16& s, const float c, const float neg, float& rs, bf16x8 (&PB)[2]) {
+#pragma unroll
+  for (int ss = 0; ss < 2; ++ss) {
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      e[j] = __builtin_amdgcn_exp2f(fmaf(s[8 * ss + j], c, neg));
+      rs += e[j];
+    }
+    u32x4 w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(e[2 * j], e[2 * j + 1]);
+    PB[ss] = __builtin_bit_cast(bf16x8, w);
+  }
+}
+
+template <int DV>
+NATSL_DEVICE void pv_half(const bf16_t* VTb, const int kt, const bf16x8 (&PB)[2], f32x16 (&acc)[DV / 32][1], const int lane) {
+  constexpr int TP = VT_PITCH, VT = DV / 32;
+  const int l32 = lane & 31, hf = lane >> 5;
+#pragma unroll
+  for (int ss = 0; ss < 2; ++ss) {
+    const int kbase = 32 * kt + 16 * ss + 4 * hf;
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+      const bf16_t* vr = VTb + (32 * vt + l32) * TP + kbase;
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
+      const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+      acc[vt][0] = mfma32(__builtin_bit_cast(bf16x8, w), PB[ss], acc[vt][0]);
+    }
+  }
+}
+
 // NQ = 32-query column tiles per wave, NWAVES waves: the workgroup owns QTILE = 32*NQ*NWAVES queries.
 template <int DK, int DV, int NQ, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
@@ -252,50 +321,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     for (int s = 0; s < KSTEPS; ++s) QB[qt][s] = ld8(qr + 16 * s);
   }
 
-  // ---- attention blocks that end at or before dstart: ids into LDS, count ----
-  // (the list is sorted, so the qualifying entries are a prefix of it)
   if (tile_start >= len) return;  // packed input: a sequence's last 256-row table slot may hold no tile of this size
-  if (tid == 0) lds_count = 0;
-  __syncthreads();
-  {
-    int cnt = 0;
-    for (int j = tid; j < n_attn; j += NTHREADS) {
-      const int e = list[j * list_stride];
-      if ((e + 1) * Bs <= dstart) {
-        ++cnt;
-        if (j < MAX_LDS_LIST) lds_list[j] = e;
-      }
-    }
-    if (cnt) atomicAdd(&lds_count, cnt);
-  }
-  __syncthreads();
-  const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
-  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;
-  const int n_iters = n_prior_chunks + n_diag;
-
-  // Chunk iterator, all wave-uniform (scalar registers): first the 64-key chunks of the prior
-  // attention blocks in list order, then the chunks from dstart on.
-  int nx_it = 0, nx_j = 0, nx_sub = 0;
-  auto next_key_start = [&]() -> int {
-    int ks;
-    if (nx_it < n_prior_chunks) {
-      int e;
-      if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
-      else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
-      ks = e * Bs + nx_sub * 64;
-      if (++nx_sub == per_blk) {
-        nx_sub = 0;
-        ++nx_j;
-      }
-    } else {
-      ks = dstart + (nx_it - n_prior_chunks) * 64;
-    }
-    ++nx_it;
-    return ks;
-  };
-  auto attn_block = [&](int blk) -> bool {
-    return type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2);
-  };
 
   f32x16 acc[VT][NQ];
 #pragma unroll
@@ -385,24 +411,183 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     }
   };
 
-  int ks_fetch = 0;  // key start of the chunk the next gload brings in (known one iteration ahead)
-  if (n_iters > 0) {
-    gload(next_key_start());
-    lstore(0);
-    if (n_iters > 1) ks_fetch = next_key_start();
-  }
+  // ---- prologue: everything the tile needs first is requested at once -----------------------
+  // The chunks from dstart on (same-block / causal rules) come FIRST: their addresses need no
+  // routing table, so their loads, the Q loads above and the reads of the block list are all in
+  // flight together.  The chunks of the prior attention blocks follow.
+  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;  // >= 1
+  gload(dstart);
+  if (tid == 0) lds_count = 0;
   __syncthreads();
+  {
+    // attention blocks that end at or before dstart: ids into LDS, count.  The list is sorted and
+    // holds distinct block ids, so entry j >= j: only the first dstart/Bs entries can qualify.
+    const int jmax = min(dstart / Bs, p.TN);
+    int cnt = 0;
+    for (int j = tid; j < jmax; j += NTHREADS) {
+      const int e = list[j * list_stride];
+      if (j < n_attn && (e + 1) * Bs <= dstart) {
+        ++cnt;
+        if (j < MAX_LDS_LIST) lds_list[j] = e;
+      }
+    }
+    if (cnt) atomicAdd(&lds_count, cnt);
+  }
+  // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
+  unsigned long long diag_attn;
+  {
+    const int blk = dstart / Bs + lane;
+    const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
+    diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
+  }
+  lstore(0);
+  __syncthreads();
+  const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
+  const int n_iters = n_diag + n_prior_chunks;
+
+  // Chunk iterator, all wave-uniform (scalar registers): the chunks from dstart on, then the
+  // 64-key chunks of the prior attention blocks in list order.
+  int nx_it = 1, nx_j = 0, nx_sub = 0;  // chunk 0 is already staged
+  auto next_key_start = [&]() -> int {
+    int ks;
+    if (nx_it < n_diag) {
+      ks = dstart + nx_it * 64;
+    } else {
+      int e;
+      if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+      else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
+      ks = e * Bs + nx_sub * 64;
+      if (++nx_sub == per_blk) {
+        nx_sub = 0;
+        ++nx_j;
+      }
+    }
+    ++nx_it;
+    return ks;
+  };
+  int ks_fetch = 0;  // key start of the chunk the next gload brings in (known one iteration ahead)
+  if (n_iters > 1) ks_fetch = next_key_start();
 
   const float c = p.scale_log2;
   f32x16 s[2][NQ];
   float mx[NQ];
+  // ---- phase B (runs first): the chunks from dstart to the end of the tile, with the same-block and causal rules
+  const int my_blk = q0 / Bs;
+  int it = 0;
+  for (; it < n_diag; ++it) {
+    const int buf = it & 1;
+    if (it + 1 < n_iters) gload(ks_fetch);
+    const int jc = (dstart >> 6) + it;  // absolute chunk index of the keys
+    const int kblk = (jc * 64) / Bs;
+    bool active = wave_valid, causal = false;
+    if (p.same_block) {
+      if (jc > my_chunk) active = false;
+      else if (jc == my_chunk) causal = true;
+      else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dstart / Bs)) & 1ull));
+    } else {
+      active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dstart / Bs)) & 1ull);
+    }
+    if (active && !NATSL_ABL(p.dbg & 8)) {
+      if (causal) scores<DK, NQ, true>(Ks + buf * 64 * KP, QB, s, mx, c, lane, qloc0);
+      else scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
+      if (needs_rescale<NQ>(mx, m_ref)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
+      exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
+    }
+    if (it + 1 < n_iters) lstore(buf ^ 1);
+    if (it + 2 < n_iters) ks_fetch = next_key_start();
+    __syncthreads();
+  }
+
   // ---- phase A: whole attention blocks before the tile; every wave, no masks.  The inner loop is
   // the fast path; an iteration whose maxima outgrow the reference leaves it, rescales, finishes
   // and re-enters.
-  int it = 0;
-  while (it < n_prior_chunks) {
+  if constexpr (NQ == 1) {
+    // Software-pipelined in halves of 32 keys, so that each wave feeds the matrix pipe and the vector
+    // ALU at the same time:  QK(0) | QK(1) with exp(0) | PV(0) with exp(1) | PV(1).
+    // A half whose maximum outgrows the reference leaves the fast loop (pending = 1 or 2), the
+    // iteration is finished on the slow path below and the loop is re-entered.
+    constexpr int KSTEPS_ = DK / 16;
+    while (it < n_iters) {
+      int pending = 0;
+      bf16x8 PB0[2], PB1[2];
+      float rs = 0.f;
+      for (; it < n_iters; ++it) {
+        const int buf = it & 1;
+        const bool more = it + 1 < n_iters;
+        const bf16_t* Kb = Ks + buf * 64 * KP;
+        const bf16_t* VTb = Vs + buf * DV * TP;
+        if (more && !NATSL_ABL(p.dbg & 1)) gload(ks_fetch);
+        if (wave_valid && !NATSL_ABL(p.dbg & 2)) {
+          qk_half<DK>(Kb, 0, QB[0], s[0][0], lane);
+          mx[0] = half_max<false>(s[0][0], 0, c, lane, 0);
+          if (__any(mx[0] > m_ref[0] + RESCALE_SLACK)) {
+            pending = 1;
+            break;
+          }
+          const float neg = m_ref[0] == -INFINITY ? 0.f : -m_ref[0];
+          rs = 0.f;
+          // QK(1) with exp(0)
+          qk_half<DK>(Kb, 1, QB[0], s[1][0], lane);
+          probs_half(s[0][0], c, neg, rs, PB0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+          for (int st = 0; st < KSTEPS_; ++st) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (st + 2 < KSTEPS_) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+          }
+          mx[0] = half_max<false>(s[1][0], 1, c, lane, 0);
+          if (__any(mx[0] > m_ref[0] + RESCALE_SLACK)) {
+            pending = 2;
+            break;
+          }
+          // PV(0) with exp(1)
+          pv_half<DV>(VTb, 0, PB0, acc, lane);
+          probs_half(s[1][0], c, neg, rs, PB1);
+#pragma unroll
+          for (int i = 0; i < 2 * VT; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+          }
+          pv_half<DV>(VTb, 1, PB1, acc, lane);
+          l_run[0] += rs;
+        }
+        if (more && !NATSL_ABL(p.dbg & 1) && !NATSL_ABL(p.dbg & 32)) lstore(buf ^ 1);
+        if (it + 2 < n_iters) ks_fetch = next_key_start();
+        __syncthreads();
+      }
+      if (pending) {
+        const int buf = it & 1;
+        const bf16_t* Kb = Ks + buf * 64 * KP;
+        const bf16_t* VTb = Vs + buf * DV * TP;
+        if (pending == 1) {
+          rescale<DV, NQ>(acc, m_ref, l_run, mx);
+          rs = 0.f;
+          qk_half<DK>(Kb, 1, QB[0], s[1][0], lane);
+          probs_half(s[0][0], c, -m_ref[0], rs, PB0);
+          mx[0] = half_max<false>(s[1][0], 1, c, lane, 0);
+        }
+        // here: exp(0) is done against the current reference and mx holds the maximum of half 1
+        pv_half<DV>(VTb, 0, PB0, acc, lane);
+        l_run[0] += rs;
+        rs = 0.f;
+        if (__any(mx[0] > m_ref[0] + RESCALE_SLACK)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
+        probs_half(s[1][0], c, m_ref[0] == -INFINITY ? 0.f : -m_ref[0], rs, PB1);
+        pv_half<DV>(VTb, 1, PB1, acc, lane);
+        l_run[0] += rs;
+        if (it + 1 < n_iters) lstore(buf ^ 1);
+        if (it + 2 < n_iters) ks_fetch = next_key_start();
+        __syncthreads();
+        ++it;
+      }
+    }
+  } else {
+  while (it < n_iters) {
     bool pending = false;
-    for (; it < n_prior_chunks; ++it) {
+    for (; it < n_iters; ++it) {
       const int buf = it & 1;
       const bool more = it + 1 < n_iters;
       if (more && !NATSL_ABL(p.dbg & 1)) gload(ks_fetch);
@@ -414,7 +599,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
         }
         exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
       }
-      if (more && !NATSL_ABL(p.dbg & 1) && !NATSL_ABL(p.dbg & 32)) lstore(buf ^ 1);
+      if (more && !NATSL_ABL(p.dbg & 1)) lstore(buf ^ 1);
       if (it + 2 < n_iters) ks_fetch = next_key_start();
       __syncthreads();
     }
@@ -428,32 +613,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
       ++it;
     }
   }
-  // ---- phase B: the chunks from dstart to the end of the tile
-  const int my_blk = q0 / Bs;
-  for (; it < n_iters; ++it) {
-    const int buf = it & 1;
-    if (it + 1 < n_iters) gload(ks_fetch);
-    const int jc = (dstart >> 6) + it - n_prior_chunks;  // absolute chunk index of the keys
-    const int kblk = (jc * 64) / Bs;
-    bool active = wave_valid, causal = false;
-    if (p.same_block) {
-      if (jc > my_chunk) active = false;
-      else if (jc == my_chunk) causal = true;
-      else active = active && (kblk == my_blk || attn_block(kblk));
-    } else {
-      active = active && jc < my_chunk && kblk < my_blk && attn_block(kblk);
-    }
-    if (active && !NATSL_ABL(p.dbg & 8)) {
-      if (causal) scores<DK, NQ, true>(Ks + buf * 64 * KP, QB, s, mx, c, lane, qloc0);
-      else scores<DK, NQ, false>(Ks + buf * 64 * KP, QB, s, mx, c, lane, 0);
-      if (needs_rescale<NQ>(mx, m_ref)) rescale<DV, NQ>(acc, m_ref, l_run, mx);
-      exp_pv<DV, NQ>(Vs + buf * DV * TP, s, acc, m_ref, l_run, c, lane);
-    }
-    if (it + 1 < n_iters) lstore(buf ^ 1);
-    if (it + 2 < n_iters) ks_fetch = next_key_start();
-    __syncthreads();
   }
-
   // ---- epilogue: normalise, transpose through LDS, coalesced stores ------------------------
   bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + wave * QW * VP;  // this wave's [QW][VP]
 #pragma unroll
