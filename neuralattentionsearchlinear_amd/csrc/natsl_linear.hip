@@ -161,8 +161,15 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
   float* Sout = p.ws_sc + unit * (4 * C);
 
   // ---- Gram products on the matrix cores: wave w owns the 32x32 tile (w/2, w%2) ------------
+  // P and TmB are stored in the order the scan kernel consumes them as MFMA A operands, so that its
+  // loads are contiguous: the 16 bytes of scan-lane (row i%16, group g4) of 16-row band i/16 and
+  // k-step s sit at ((2(i/16) + s) * 64 + 16 g4 + i%16) * 16 bytes.  Within a k-step the 32
+  // contraction tokens are permuted: slot (g4, e) holds token 8(2(g4&1) + e/4) + 4(g4/2) + e%4,
+  // which is how one lane of the transposed 32x32 Gram accumulator holds them.
   {
     const int ti = wave >> 1, tj = wave & 1, l32 = lane & 31, hf = lane >> 5;
+    const int i = 32 * ti + l32;  // P row owned by this lane
+    bf16_t* prow = Pout + ((size_t)((2 * (i >> 4) + tj) * 64 + (i & 15))) * 8;
     if (ti >= tj) {
       f32x16 gk, gq;
 #pragma unroll
@@ -171,29 +178,45 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
       for (int s = 0; s < DK / 16; ++s) {
         const bf16x8 kb = ld8(Ks + (32 * tj + l32) * KP + 16 * s + 8 * hf);
         const bf16x8 qa = ld8(Qs + (32 * ti + l32) * KP + 16 * s + 8 * hf);
-        gq = mfma32(qa, kb, gq);
+        gq = mfma32(kb, qa, gq);  // transposed: lane = query row i, registers = key tokens j
         if (DELTA) {
           const bf16x8 ka = ld8(Ks + (32 * ti + l32) * KP + 16 * s + 8 * hf);
-          gk = mfma32(ka, kb, gk);
+          gk = mfma32(ka, kb, gk);  // lane = column j, registers = rows i
         }
       }
-      const int j = 32 * tj + l32;
-      const float gj = gam[j], rkj = rk[j];
+      {
+        const float gi = gam[i], fi = p.scale * rq[i];
+        u32x4 w[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 32 * ti + 8 * (r >> 2) + 4 * hf + (r & 3);
-        const float dec = i >= j ? __expf(gam[i] - gj) : 0.f;
-        Pout[i * C + j] = f32_to_bf16(p.scale * rq[i] * rkj * gq[r] * dec);
-        if (DELTA) Am[i * AP + j] = i > j ? bet[i] * rk[i] * rkj * gk[r] * dec : 0.f;
+        for (int r = 0; r < 16; r += 2) {
+          const int j0 = 32 * tj + 8 * (r >> 2) + 4 * hf + (r & 3);
+          const float p0 = i >= j0 ? fi * rk[j0] * gq[r] * __expf(gi - gam[j0]) : 0.f;
+          const float p1 = i >= j0 + 1 ? fi * rk[j0 + 1] * gq[r + 1] * __expf(gi - gam[j0 + 1]) : 0.f;
+          w[r >> 3][(r >> 1) & 3] = pack_bf16x2(p0, p1);
+        }
+        *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = w[0];
+        *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = w[1];
+      }
+      if (DELTA) {
+        const int j = 32 * tj + l32;
+        const float gj = gam[j], rkj = rk[j];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int ii = 32 * ti + 8 * (r >> 2) + 4 * hf + (r & 3);
+          Am[ii * AP + j] = ii > j ? bet[ii] * rk[ii] * rkj * gk[r] * __expf(gam[ii] - gj) : 0.f;
+        }
       }
     } else {
       // the strictly upper 32x32 tile is zero
-      const int l32 = lane & 31, hf = lane >> 5;
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = z;
+      *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = z;
+      if (DELTA) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 8 * (r >> 2) + 4 * hf + (r & 3), j = 32 + l32;
-        Pout[i * C + j] = 0;
-        if (DELTA) Am[i * AP + j] = 0.f;
+        for (int r = 0; r < 16; ++r) {
+          const int ii = 8 * (r >> 2) + 4 * hf + (r & 3), j = 32 + l32;
+          Am[ii * AP + j] = 0.f;
+        }
       }
     }
   }
@@ -274,20 +297,18 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
       __syncthreads();
     }
   }
-  // TmB = Tm * diag(beta), bf16, rows of 16 contiguous elements per thread
+  // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above)
   if (!NATSL_ABL(p.dbg & 128)) {
     const int row = tid >> 2, cb = tid & 3;
-    u32x4 w[2];
+    float x[16];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = 16 * cb + 2 * e;
-      const float x0 = cb <= (row >> 4) ? Xm[row * AP + j] * bet[j] : 0.f;
-      const float x1 = cb <= (row >> 4) ? Xm[row * AP + j + 1] * bet[j + 1] : 0.f;
-      w[e >> 2][e & 3] = pack_bf16x2(x0, x1);
-    }
-    u32x4* dst = reinterpret_cast<u32x4*>(Tout + row * C + 16 * cb);
-    dst[0] = w[0];
-    dst[1] = w[1];
+    for (int e = 0; e < 16; ++e) x[e] = cb <= (row >> 4) ? Xm[row * AP + 16 * cb + e] * bet[16 * cb + e] : 0.f;
+    u32x4 w0, w1;  // tokens {0..3, 8..11} and {4..7, 12..15} of this thread's 16
+    w0[0] = pack_bf16x2(x[0], x[1]);  w0[1] = pack_bf16x2(x[2], x[3]);   w0[2] = pack_bf16x2(x[8], x[9]);   w0[3] = pack_bf16x2(x[10], x[11]);
+    w1[0] = pack_bf16x2(x[4], x[5]);  w1[1] = pack_bf16x2(x[6], x[7]);   w1[2] = pack_bf16x2(x[12], x[13]); w1[3] = pack_bf16x2(x[14], x[15]);
+    bf16_t* trow = Tout + ((size_t)((2 * (row >> 4) + (cb >> 1)) * 64 + (row & 15))) * 8;
+    *reinterpret_cast<u32x4*>(trow + (cb & 1) * 128) = w0;
+    *reinterpret_cast<u32x4*>(trow + (2 + (cb & 1)) * 128) = w1;
   }
 }
 
@@ -369,54 +390,53 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
   // Two register sets, used alternately by the two halves of the (unrolled-by-2) chunk loop: while
   // one set feeds the matrix cores the other receives the next chunk's loads.
   struct Operands {
-    bf16x8 kA[KS], qA[KS], TA[2], PA[2];
+    bf16x8 qA[KS], TA[2], PA[2];
     f32x4 se, sq, sk;
     float dec, glast, linf;
-    u32x4 vld;
+    u32x4 kld[KS], vld;  // row-contiguous k and v pieces on their way to LDS
   };
   const int a_row = 16 * wave + i16;          // this lane's A-operand row (token within the chunk)
   const int v_ld_row = tid >> 2, v_ld_seg = tid & 3;
+  const int k_ld_row = tid >> 4, k_ld_seg = tid & 15;  // k staging: 16 lanes cover one 256-byte row (DK = 128)
   const int r0 = 16 * wave + 4 * g4;          // first of this lane's four accumulator rows
+  // where those four tokens sit in the contraction order P and TmB were stored in
+  const int perm0 = 32 * (wave >> 1) + 8 * (2 * (g4 & 1) + (wave & 1)) + 4 * (g4 >> 1);
   // running pointers, advanced by one chunk per load; rows past the end of the sequence are clamped
   // (beta = 0 there makes their v_new exactly 0, and their outputs are never stored)
-  const bf16_t* k_ptr = kp + 8 * g4;
+  const bf16_t* k_ptr = kp + 8 * k_ld_seg;
   const bf16_t* q_ptr = qp + 8 * g4;
   const bf16_t* v_ptr = vp + 8 * v_ld_seg;
   const size_t unit0 = (size_t)chunk_off * p.H + h;
-  const bf16_t* P_ptr = p.ws_p + unit0 * (C * C) + a_row * C + 8 * g4;
-  const bf16_t* T_ptr = p.ws_tm + unit0 * (C * C) + a_row * C + 8 * g4;
+  // P and TmB come in A-operand order: 16 contiguous bytes per lane, 1 KiB per wave and k-step
+  const bf16_t* P_ptr = p.ws_p + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
+  const bf16_t* T_ptr = p.ws_tm + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
   const float* sc_ptr = p.ws_sc + unit0 * (4 * C);
   const size_t unit_step = (size_t)p.H * (C * C), sc_step = (size_t)p.H * (4 * C);
   int next_c = 0;
+  constexpr int KROWS = 256 / (DK / 8);  // token rows one pass of the k staging covers (16 for DK=128, 32 for DK=64)
   auto gload = [&](Operands& A) {
-    if (NATSL_ABL(p.dbg & 16)) {
-      // timing experiment: the same bytes with row-contiguous (fully coalesced) lane addressing
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int tok = min(next_c * C + 16 * wave + 4 * s + g4, len - 1);
-        A.kA[s] = ld8(kp + (size_t)tok * qk_row + 8 * i16);
-        A.qA[s] = ld8(qp + (size_t)tok * qk_row + 8 * i16);
-      }
-      const bf16_t* Pb = P_ptr - (a_row * C + 8 * g4), *Tb = T_ptr - (a_row * C + 8 * g4);
-      A.PA[0] = ld8(Pb + (16 * wave + (lane >> 3)) * C + 8 * (lane & 7));
-      A.PA[1] = ld8(Pb + (16 * wave + 8 + (lane >> 3)) * C + 8 * (lane & 7));
-      A.TA[0] = ld8(Tb + (16 * wave + (lane >> 3)) * C + 8 * (lane & 7));
-      A.TA[1] = ld8(Tb + (16 * wave + 8 + (lane >> 3)) * C + 8 * (lane & 7));
-    } else {
     const int tok = min(next_c * C + a_row, len - 1);
-    const bf16_t* kr = k_ptr + (size_t)tok * qk_row;
     const bf16_t* qr = q_ptr + (size_t)tok * qk_row;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      A.kA[s] = ld8(kr + 32 * s);
-      A.qA[s] = ld8(qr + 32 * s);
+    for (int s = 0; s < KS; ++s) A.qA[s] = ld8(qr + 32 * s);
+    if (DK == 128) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int kt = min(next_c * C + k_ld_row + KROWS * s, len - 1);
+        A.kld[s] = *reinterpret_cast<const u32x4*>(k_ptr + (size_t)kt * qk_row);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int kt = min(next_c * C + (tid >> 3) + KROWS * s, len - 1);
+        A.kld[s] = *reinterpret_cast<const u32x4*>(kp + 8 * (tid & 7) + (size_t)kt * qk_row);
+      }
     }
     A.PA[0] = ld8(P_ptr);
-    A.PA[1] = ld8(P_ptr + 32);
+    A.PA[1] = ld8(P_ptr + 512);
     if (DELTA) {
       A.TA[0] = ld8(T_ptr);
-      A.TA[1] = ld8(T_ptr + 32);
-    }
+      A.TA[1] = ld8(T_ptr + 512);
     }
     A.se = *reinterpret_cast<const f32x4*>(sc_ptr + r0);
     A.sq = *reinterpret_cast<const f32x4*>(sc_ptr + C + r0);
@@ -433,8 +453,13 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     ++next_c;
   };
   auto lstore = [&](const Operands& A, int buf) {
+    if (DK == 128) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]) = A.kA[s];
+      for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][(k_ld_row + KROWS * s) * KP + 8 * k_ld_seg]) = A.kld[s];
+    } else {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][((tid >> 3) + KROWS * s) * KP + 8 * (tid & 7)]) = A.kld[s];
+    }
     *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = A.vld;
   };
 
@@ -463,8 +488,9 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       const bf16x8 sb0 = ld8(ST + i16 * KP + 32 * s + 8 * g4);
       const bf16x8 sb1 = ld8(ST + (16 + i16) * KP + 32 * s + 8 * g4);
       if (DELTA) {
-        R[0] = mfma16(CUR.kA[s], sb0, R[0]);
-        R[1] = mfma16(CUR.kA[s], sb1, R[1]);
+        const bf16x8 ka = ld8(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]);
+        R[0] = mfma16(ka, sb0, R[0]);
+        R[1] = mfma16(ka, sb1, R[1]);
       }
       O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
       O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
@@ -483,7 +509,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
         f32x4 X;
 #pragma unroll
         for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - CUR.se[r] * R[nn][r];
-        *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(X);
+        *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + perm0) = pack4(X);
       }
       __syncthreads();
       // (3) v_new = TmB X
@@ -500,7 +526,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       f32x4 vt;
 #pragma unroll
       for (int r = 0; r < 4; ++r) vt[r] = VN[nn][r] * CUR.sk[r];
-      *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(VN[nn]);
+      *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + perm0) = pack4(VN[nn]);
       *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
     }
     __syncthreads();
