@@ -387,89 +387,98 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
   };
 
   // ---- operand staging ------------------------------------------------------------------------
-  // Two register sets, used alternately by the two halves of the (unrolled-by-2) chunk loop: while
-  // one set feeds the matrix cores the other receives the next chunk's loads.
+  // Two register sets hold the MFMA A operands (q, TmB, P) and the per-token scales of chunks c and
+  // c+1.  Each piece of the set in use is reloaded with chunk c+2's data right after its last use,
+  // so every one of these loads has two steps to arrive.  k and v go through LDS (double-buffered):
+  // they are loaded at the start of step c for chunk c+1 and stored at its end.
   struct Operands {
     bf16x8 qA[KS], TA[2], PA[2];
     f32x4 se, sq, sk;
     float dec, glast, linf;
+  };
+  struct Staging {
     u32x4 kld[KS], vld;  // row-contiguous k and v pieces on their way to LDS
   };
   const int a_row = 16 * wave + i16;          // this lane's A-operand row (token within the chunk)
   const int v_ld_row = tid >> 2, v_ld_seg = tid & 3;
-  const int k_ld_row = tid >> 4, k_ld_seg = tid & 15;  // k staging: 16 lanes cover one 256-byte row (DK = 128)
   const int r0 = 16 * wave + 4 * g4;          // first of this lane's four accumulator rows
   // where those four tokens sit in the contraction order P and TmB were stored in
   const int perm0 = 32 * (wave >> 1) + 8 * (2 * (g4 & 1) + (wave & 1)) + 4 * (g4 >> 1);
-  // running pointers, advanced by one chunk per load; rows past the end of the sequence are clamped
-  // (beta = 0 there makes their v_new exactly 0, and their outputs are never stored)
+  // k staging: one pass of the 256 threads covers KROWS token rows of DK*2 bytes
+  constexpr int KSEGS = DK / 8, KROWS = 256 / KSEGS;
+  const int k_ld_row = tid / KSEGS, k_ld_seg = tid % KSEGS;
+  // rows past the end of the sequence are clamped (beta = 0 there makes their v_new exactly 0, and
+  // their outputs are never stored)
   const bf16_t* k_ptr = kp + 8 * k_ld_seg;
   const bf16_t* q_ptr = qp + 8 * g4;
   const bf16_t* v_ptr = vp + 8 * v_ld_seg;
   const size_t unit0 = (size_t)chunk_off * p.H + h;
-  // P and TmB come in A-operand order: 16 contiguous bytes per lane, 1 KiB per wave and k-step
-  const bf16_t* P_ptr = p.ws_p + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
-  const bf16_t* T_ptr = p.ws_tm + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
-  const float* sc_ptr = p.ws_sc + unit0 * (4 * C);
   const size_t unit_step = (size_t)p.H * (C * C), sc_step = (size_t)p.H * (4 * C);
-  int next_c = 0;
-  constexpr int KROWS = 256 / (DK / 8);  // token rows one pass of the k staging covers (16 for DK=128, 32 for DK=64)
-  auto gload = [&](Operands& A) {
-    const int tok = min(next_c * C + a_row, len - 1);
-    const bf16_t* qr = q_ptr + (size_t)tok * qk_row;
+  // P and TmB come in A-operand order: 16 contiguous bytes per lane, 1 KiB per wave and k-step
+  const bf16_t* P_base = p.ws_p + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
+  const bf16_t* T_base = p.ws_tm + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
+  const float* sc_base = p.ws_sc + unit0 * (4 * C);
+  // the pieces of an operand set, each loadable on its own (cc = chunk index, must be < NT)
+  auto load_q = [&](Operands& A, int cc) {
+    const bf16_t* qr = q_ptr + (size_t)min(cc * C + a_row, len - 1) * qk_row;
 #pragma unroll
     for (int s = 0; s < KS; ++s) A.qA[s] = ld8(qr + 32 * s);
-    if (DK == 128) {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int kt = min(next_c * C + k_ld_row + KROWS * s, len - 1);
-        A.kld[s] = *reinterpret_cast<const u32x4*>(k_ptr + (size_t)kt * qk_row);
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int kt = min(next_c * C + (tid >> 3) + KROWS * s, len - 1);
-        A.kld[s] = *reinterpret_cast<const u32x4*>(kp + 8 * (tid & 7) + (size_t)kt * qk_row);
-      }
-    }
-    A.PA[0] = ld8(P_ptr);
-    A.PA[1] = ld8(P_ptr + 512);
-    if (DELTA) {
-      A.TA[0] = ld8(T_ptr);
-      A.TA[1] = ld8(T_ptr + 512);
-    }
-    A.se = *reinterpret_cast<const f32x4*>(sc_ptr + r0);
-    A.sq = *reinterpret_cast<const f32x4*>(sc_ptr + C + r0);
-    A.sk = *reinterpret_cast<const f32x4*>(sc_ptr + 2 * C + r0);
-    A.dec = sc_ptr[3 * C];
-    A.glast = sc_ptr[3 * C + 1];
-    A.linf = sc_ptr[3 * C + 2];
-    const int vt = next_c * C + v_ld_row;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    A.vld = vt < len ? *reinterpret_cast<const u32x4*>(v_ptr + (size_t)vt * v_row) : z;  // v must be 0 past the end
-    P_ptr += unit_step;
-    T_ptr += unit_step;
-    sc_ptr += sc_step;
-    ++next_c;
   };
-  auto lstore = [&](const Operands& A, int buf) {
-    if (DK == 128) {
+  auto load_T = [&](Operands& A, int cc) {
+    A.TA[0] = ld8(T_base + cc * unit_step);
+    A.TA[1] = ld8(T_base + cc * unit_step + 512);
+  };
+  auto load_P = [&](Operands& A, int cc) {
+    A.PA[0] = ld8(P_base + cc * unit_step);
+    A.PA[1] = ld8(P_base + cc * unit_step + 512);
+  };
+  auto load_se = [&](Operands& A, int cc) { A.se = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + r0); };
+  auto load_sq = [&](Operands& A, int cc) { A.sq = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + C + r0); };
+  auto load_sk = [&](Operands& A, int cc) { A.sk = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + 2 * C + r0); };
+  auto load_scalars = [&](Operands& A, int cc) {
+    const float* sp = sc_base + cc * sc_step + 3 * C;
+    A.dec = sp[0];
+    A.glast = sp[1];
+    A.linf = sp[2];
+  };
+  auto load_all = [&](Operands& A, int cc) {
+    load_q(A, cc);
+    if (DELTA) load_se(A, cc);
+    if (DELTA) load_T(A, cc);
+    load_sk(A, cc);
+    load_P(A, cc);
+    load_sq(A, cc);
+    load_scalars(A, cc);
+  };
+  auto gload_kv = [&](Staging& G, int cc) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][(k_ld_row + KROWS * s) * KP + 8 * k_ld_seg]) = A.kld[s];
-    } else {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][((tid >> 3) + KROWS * s) * KP + 8 * (tid & 7)]) = A.kld[s];
+    for (int s = 0; s < KS; ++s) {
+      const int kt = min(cc * C + k_ld_row + KROWS * s, len - 1);
+      G.kld[s] = *reinterpret_cast<const u32x4*>(k_ptr + (size_t)kt * qk_row);
     }
-    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = A.vld;
+    const int vt = cc * C + v_ld_row;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    G.vld = vt < len ? *reinterpret_cast<const u32x4*>(v_ptr + (size_t)vt * v_row) : z;  // v must be 0 past the end
+  };
+  auto lstore = [&](const Staging& G, int buf) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][(k_ld_row + KROWS * s) * KP + 8 * k_ld_seg]) = G.kld[s];
+    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = G.vld;
   };
 
   float gsum = 0.f;
-  // one chunk: CUR holds its operands (already staged in kbuf/vbuf[buf]); NXT receives the next chunk's
-  auto step = [&](const int c, const int buf, const Operands& CUR, Operands& NXT) {
+  // one chunk: CUR holds its operands, kbuf/vbuf[buf] its k and v tiles
+  Staging G;
+  auto step = [&](const int c, const int buf, Operands& CUR) {
     __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
-    const bool more = c + 1 < NT;
-    if (more) gload(NXT);
-    if (NATSL_ABL(p.dbg & 4)) { __syncthreads(); __syncthreads(); if (more) lstore(NXT, buf ^ 1); return; }
+    const bool more = c + 1 < NT, more2 = c + 2 < NT;
+    if (more) gload_kv(G, c + 1);
+    if (NATSL_ABL(p.dbg & 4)) {
+      if (more2) load_all(CUR, c + 2);
+      __syncthreads(); __syncthreads();
+      if (more) lstore(G, buf ^ 1);
+      return;
+    }
 
     if (c % per_blk == 0) {
 #pragma unroll
@@ -495,6 +504,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
       O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
     }
+    if (more2) load_q(CUR, c + 2);
     // (2) v in accumulator layout via the transposing read; X = v - se * R
     f32x4 VN[2];
 #pragma unroll
@@ -511,6 +521,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
         for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - CUR.se[r] * R[nn][r];
         *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + perm0) = pack4(X);
       }
+      if (more2) load_se(CUR, c + 2);
       __syncthreads();
       // (3) v_new = TmB X
 #pragma unroll
@@ -519,6 +530,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
         for (int s = 0; s < 2; ++s) VN[nn] = mfma16(CUR.TA[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
       }
+      if (more2) load_T(CUR, c + 2);
     }
     // (4) v_new and sk * v_new, transposed, for the two products that reduce over tokens
 #pragma unroll
@@ -529,6 +541,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + perm0) = pack4(VN[nn]);
       *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
     }
+    if (more2) load_sk(CUR, c + 2);
     __syncthreads();
     // (5) o = sq * O1 + P v_new
 #pragma unroll
@@ -543,6 +556,10 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
       for (int r = 0; r < 4; ++r) Os[(r0 + r) * VP + 16 * nn + i16] = f32_to_bf16(O[r]);
     }
+    if (more2) {
+      load_P(CUR, c + 2);
+      load_sq(CUR, c + 2);
+    }
     {
       // each wave stores the 16 rows it owns: 4 lanes x 16 bytes per row
       __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -554,7 +571,10 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     // (6) state update / roll-back
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
     gsum += CUR.glast;
-    if (CUR.linf != 0.f || !last_of_block) {
+    const float dec_c = CUR.dec;
+    const bool keep = CUR.linf != 0.f || !last_of_block;
+    if (more2) load_scalars(CUR, c + 2);
+    if (keep) {
 #pragma unroll
       for (int mi = 0; mi < MT; ++mi) {
         const int m = wave * MT + mi;
@@ -567,7 +587,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
         for (int nn = 0; nn < 2; ++nn) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= CUR.dec;
+          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= dec_c;
 #pragma unroll
           for (int s = 0; s < 2; ++s) S[mi][nn] = mfma16(kt[s], ld8(VTT + (16 * nn + i16) * XP + 32 * s + 8 * g4), S[mi][nn]);
         }
@@ -583,18 +603,20 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     }
     // (7) bf16 copy of the state and the staged k, v tiles for the next step
     write_ST();
-    if (more) lstore(NXT, buf ^ 1);
+    if (more) lstore(G, buf ^ 1);
   };
 
   Operands A0, A1;
   if (NT > 0) {
-    gload(A0);
-    lstore(A0, 0);
+    gload_kv(G, 0);
+    load_all(A0, 0);
+    if (NT > 1) load_all(A1, 1);
+    lstore(G, 0);
   }
   write_ST();
   for (int c = 0; c < NT; c += 2) {
-    step(c, 0, A0, A1);
-    if (c + 1 < NT) step(c + 1, 1, A1, A0);
+    step(c, 0, A0);
+    if (c + 1 < NT) step(c + 1, 1, A1);
   }
 
   if (p.hs) {
