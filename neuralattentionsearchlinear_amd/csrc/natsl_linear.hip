@@ -64,6 +64,13 @@ struct LinearParams {
 constexpr int C = 64;
 constexpr int BV = 32;
 
+// Development build only: per-phase cycle counters of the scan's step, written over the first floats of ht.
+#ifdef NATSL_PHASE_TIMING
+#define NATSL_TICK(i) { const long long now_ = __builtin_readcyclecounter(); tacc[i] += now_ - tlast; tlast = now_; }
+#else
+#define NATSL_TICK(i)
+#endif
+
 NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
   float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i]
                                : bf16_to_f32(reinterpret_cast<const bf16_t*>(types)[i]);
@@ -467,16 +474,25 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
   };
 
   float gsum = 0.f;
+#ifdef NATSL_PHASE_TIMING
+  long long tacc[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_readcyclecounter();
+#endif
   // one chunk: CUR holds its operands, kbuf/vbuf[buf] its k and v tiles
   Staging G;
   auto step = [&](const int c, const int buf, Operands& CUR) {
+    NATSL_TICK(9)
     __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
-    const bool more = c + 1 < NT, more2 = c + 2 < NT;
-    if (more) gload_kv(G, c + 1);
+    NATSL_TICK(0)
+    // Loads are issued unconditionally (chunk indices clamped to the last chunk): a load inside a
+    // branch would force the waits below to assume it may not have been issued, i.e. to drain the queue.
+    const int c1 = min(c + 1, NT - 1), c2 = min(c + 2, NT - 1);
+    const float dec_c = CUR.dec, glast_c = CUR.glast, linf_c = CUR.linf;
+    load_scalars(CUR, c2);  // first, so that nothing younger has to be waited for along with them
+    gload_kv(G, c1);
     if (NATSL_ABL(p.dbg & 4)) {
-      if (more2) load_all(CUR, c + 2);
+      load_q(CUR, c2); load_se(CUR, c2); load_T(CUR, c2); load_sk(CUR, c2); load_P(CUR, c2); load_sq(CUR, c2);
       __syncthreads(); __syncthreads();
-      if (more) lstore(G, buf ^ 1);
+      lstore(G, buf ^ 1);
       return;
     }
 
@@ -504,7 +520,8 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
       O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
     }
-    if (more2) load_q(CUR, c + 2);
+    NATSL_TICK(1)
+    load_q(CUR, c2);
     // (2) v in accumulator layout via the transposing read; X = v - se * R
     f32x4 VN[2];
 #pragma unroll
@@ -521,8 +538,10 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
         for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - CUR.se[r] * R[nn][r];
         *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + perm0) = pack4(X);
       }
-      if (more2) load_se(CUR, c + 2);
+      load_se(CUR, c2);
+      NATSL_TICK(2)
       __syncthreads();
+      NATSL_TICK(3)
       // (3) v_new = TmB X
 #pragma unroll
       for (int nn = 0; nn < 2; ++nn) {
@@ -530,7 +549,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
         for (int s = 0; s < 2; ++s) VN[nn] = mfma16(CUR.TA[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
       }
-      if (more2) load_T(CUR, c + 2);
+      load_T(CUR, c2);
     }
     // (4) v_new and sk * v_new, transposed, for the two products that reduce over tokens
 #pragma unroll
@@ -541,8 +560,10 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + perm0) = pack4(VN[nn]);
       *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
     }
-    if (more2) load_sk(CUR, c + 2);
+    load_sk(CUR, c2);
+    NATSL_TICK(4)
     __syncthreads();
+    NATSL_TICK(5)
     // (5) o = sq * O1 + P v_new
 #pragma unroll
     for (int nn = 0; nn < 2; ++nn) {
@@ -556,10 +577,8 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
       for (int r = 0; r < 4; ++r) Os[(r0 + r) * VP + 16 * nn + i16] = f32_to_bf16(O[r]);
     }
-    if (more2) {
-      load_P(CUR, c + 2);
-      load_sq(CUR, c + 2);
-    }
+    load_P(CUR, c2);
+    load_sq(CUR, c2);
     {
       // each wave stores the 16 rows it owns: 4 lanes x 16 bytes per row
       __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -568,12 +587,11 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       if (tok < len)
         *reinterpret_cast<u32x4*>(op + (size_t)tok * v_row + 8 * (lane & 3)) = *reinterpret_cast<const u32x4*>(Os + row * VP + 8 * (lane & 3));
     }
+    NATSL_TICK(6)
     // (6) state update / roll-back
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
-    gsum += CUR.glast;
-    const float dec_c = CUR.dec;
-    const bool keep = CUR.linf != 0.f || !last_of_block;
-    if (more2) load_scalars(CUR, c + 2);
+    gsum += glast_c;
+    const bool keep = linf_c != 0.f || !last_of_block;
     if (keep) {
 #pragma unroll
       for (int mi = 0; mi < MT; ++mi) {
@@ -601,9 +619,11 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
           for (int r = 0; r < 4; ++r) S[mi][nn][r] = Ssave[mi][nn][r] * f;
     }
+    NATSL_TICK(7)
     // (7) bf16 copy of the state and the staged k, v tiles for the next step
     write_ST();
-    if (more) lstore(G, buf ^ 1);
+    lstore(G, buf ^ 1);
+    NATSL_TICK(8)
   };
 
   Operands A0, A1;
@@ -643,6 +663,12 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
           p.ht[((size_t)chain * DK + kd) * p.V + vc] = S[mi][nn][r];
         }
   }
+#ifdef NATSL_PHASE_TIMING
+  if (p.ht && blockIdx.x == 17 && (tid & 63) == 0) {
+    __syncthreads();
+    for (int i = 0; i < 10; ++i) p.ht[10 * wave + i] = (float)tacc[i] / NT;
+  }
+#endif
 }
 
 constexpr size_t WS_UNIT_BYTES = (size_t)C * C * 2 * 2 + 4 * C * 4;
