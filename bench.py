@@ -55,7 +55,7 @@ def make_inputs(w, torch, device):
 
 # HBM bytes per launch of the dominant kernel (read + written), from FETCH_SIZE / WRITE_SIZE counter runs of this
 # script scaled by a 1 GiB copy in the same run; the counter summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"hybrid_gdn_B8_T8192_H16_d128_p25": 809.0e6 + 302.3e6}
+MEASURED_TRAFFIC = {"hybrid_gdn_B8_T8192_H16_d128_p25": 871.5e6 + 302.5e6}
 
 
 def softmax_flops(types, T, block, K, V):
@@ -154,15 +154,28 @@ def main():
             del src, dst
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    n_timed_events = len(events)
+    # a few more steps with the two branches one after the other on one stream: each kernel's duration alone
+    with torch.no_grad():
+        _mixed_common.CONCURRENT_BRANCHES = False
+        step()
+        torch.cuda.synchronize()
+        _mixed_common.TIMING_HOOK = hook
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        _mixed_common.TIMING_HOOK = None
+        _mixed_common.CONCURRENT_BRANCHES = True
     tokens = w["B"] * w["T"]
     value = tokens / (ms_per_step * 1e-3)
 
-    def avg_ms(tag):
-        starts = [e for n, e in events if n == tag + ":start"]
-        ends = [e for n, e in events if n == tag + ":end"]
+    def avg_ms(tag, evs):
+        starts = [e for n, e in evs if n == tag + ":start"]
+        ends = [e for n, e in evs if n == tag + ":end"]
         return sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / max(1, len(starts))
 
-    sm_ms, lin_ms = avg_ms("softmax"), avg_ms("linear")
+    sm_ms, lin_ms = avg_ms("softmax", events[:n_timed_events]), avg_ms("linear", events[:n_timed_events])
+    sm_alone_ms, lin_alone_ms = avg_ms("softmax", events[n_timed_events:]), avg_ms("linear", events[n_timed_events:])
     types_host = ty.cpu()
     f_attn = softmax_flops(types_host, w["T"], w["block"], w["K"], w["V"])
     f_gdn = gdn_flops(types_host, w["K"], w["V"])
@@ -170,21 +183,24 @@ def main():
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", kernel="softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
                     unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=MEASURED_TRAFFIC.get(args.workload), launch_ms=sm_ms,
-                    algorithmic_flops=f_attn)
+                    algorithmic_flops=f_attn,
+                    # the same kernel with the GPU to itself (branches launched one after the other, outside the timed region)
+                    launch_ms_alone=sm_alone_ms, frac_alone=f_attn / (sm_alone_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS)
     else:
         # GDN-only workload: HBM-bound; algorithmic bytes = q,k,v read + o written + g,beta + final state
         B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
         nbytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * 6 + B * H * K * V * 4
         achieved = nbytes / (lin_ms * 1e-3) / 1e9
         roof = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=achieved, peak=PEAK_HBM_GBS,
-                    unit="GB/s", frac=achieved / PEAK_HBM_GBS, traffic=None, launch_ms=lin_ms, algorithmic_bytes=nbytes)
+                    unit="GB/s", frac=achieved / PEAK_HBM_GBS, traffic=None, launch_ms=lin_ms, algorithmic_bytes=nbytes,
+                    launch_ms_alone=lin_alone_ms, frac_alone=nbytes / (lin_alone_ms * 1e-3) / 1e9 / PEAK_HBM_GBS)
 
     rec = dict(
         metric="hybrid-layer fwd tokens/sec @T=8192,H=16,d=128 bf16; % of MFMA/HBM roofline",
         value=value, unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step,
         higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
         config=dict(workload=args.workload, **w, attn_fraction=float(types_host[..., 0].float().mean()),
-                    softmax_ms=sm_ms, linear_ms=lin_ms, step_flops=f_attn + f_gdn,
+                    softmax_ms=sm_ms, linear_ms=lin_ms, softmax_alone_ms=sm_alone_ms, linear_alone_ms=lin_alone_ms, step_flops=f_attn + f_gdn,
                     step_frac_of_mfma_peak=(f_attn + f_gdn) / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS),
         roofline=roof,
     )

@@ -16,6 +16,10 @@ _attn_streams: dict = {}
 # caller can record events on the stream the kernels were launched on.
 TIMING_HOOK = None
 
+# The softmax branch runs on a side stream next to the linear branch.  Set to False to launch both on the
+# caller's stream, one after the other (used to time each kernel alone).
+CONCURRENT_BRANCHES = True
+
 
 def _mark(name, stream):
     if TIMING_HOOK is not None:
@@ -117,8 +121,9 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
 
     r = route(types, T, nats_block_size, seqs)
     cur = torch.cuda.current_stream(dev)
-    side = _get_attn_stream(dev)
-    side.wait_stream(cur)
+    side = _get_attn_stream(dev) if CONCURRENT_BRANCHES else cur
+    if side is not cur:
+        side.wait_stream(cur)
     with torch.cuda.stream(side):
         _mark("softmax:start", side)
         o_attn, _lse, _ = parallel_attn_nats_fwd(
@@ -133,9 +138,10 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
                            nats_block_size, flags, output_final_state, seqs, block_start_state=want_start)
     o_lin, ht = res[0], res[1]
     _mark("linear:end", cur)
-    cur.wait_stream(side)
-    for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
-        t.record_stream(side)
+    if side is not cur:
+        cur.wait_stream(side)
+        for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
+            t.record_stream(side)
     if io_dtype != torch.bfloat16:
         o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
     if not inference:
