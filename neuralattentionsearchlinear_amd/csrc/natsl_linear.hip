@@ -83,18 +83,22 @@ NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
 template <int DK, bool DELTA>
 __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) {
   constexpr int KP = DK + 8;   // bf16 row pitch
-  constexpr int AP = 68;       // fp32 row pitch of the 64x64 fp32 matrices (16-byte multiple)
   constexpr int KL = DK / 32;  // 16-byte loads per thread per tile
+  // The 64x64 fp32 matrices of the solve are kept as their ten lower 16x16 blocks, block (i, k) at
+  // index i(i+1)/2 + k, rows of BP floats.  A = strictly lower system matrix; X = (I+A)^-1 row-major;
+  // Xt = the same blocks transposed (so that a block serves as an MFMA B operand with one 16-byte read).
+  constexpr int BP = 20, BLK = 16 * BP, NBLK = 10;
+  constexpr int TILE_BYTES = 2 * C * KP * 2, SOLVE_BYTES = 3 * NBLK * BLK * 4;
   // LDS: the q, k tiles are dead once the Gram products are done; the solve reuses their space
-  constexpr int TILE_BYTES = 2 * C * KP * 2, MAT_BYTES = C * AP * 4;
-  constexpr int REGION0 = DELTA ? (TILE_BYTES > 2 * MAT_BYTES ? TILE_BYTES : 2 * MAT_BYTES) : TILE_BYTES;
+  constexpr int REGION0 = (DELTA && SOLVE_BYTES > TILE_BYTES) ? SOLVE_BYTES : TILE_BYTES;
   __shared__ __align__(16) unsigned char region0[REGION0];
-  __shared__ __align__(16) float Am[DELTA ? C * AP : 4];
-  __shared__ float gam[C], rq[C], rk[C], bet[C];
+  __shared__ __align__(16) float gam[C], rq[C], rk[C], bet[C];
   bf16_t* Qs = reinterpret_cast<bf16_t*>(region0);
   bf16_t* Ks = Qs + C * KP;
-  float* Xm = reinterpret_cast<float*>(region0);             // (I+A)^-1, block lower triangular
-  float* Mm = reinterpret_cast<float*>(region0 + MAT_BYTES);  // inner sums of the block merge
+  float* Ab = reinterpret_cast<float*>(region0);
+  float* Xb = Ab + NBLK * BLK;
+  float* Xt = Xb + NBLK * BLK;
+  auto bidx = [](int i, int k) { return i * (i + 1) / 2 + k; };
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
@@ -177,8 +181,9 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     const int ti = wave >> 1, tj = wave & 1, l32 = lane & 31, hf = lane >> 5;
     const int i = 32 * ti + l32;  // P row owned by this lane
     bf16_t* prow = Pout + ((size_t)((2 * (i >> 4) + tj) * 64 + (i & 15))) * 8;
+    f32x16 gk;
     if (ti >= tj) {
-      f32x16 gk, gq;
+      f32x16 gq;
 #pragma unroll
       for (int r = 0; r < 16; ++r) gk[r] = gq[r] = 0.f;
 #pragma unroll
@@ -192,37 +197,45 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
         }
       }
       {
+        // this lane's 16 key tokens are four runs of four: 16-byte reads of their gamma and 1/|k|
         const float gi = gam[i], fi = p.scale * rq[i];
         u32x4 w[2];
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const int j0 = 32 * tj + 8 * (r >> 2) + 4 * hf + (r & 3);
-          const float p0 = i >= j0 ? fi * rk[j0] * gq[r] * __expf(gi - gam[j0]) : 0.f;
-          const float p1 = i >= j0 + 1 ? fi * rk[j0 + 1] * gq[r + 1] * __expf(gi - gam[j0 + 1]) : 0.f;
-          w[r >> 3][(r >> 1) & 3] = pack_bf16x2(p0, p1);
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int j0 = 32 * tj + 8 * q4 + 4 * hf;
+          const f32x4 gj = *reinterpret_cast<const f32x4*>(gam + j0), rj = *reinterpret_cast<const f32x4*>(rk + j0);
+          float pv[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pv[e] = i >= j0 + e ? fi * rj[e] * gq[4 * q4 + e] * __expf(gi - gj[e]) : 0.f;
+          w[q4 >> 1][2 * (q4 & 1)] = pack_bf16x2(pv[0], pv[1]);
+          w[q4 >> 1][2 * (q4 & 1) + 1] = pack_bf16x2(pv[2], pv[3]);
         }
         *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = w[0];
         *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = w[1];
-      }
-      if (DELTA) {
-        const int j = 32 * tj + l32;
-        const float gj = gam[j], rkj = rk[j];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int ii = 32 * ti + 8 * (r >> 2) + 4 * hf + (r & 3);
-          Am[ii * AP + j] = ii > j ? bet[ii] * rk[ii] * rkj * gk[r] * __expf(gam[ii] - gj) : 0.f;
-        }
       }
     } else {
       // the strictly upper 32x32 tile is zero
       const u32x4 z = {0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = z;
       *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = z;
-      if (DELTA) {
+    }
+    if (DELTA) {
+      // all waves are done reading the q, k tiles before the A blocks overwrite them
+      __syncthreads();
+      if (ti >= tj) {
+        const int j = 32 * tj + l32;
+        const float gj = gam[j], rkj = rk[j];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int ii = 8 * (r >> 2) + 4 * hf + (r & 3), j = 32 + l32;
-          Am[ii * AP + j] = 0.f;
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int i0 = 32 * ti + 8 * q4 + 4 * hf;  // rows i0..i0+3, all in one 16-row block
+          const f32x4 gi4 = *reinterpret_cast<const f32x4*>(gam + i0), ri4 = *reinterpret_cast<const f32x4*>(rk + i0),
+                      bi4 = *reinterpret_cast<const f32x4*>(bet + i0);
+          if ((i0 >> 4) >= (j >> 4)) {
+            float* dst = Ab + bidx(i0 >> 4, j >> 4) * BLK + (i0 & 15) * BP + (j & 15);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              dst[e * BP] = i0 + e > j ? bi4[e] * ri4[e] * rkj * gk[4 * q4 + e] * __expf(gi4[e] - gj) : 0.f;
+          }
         }
       }
     }
@@ -248,68 +261,72 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
   if (NATSL_ABL(p.dbg & 64)) return;  // no solve, no Tm store
   __syncthreads();
 
-  // ---- Tm = (I + A)^-1, fp32, blocked 4x4 with 16x16 blocks ----------------------------------
-  // diagonal blocks: forward substitution, one (block, column) per lane of wave 0
-  if (wave == 0) {
-    const int b0 = 16 * (lane >> 4), col = lane & 15;
+  // ---- X = (I + A)^-1 in fp32, 4x4 blocks of 16x16 ------------------------------------------
+  // diagonal blocks by forward substitution: wave b owns block (b, b), one column per lane
+  const int x16 = lane & 15, g4 = lane >> 4;
+  if (lane < 16) {
+    const float* Ad = Ab + bidx(wave, wave) * BLK;
+    f32x4 arow[16][4];
+#pragma unroll
+    for (int r = 1; r < 16; ++r)
+#pragma unroll
+      for (int j4 = 0; j4 < (r + 3) / 4; ++j4) arow[r][j4] = *reinterpret_cast<const f32x4*>(Ad + r * BP + 4 * j4);
     float x[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      float acc = r == col ? 1.f : 0.f;
+      float acc = r == x16 ? 1.f : 0.f;
 #pragma unroll
-      for (int j4 = 0; j4 < (r + 3) / 4; ++j4) {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(Am + (b0 + r) * AP + b0 + 4 * j4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (4 * j4 + e < r) acc -= a[e] * x[4 * j4 + e];
-      }
+      for (int j = 0; j < r; ++j) acc -= arow[r][j >> 2][j & 3] * x[j];
       x[r] = acc;
-      Xm[(b0 + r) * AP + b0 + col] = acc;
     }
+    float* Xd = Xb + bidx(wave, wave) * BLK;
+    float* Xtd = Xt + bidx(wave, wave) * BLK;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) Xd[r * BP + x16] = x[r];
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4)
+      *reinterpret_cast<f32x4*>(Xtd + x16 * BP + 4 * r4) = (f32x4){x[4 * r4], x[4 * r4 + 1], x[4 * r4 + 2], x[4 * r4 + 3]};
   }
   __syncthreads();
-  // off-diagonal blocks by block forward substitution, one block diagonal at a time:
-  //   X_ik = -X_ii * sum_{j=k}^{i-1} A_ij X_jk        (i = k + d)
-  {
-    const int r = tid >> 4, cc = tid & 15;
+  // off-diagonal blocks, one block diagonal at a time, on the fp32 matrix cores:
+  //   X_ik = -X_ii * sum_{j=k}^{i-1} A_ij X_jk        (i = k + d; wave k owns block (k+d, k))
+  // MFMA 16x16x4: lane (x, g) supplies A[x][kk] and B[kk][x].  With kk = 4g + s in step s, the A
+  // operand of all four steps is one 16-byte row read, and an accumulator (lane = column x, registers
+  // = rows 4g..4g+3) is already a B operand, so the inner sum feeds the second product from registers.
 #pragma unroll
-    for (int d = 1; d < 4; ++d) {
+  for (int d = 1; d < 4; ++d) {
+    if (wave + d < 4) {
+      const int k = wave, i = wave + d;
+      f32x4 M = {0.f, 0.f, 0.f, 0.f};
+      for (int j = k; j < i; ++j) {
+        const f32x4 a4 = *reinterpret_cast<const f32x4*>(Ab + bidx(i, j) * BLK + x16 * BP + 4 * g4);
+        const f32x4 b4 = *reinterpret_cast<const f32x4*>(Xt + bidx(j, k) * BLK + x16 * BP + 4 * g4);
 #pragma unroll
-      for (int k = 0; k + d < 4; ++k) {
-        const int i = k + d;
-        float acc = 0.f;
-#pragma unroll
-        for (int j = k; j < i; ++j)
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) {
-            const f32x4 a = *reinterpret_cast<const f32x4*>(Am + (16 * i + r) * AP + 16 * j + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc += a[e] * Xm[(16 * j + 4 * e4 + e) * AP + 16 * k + cc];
-          }
-        Mm[(16 * i + r) * AP + 16 * k + cc] = acc;
+        for (int st = 0; st < 4; ++st) M = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[st], b4[st], M, 0, 0, 0);
       }
-      __syncthreads();
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(Xb + bidx(i, i) * BLK + x16 * BP + 4 * g4);
+      f32x4 Xa = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int k = 0; k + d < 4; ++k) {
-        const int i = k + d;
-        float acc = 0.f;
+      for (int st = 0; st < 4; ++st) Xa = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[st], M[st], Xa, 0, 0, 0);
+      float* Xo = Xb + bidx(i, k) * BLK;
 #pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-          const f32x4 a = *reinterpret_cast<const f32x4*>(Xm + (16 * i + r) * AP + 16 * i + 4 * e4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc -= a[e] * Mm[(16 * i + 4 * e4 + e) * AP + 16 * k + cc];
-        }
-        Xm[(16 * i + r) * AP + 16 * k + cc] = acc;
-      }
-      __syncthreads();
+      for (int r = 0; r < 4; ++r) Xo[(4 * g4 + r) * BP + x16] = -Xa[r];
+      *reinterpret_cast<f32x4*>(Xt + bidx(i, k) * BLK + x16 * BP + 4 * g4) = (f32x4){-Xa[0], -Xa[1], -Xa[2], -Xa[3]};
     }
+    __syncthreads();
   }
   // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above)
   if (!NATSL_ABL(p.dbg & 128)) {
     const int row = tid >> 2, cb = tid & 3;
     float x[16];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) x[e] = cb <= (row >> 4) ? Xm[row * AP + 16 * cb + e] * bet[16 * cb + e] : 0.f;
+    for (int e4 = 0; e4 < 4; ++e4) {
+      const f32x4 xv = cb <= (row >> 4) ? *reinterpret_cast<const f32x4*>(Xb + bidx(row >> 4, cb <= (row >> 4) ? cb : 0) * BLK + (row & 15) * BP + 4 * e4)
+                                        : (f32x4){0.f, 0.f, 0.f, 0.f};
+      const f32x4 bv = *reinterpret_cast<const f32x4*>(bet + 16 * cb + 4 * e4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * e4 + e] = xv[e] * bv[e];
+    }
     u32x4 w0, w1;  // tokens {0..3, 8..11} and {4..7, 12..15} of this thread's 16
     w0[0] = pack_bf16x2(x[0], x[1]);  w0[1] = pack_bf16x2(x[2], x[3]);   w0[2] = pack_bf16x2(x[8], x[9]);   w0[3] = pack_bf16x2(x[10], x[11]);
     w1[0] = pack_bf16x2(x[4], x[5]);  w1[1] = pack_bf16x2(x[6], x[7]);   w1[2] = pack_bf16x2(x[12], x[13]); w1[3] = pack_bf16x2(x[14], x[15]);
