@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
     ap.add_argument("--cpu-batch", type=int, default=4, help="sequences of the slice timed on the CPU")
+    ap.add_argument("--serial-branches", action="store_true",
+                    help="force the softmax and the linear branch onto one stream, one after the other (default: the operator decides)")
+    ap.add_argument("--concurrent-branches", action="store_true", help="force the softmax branch onto a side stream")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device copy after the timed steps, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -136,6 +139,8 @@ def main():
                                    output_final_state_gated_delta=True, decay_for_non_gdn_blocks=True), ty
 
     with torch.no_grad():
+        if args.serial_branches or args.concurrent_branches:
+            _mixed_common.CONCURRENT_BRANCHES = bool(args.concurrent_branches)
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
@@ -165,7 +170,7 @@ def main():
             step()
         torch.cuda.synchronize()
         _mixed_common.TIMING_HOOK = None
-        _mixed_common.CONCURRENT_BRANCHES = True
+        _mixed_common.CONCURRENT_BRANCHES = None
     tokens = w["B"] * w["T"]
     value = tokens / (ms_per_step * 1e-3)
 

@@ -16,9 +16,21 @@ _attn_streams: dict = {}
 # caller can record events on the stream the kernels were launched on.
 TIMING_HOOK = None
 
-# The softmax branch runs on a side stream next to the linear branch.  Set to False to launch both on the
-# caller's stream, one after the other (used to time each kernel alone).
-CONCURRENT_BRANCHES = True
+# Where the softmax branch is launched.  True: on a side stream next to the linear branch (as the
+# reference's Mamba operator does); False: on the caller's stream, one branch after the other (as the
+# reference's GDN operator does); None: decide per call - side by side only when the linear branch's scan
+# has too few workgroups to fill the GPU on its own.  Both kernels are sized to occupy whole CUs, so when
+# each fills the machine alone, running them side by side gains nothing (measured) and only blurs timings.
+CONCURRENT_BRANCHES = None
+_SCAN_V_SLICE = 32          # value columns per scan workgroup (BV in csrc/natsl_linear.hip)
+_SCAN_WGS_PER_CU = 2        # scan workgroups resident per CU
+
+
+def _run_side_by_side(dev, n_chains: int, V: int) -> bool:
+    if CONCURRENT_BRANCHES is not None:
+        return bool(CONCURRENT_BRANCHES)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    return n_chains * (V // _SCAN_V_SLICE) < _SCAN_WGS_PER_CU * cus
 
 
 def _mark(name, stream):
@@ -121,7 +133,8 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
 
     r = route(types, T, nats_block_size, seqs)
     cur = torch.cuda.current_stream(dev)
-    side = _get_attn_stream(dev) if CONCURRENT_BRANCHES else cur
+    n_chains = (seqs.n_seqs if seqs is not None else q_lattn.shape[0]) * q_lattn.shape[2]
+    side = _get_attn_stream(dev) if _run_side_by_side(dev, n_chains, v_lattn.shape[-1]) else cur
     if side is not cur:
         side.wait_stream(cur)
     with torch.cuda.stream(side):
