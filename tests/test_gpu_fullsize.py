@@ -1,0 +1,195 @@
+"""GPU parity at the FULL sizes the path is specified on, through size-independent properties.
+
+The fp32 oracle would take minutes to hours at these shapes, so the checks are properties that hold for
+any correct implementation:
+  * the softmax branch on single (sequence, head) slices against a dense fp32 masked softmax built from
+    the oracle's visibility rule (tolerance: max-abs 2e-2, rel-L2 5e-3, as everywhere);
+  * exact homogeneity: every output is linear in v, and scaling by a power of two is exact in bf16 and
+    fp32, so o(2v) == 2 o(v) BIT FOR BIT, for the softmax, GDN and Mamba branches (up to denormal flushes);
+  * state hand-off: a sequence run in one call equals the same sequence run as two calls with the first
+    call's final state as the second's initial state (bit-exact: same chunk grid, fp32 state);
+  * packed input: sequences packed into one row (cu_seqlens) give bit-identical outputs to separate calls.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import softmax_branch as SB
+from tests._util import assert_close, make_types
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+def _randn(shape, seed, dtype=torch.bfloat16):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    return torch.randn(*shape, device=DEV, generator=g, dtype=torch.float32).to(dtype)
+
+
+def _inputs(B, T, H, K, V, seed):
+    q, k, v = _randn((B, T, H, K), seed), _randn((B, T, H, K), seed + 1), _randn((B, T, H, V), seed + 2)
+    g = -F.softplus(_randn((B, T, H), seed + 3, torch.float32))
+    beta = torch.sigmoid(_randn((B, T, H), seed + 4, torch.float32)).to(torch.bfloat16)
+    return q, k, v, g, beta
+
+
+def _assert_doubles(o2, o1, what):
+    """o2 == 2*o1 bit for bit, except where an intermediate product falls into the denormal range (flushed by
+    the matrix cores): there the two runs may differ by one rounding.  Allow at most one element in a million,
+    and only by a negligible amount."""
+    d = (o2.float() - 2 * o1.float()).abs()
+    bad = int((d != 0).sum())
+    assert bad <= max(1, o1.numel() // 1_000_000) and float(d.max()) <= 1e-4, f"{what}: {bad} elements differ, max {float(d.max()):.3e}"
+
+
+def _linear(kind, q, k, v, g, beta, h0, types, block, scale, decay=True, seqs=None, final=True):
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd._mixed_common import linear_chunk_fwd
+    flags = (_capi.DECAY_NON_LINEAR if decay else 0) | _capi.INTRA_CHUNK | (_capi.QK_L2NORM if kind == 'gdn' else 0)
+    with torch.no_grad():
+        return linear_chunk_fwd(kind, q, k, v, g, beta, h0, types, scale, block, flags, final, seqs)
+
+
+def _softmax(q, k, v, types, block, scale, same_block=True, seqs=None):
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_fwd
+    with torch.no_grad():
+        r = nats_util.route(types, q.shape[1], block, seqs)
+        o, lse, _ = parallel_attn_nats_fwd(q, k, v, types, r['nats_block_indices'], None, scale, block,
+                                           compute_incomplete_chunk_scores=same_block, n_nats_blocks=r['n_nats_blocks'], seqs=seqs)
+    return o, lse
+
+
+# --------------------------------------------------------------------------------------------
+# c2: B8 T8192 H16 K=V=128, 25 % attention blocks
+# --------------------------------------------------------------------------------------------
+C2 = dict(B=8, T=8192, H=16, K=128, V=128, block=64, p=0.25)
+
+
+@pytest.fixture(scope="module")
+def c2():
+    w = C2
+    q, k, v, g, beta = _inputs(w['B'], w['T'], w['H'], w['K'], w['V'], 100)
+    ty = make_types(w['B'], w['T'] // w['block'], w['H'], w['p'], 7, torch.bfloat16).to(DEV)
+    return dict(q=q, k=k, v=v, g=g, beta=beta, ty=ty)
+
+
+@pytest.mark.parametrize("same_block", [True, False])
+def test_c2_softmax_slices_against_dense_fp32(c2, same_block):
+    w = C2
+    scale = w['K'] ** -0.5
+    o, lse = _softmax(c2['q'], c2['k'], c2['v'], c2['ty'], w['block'], scale, same_block)
+    for b, h in ((0, 0), (3, 5), (7, 15)):
+        mask = SB.visibility_mask(c2['ty'][b, :, h, 0].float().cpu(), w['T'], w['block'], same_block).to(DEV)
+        qf, kf, vf = (c2[n][b, :, h].float() for n in ('q', 'k', 'v'))
+        s = (qf @ kf.T) * scale
+        s = s.masked_fill(~mask, float('-inf'))
+        seen = mask.any(-1)
+        p = torch.softmax(s, -1).nan_to_num(0.0)          # rows that see no key give 0
+        ref = p @ vf
+        assert_close(o[b, :, h].float(), ref, f"o_attn[{b},:,{h}]")
+        lse_ref = torch.where(seen, torch.logsumexp(s, -1) * 1.4426950408889634, torch.zeros_like(seen, dtype=torch.float32))
+        assert float((lse[b, :, h] - lse_ref).abs().max()) <= 2e-2, "lse (log2 units)"
+
+
+def test_c2_outputs_are_exactly_homogeneous_in_v(c2):
+    w = C2
+    scale = w['K'] ** -0.5
+    o1, _ = _softmax(c2['q'], c2['k'], c2['v'], c2['ty'], w['block'], scale)
+    o2, _ = _softmax(c2['q'], c2['k'], c2['v'] * 2, c2['ty'], w['block'], scale)
+    assert torch.equal(o2, o1 * 2), "softmax branch: o(2v) != 2 o(v)"
+    l1, s1 = _linear('gdn', c2['q'], c2['k'], c2['v'], c2['g'], c2['beta'], None, c2['ty'], w['block'], scale)
+    l2, s2 = _linear('gdn', c2['q'], c2['k'], c2['v'] * 2, c2['g'], c2['beta'], None, c2['ty'], w['block'], scale)
+    _assert_doubles(l2, l1, "GDN branch: o(2v) vs 2 o(v)")
+    assert torch.equal(s2, s1 * 2), "GDN branch: S(2v) != 2 S(v)"
+    assert torch.isfinite(l1.float()).all() and torch.isfinite(s1).all()
+
+
+def test_c2_gdn_state_hand_off(c2):
+    w = C2
+    scale = w['K'] ** -0.5
+    half = w['T'] // 2
+    nb = half // w['block']
+    o, s = _linear('gdn', c2['q'], c2['k'], c2['v'], c2['g'], c2['beta'], None, c2['ty'], w['block'], scale)
+    sl = lambda t, a, b: t[:, a:b].contiguous()
+    oa, sa = _linear('gdn', *(sl(c2[n], 0, half) for n in ('q', 'k', 'v', 'g', 'beta')), None, sl(c2['ty'], 0, nb), w['block'], scale)
+    ob, sb = _linear('gdn', *(sl(c2[n], half, w['T']) for n in ('q', 'k', 'v', 'g', 'beta')), sa, sl(c2['ty'], nb, 2 * nb), w['block'], scale)
+    assert torch.equal(o[:, :half], oa) and torch.equal(o[:, half:], ob), "outputs differ across the hand-off"
+    assert torch.equal(s, sb), "final state differs across the hand-off"
+
+
+# --------------------------------------------------------------------------------------------
+# c1: B4 T4096 H16 K=V=128, every block linear
+# --------------------------------------------------------------------------------------------
+def test_c1_all_linear_matches_token_recurrence_on_a_slice():
+    """All blocks linear: the chunked kernels must equal the plain token-by-token gated delta rule.  The
+    recurrence (oracle) is run for two (sequence, head) slices only."""
+    from oracle import linear_branch as LB
+    B, T, H, K, V, block = 4, 4096, 16, 128, 128, 64
+    q, k, v, g, beta = _inputs(B, T, H, K, V, 300)
+    ty = make_types(B, T // block, H, 0.0, 1, torch.bfloat16).to(DEV)
+    scale = K ** -0.5
+    o, s = _linear('gdn', q, k, v, g, beta, None, ty, block, scale)
+    for b, h in ((0, 0), (3, 11)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()
+        lin = torch.ones(1, T // block, 1)
+        o_ref, s_ref = LB.gdn_token_recurrence(sl(q), sl(k), sl(v), sl(g), sl(beta), lin, scale, None, block=block)
+        assert_close(o[b:b + 1, :, h:h + 1].float(), o_ref, f"o_gdn[{b},:,{h}]")
+        assert_close(s[b:b + 1, h:h + 1], s_ref, f"final_state[{b},{h}]")
+
+
+# --------------------------------------------------------------------------------------------
+# c3: B1 T65536 H32 K=V=128, 10 % attention, also packed as 8192/16384/16384/24576
+# --------------------------------------------------------------------------------------------
+def test_c3_packed_equals_separate_calls():
+    from neuralattentionsearchlinear_amd.nats_util import pack_sequences
+    T, H, K, V, block = 65536, 32, 128, 128, 64
+    lens = [8192, 16384, 16384, 24576]
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    q, k, v, g, beta = _inputs(1, T, H, K, V, 500)
+    parts = [make_types(1, n // block, H, 0.10, 20 + i, torch.bfloat16) for i, n in enumerate(lens)]
+    ty = torch.cat(parts, 1).to(DEV)
+    scale = K ** -0.5
+    cud = torch.tensor(cu, dtype=torch.int64, device=DEV)
+    seqs = pack_sequences(cud, None, block, torch.device(DEV))
+    o_attn, lse = _softmax(q, k, v, ty, block, scale, True, seqs)
+    o_lin, s = _linear('gdn', q, k, v, g, beta, None, ty, block, scale, seqs=seqs)
+    assert s.shape == (len(lens), H, K, V)
+    nb0 = 0
+    for i, (a, b) in enumerate(zip(cu[:-1], cu[1:])):
+        nb = (b - a) // block
+        sl = lambda t: t[:, a:b].contiguous()
+        tyi = ty[:, nb0:nb0 + nb].contiguous()
+        oa, la = _softmax(sl(q), sl(k), sl(v), tyi, block, scale, True)
+        ol, si = _linear('gdn', sl(q), sl(k), sl(v), sl(g), sl(beta), None, tyi, block, scale)
+        assert torch.equal(o_attn[:, a:b], oa) and torch.equal(lse[:, a:b], la), f"softmax branch, sequence {i}"
+        assert torch.equal(o_lin[:, a:b], ol) and torch.equal(s[i:i + 1], si), f"GDN branch, sequence {i}"
+        nb0 += nb
+
+
+# --------------------------------------------------------------------------------------------
+# c4: Mamba, B4 T8192 H32, state K=128, head V=64, selector block 256, 25 % attention
+# --------------------------------------------------------------------------------------------
+def test_c4_mamba_homogeneity_and_hand_off():
+    B, T, H, K, V, block = 4, 8192, 32, 128, 64, 256
+    q, k, v, g, _ = _inputs(B, T, H, K, V, 700)
+    ty = make_types(B, T // block, H, 0.25, 3, torch.bfloat16).to(DEV)
+    o, s = _linear('mamba', q, k, v, g, None, None, ty, block, 1.0)
+    o2, s2 = _linear('mamba', q, k, v * 2, g, None, None, ty, block, 1.0)
+    _assert_doubles(o2, o, "Mamba branch: o(2x) vs 2 o(x)")
+    assert torch.equal(s2, s * 2), "Mamba branch: S(2x) != 2 S(x)"
+    half, nb = T // 2, T // 2 // block
+    sl = lambda t, a, b: t[:, a:b].contiguous()
+    oa, sa = _linear('mamba', *(sl(t, 0, half) for t in (q, k, v, g)), None, None, sl(ty, 0, nb), block, 1.0)
+    ob, sb = _linear('mamba', *(sl(t, half, T) for t in (q, k, v, g)), None, sa, sl(ty, nb, 2 * nb), block, 1.0)
+    assert torch.equal(o[:, :half], oa) and torch.equal(o[:, half:], ob) and torch.equal(s, sb), "state hand-off"
+    # the attention view of the same layer: K=128, V=64, block 256
+    oa1, _ = _softmax(q, k, v, ty, block, K ** -0.5)
+    oa2, _ = _softmax(q, k, v * 2, ty, block, K ** -0.5)
+    assert torch.equal(oa2, oa1 * 2)
+    mask = SB.visibility_mask(ty[1, :, 4, 0].float().cpu(), T, block, True).to(DEV)
+    sc = (q[1, :, 4].float() @ k[1, :, 4].float().T) * K ** -0.5
+    ref = torch.softmax(sc.masked_fill(~mask, float('-inf')), -1) @ v[1, :, 4].float()
+    assert_close(oa1[1, :, 4].float(), ref, "o_attn slice")
