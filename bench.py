@@ -22,6 +22,11 @@ WORKLOADS = {
     "gdn_only_B4_T4096_H16_d128": dict(B=4, T=4096, H=16, K=128, V=128, p_attn=0.0, block=64),
     "hybrid_gdn_B1_T65536_H32_d128_p10": dict(B=1, T=65536, H=32, K=128, V=128, p_attn=0.10, block=64),
 }
+# decode: one new token per sequence on cached states, the attention branch over the cached keys/values of the
+# attention-typed blocks (p_attn of the context) plus the current block; not the headline metric
+DECODE_WORKLOADS = {
+    "decode_gdn_B8_ctx8192_H16_d128_p25": dict(B=8, ctx=8192, H=16, K=128, V=128, p_attn=0.25, block=64, n_in_block=17),
+}
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 
@@ -93,12 +98,58 @@ def cpu_baseline(host, w, types_host, torch, max_heads=None, max_batch=None):
     return dict(value=tok_s, unit="tokens/s", cores=threads, kind="port", sample=sample)
 
 
+def bench_decode(args):
+    """One decode step (new token of every sequence): masked attention over the cached keys/values + the gated
+    delta rule on the cached state.  HBM-bound: the states are read and written once, the caches read once."""
+    import torch
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn_recurrent
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    w = DECODE_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    B, H, K, V, block = w["B"], w["H"], w["K"], w["V"], w["block"]
+    TK = int(w["ctx"] * w["p_attn"]) // block * block + w["n_in_block"] + 1      # cached attention blocks + current block + new token
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    q, k, v = rn(B, 1, H, K).bfloat16(), rn(B, 1, H, K).bfloat16(), rn(B, 1, H, V).bfloat16()
+    ka, va = rn(B, TK, H, K).bfloat16(), rn(B, TK, H, V).bfloat16()
+    mask = torch.ones(B, H, 1, TK, dtype=torch.bool, device=dev)
+    S, S0 = rn(B, H, K, V) * 0.1, rn(B, H, K, V) * 0.1
+    gl = -torch.nn.functional.softplus(rn(B, 1, H))
+    gcum = -torch.rand(B, H, device=dev, generator=g) * 5
+    beta = torch.sigmoid(rn(B, 1, H)).bfloat16()
+    ty = torch.ones(B, 1, H, 2, device=dev, dtype=torch.bfloat16)
+
+    def step():
+        return nats_mixed_attn_gdn_recurrent(q, ka, va, q, k, v, mask, S, S0, gl, gcum, beta, ty, n_tokens_in_current_block=w["n_in_block"],
+                                             nats_block_size=block, ops_for_incomplete_chunks="all", decay_for_non_gdn_blocks=True)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    nbytes = B * H * K * V * 4 * 3 + B * TK * H * (K + V) * 2 + B * H * (2 * K + 2 * V) * 2 * 2
+    print(json.dumps(dict(
+        metric="hybrid-layer decode tokens/sec (one new token per sequence) @ctx=8192,H=16,d=128 bf16", value=B / (ms * 1e-3),
+        unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak",
+        vs_baseline=None, dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w, cached_keys=TK),
+        roofline=dict(bound="hbm", kernel="gdn_recurrent_kernel+attn_masked_kernel", achieved=nbytes / (ms * 1e-3) / 1e9,
+                      peak=PEAK_HBM_GBS, unit="GB/s", frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, traffic=None,
+                      algorithmic_bytes=nbytes, note="whole step incl. launch overheads of two kernels"))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
     ap.add_argument("--cpu-batch", type=int, default=4, help="sequences of the slice timed on the CPU")
@@ -114,6 +165,8 @@ def main():
               "GPU; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload in DECODE_WORKLOADS:
+        return bench_decode(args)
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn

@@ -142,6 +142,47 @@ int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const 
                         const void* w2, void* y, int64_t rows, int D, int dtype, float eps, int w_dtype,
                         natsl_stream_t stream);
 
+/* Decode: T tokens that continue the current (incomplete) selector block of N cached sequences, token by
+ * token.  Per token: S *= e^g; d = beta (v - S^T k); S += k d^T; o = scale S^T q (k, q L2-normalised with
+ * NATSL_QK_L2NORM).  Only the first min(T, block - n_tokens_in_block) tokens are processed.  If they
+ * complete the block (n_tokens_in_block + T >= block) and the block is not typed linear, S is restored to
+ * h_block_start (times e^(g_cumsum + sum of g) with NATSL_DECAY_NON_LINEAR), and in either case
+ * h_block_start <- S.  q,k [N,T,H,K], v,o [N,T,H,V], beta [N,T,H] in `dtype`; g fp32 [N,T,H];
+ * g_cumsum fp32 [N,H] or NULL (0): sum of g over the tokens already in the block; h0 fp32 [N,H,K,V] or NULL
+ * (zeros); h_block_start fp32 [N,H,K,V] in/out; ht fp32 [N,H,K,V] or NULL; types [N,1,HN,2] (op 1 = linear);
+ * n_tokens_in_block int32 [N] or NULL (then the scalar is used for every sequence).
+ * Replaces fused_recurrent_gated_delta_rule_nats_fwd, src/nats/ops/gated_delta_rule/fused_recurrent.py:360-470
+ * (kernel :28-358) as called with update_hs_for_each_iter=True at
+ * src/nats/ops/mixed_ops/mixed_attn_gdn.py:485-503. */
+int natsl_gdn_recurrent_fwd(const void* q, const void* k, const void* v, const float* g, const float* g_cumsum,
+                            const void* beta, const float* h0, float* h_block_start, void* o, float* ht,
+                            const void* types, int types_dtype, const int32_t* n_tokens_in_block,
+                            int n_tokens_in_block_scalar, int N, int T, int H, int HN, int K, int V, int block,
+                            float scale, int flags, int dtype, natsl_stream_t stream);
+
+/* The same for the Mamba2 (SSD) branch: S *= e^g; S += k v^T; o = scale S^T q (q = C, k = B, v = x*dt); no beta,
+ * no normalisation (NATSL_QK_L2NORM is ignored).
+ * Replaces fused_recurrent_mamba_nats_fwd (src/nats/ops/mamba/fused_recurrent.py, kernel :150-300) as called
+ * at src/nats/ops/mixed_ops/mixed_attn_mamba.py:498-514. */
+int natsl_mamba_recurrent_fwd(const void* q, const void* k, const void* v, const float* g, const float* g_cumsum,
+                              const float* h0, float* h_block_start, void* o, float* ht, const void* types,
+                              int types_dtype, const int32_t* n_tokens_in_block, int n_tokens_in_block_scalar, int N,
+                              int T, int H, int HN, int K, int V, int block, float scale, int flags, int dtype,
+                              natsl_stream_t stream);
+
+/* Decode: softmax attention of TQ queries over TK cached keys under an explicit visibility mask.
+ * q [B,TQ,HQ,K], k [B,TK,HKV,K], v [B,TK,HKV,V], o [B,TQ,HQ,V] in `dtype`; mask uint8 [B,HM,TQ,TK], non-zero =
+ * visible, HM divides HQ; query head hq uses kv head hq/(HQ/HKV) and mask head hq/(HQ/HM).  A query that sees
+ * no key gives 0.  With a workspace of natsl_attn_masked_workspace_bytes() the keys of one query are split over
+ * several workgroups (needed to fill the GPU when B*TQ*HQ is small); with workspace = NULL one workgroup
+ * handles a query.
+ * Replaces repeat_masks + torch.nn.functional.scaled_dot_product_attention at
+ * src/nats/ops/mixed_ops/mixed_attn_gdn.py:475-481. */
+size_t natsl_attn_masked_workspace_bytes(int B, int TQ, int TK, int HQ, int V);
+int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
+                          int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
+                          size_t workspace_bytes, natsl_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

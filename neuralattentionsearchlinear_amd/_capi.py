@@ -39,6 +39,15 @@ _SIGNATURES = {
                                       c_int, c_void_p, c_int, c_int, c_void_p]),
     "natsl_norm_gate_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                     c_float, c_int, c_void_p]),
+    "natsl_gdn_recurrent_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_float, c_int, c_int, c_void_p]),
+    "natsl_mamba_recurrent_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          c_float, c_int, c_int, c_void_p]),
+    "natsl_attn_masked_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "natsl_attn_masked_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_int, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
 }
 
 

@@ -101,3 +101,125 @@ def nats_mixed_attn_gdn_chunk_inference(
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
         qk_l2norm=lattn_use_qk_l2norm_in_kernel, inference=True, op_type_last_chunk=op_type_last_chunk,
         n_tokens_in_current_block=n_tokens_in_current_block)
+
+
+def fused_recurrent_gated_delta_rule_nats_fwd(q, k, v, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block,
+                                              nats_block_size, scale, initial_state, initial_state_in_current_block,
+                                              output_final_state=True, use_qk_l2norm_in_kernel=True,
+                                              decay_for_non_gdn_blocks=False):
+    """The gated delta rule token by token on a cached state, for tokens that continue the current selector
+    block (src/nats/ops/gated_delta_rule/fused_recurrent.py:360-470 with update_hs_for_each_iter=True).
+    -> (o, final_state or None, initial_state_in_current_block); the last is updated in place when the
+    tokens complete the block, as the reference's kernel does."""
+    from . import _capi
+    N, T, H, K = q.shape
+    V = v.shape[-1]
+    if nats_block_types.shape[1] != 1:
+        raise AssertionError("the recurrent form only continues the current selector block: nats_block_types must hold one block")  # :417-419
+    HN = nats_block_types.shape[2]
+    dev = q.device
+    q, k, v, beta = (t.contiguous() for t in (q, k, v, beta))
+    if not (q.dtype == k.dtype == v.dtype == beta.dtype):
+        raise ValueError("q, k, v, beta must share a dtype")
+    g = g.to(torch.float32).contiguous()
+    types = nats_block_types if nats_block_types.dtype in (torch.float32, torch.bfloat16) else nats_block_types.float()
+    types = types.contiguous()
+    if initial_state is not None:
+        initial_state = initial_state.to(torch.float32).contiguous()
+    if initial_state_in_current_block is None:                                           # :398-402
+        initial_state_in_current_block = (initial_state.clone() if initial_state is not None
+                                          else torch.zeros(N, H, K, V, dtype=torch.float32, device=dev))
+    if initial_state_in_current_block.dtype != torch.float32 or not initial_state_in_current_block.is_contiguous():
+        raise ValueError("initial_state_in_current_block must be a contiguous fp32 tensor (it is updated in place)")
+    if g_cumsum is not None:
+        g_cumsum = g_cumsum.to(torch.float32).reshape(N, H).contiguous()
+    if torch.is_tensor(n_tokens_in_current_block):
+        n_ptr, n_scalar = n_tokens_in_current_block.to(device=dev, dtype=torch.int32).contiguous(), 0
+    else:
+        n_ptr, n_scalar = None, int(n_tokens_in_current_block)
+    o = torch.empty(N, T, H, V, dtype=q.dtype, device=dev)
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
+    flags = (_capi.DECAY_NON_LINEAR if decay_for_non_gdn_blocks else 0) | (_capi.QK_L2NORM if use_qk_l2norm_in_kernel else 0)
+    rc = _capi.lib().natsl_gdn_recurrent_fwd(
+        _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), _capi.ptr(g_cumsum), _capi.ptr(beta), _capi.ptr(initial_state),
+        _capi.ptr(initial_state_in_current_block), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype),
+        _capi.ptr(n_ptr), n_scalar, N, T, H, HN, K, V, int(nats_block_size), float(scale), flags, _capi.dtype_code(q.dtype),
+        _capi.stream_ptr(dev))
+    _capi.check(rc, "natsl_gdn_recurrent_fwd")
+    return o, ht, initial_state_in_current_block
+
+
+def masked_attention(q, k, v, attn_msk, scale):
+    """Softmax attention of a few queries over cached keys under a boolean mask [B, HM, TQ, TK] (HM divides the
+    number of query heads); replaces repeat_masks + scaled_dot_product_attention at
+    src/nats/ops/mixed_ops/mixed_attn_gdn.py:475-481.  A query that sees no key gives 0."""
+    from . import _capi
+    B, TQ, HQ, K = q.shape
+    TK, HKV, V = k.shape[1], k.shape[2], v.shape[-1]
+    if attn_msk.dim() != 4 or attn_msk.shape[0] != B or attn_msk.shape[2] != TQ or attn_msk.shape[3] != TK:
+        raise ValueError(f"attn_msk must be [B, heads, {TQ}, {TK}], got {tuple(attn_msk.shape)}")
+    q, k, v = (t.contiguous() for t in (q, k, v))
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+    mask = attn_msk.to(torch.bool).contiguous().view(torch.uint8)
+    o = torch.empty(B, TQ, HQ, V, dtype=q.dtype, device=q.device)
+    L = _capi.lib()
+    ws_bytes = L.natsl_attn_masked_workspace_bytes(B, TQ, TK, HQ, V)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    rc = L.natsl_attn_masked_fwd(_capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(mask), _capi.ptr(o), B, TQ, TK, HQ,
+                                 HKV, mask.shape[1], K, V, float(scale), _capi.dtype_code(q.dtype), _capi.ptr(ws), ws_bytes,
+                                 _capi.stream_ptr(q.device))
+    _capi.check(rc, "natsl_attn_masked_fwd")
+    return o
+
+
+def nats_mixed_attn_gdn_recurrent(
+        q_attn: torch.Tensor, k_attn: torch.Tensor, v_attn: torch.Tensor,
+        q_lattn: torch.Tensor, k_lattn: torch.Tensor, v_lattn: torch.Tensor,
+        attn_msk: torch.Tensor,
+        initial_state_gated_delta: torch.Tensor,
+        initial_state_gated_delta_chunk_start: torch.Tensor,
+        g: torch.Tensor,
+        g_cumsum: torch.Tensor,
+        beta: torch.Tensor,
+        nats_block_types: torch.Tensor,
+        n_tokens_in_current_block: int = 0,
+        scale_attn=None, scale_lattn=None,
+        cu_seqlens=None, cu_seqlens_nats=None,
+        nats_block_size: int = 64,
+        attn_sw_size: int | None = None,
+        ops_for_incomplete_chunks: str = 'gated_delta_net',
+        output_final_state_gated_delta: bool = False,
+        decay_for_non_gdn_blocks: bool = False,
+        incomplete_block_start_with_ht: bool = True,
+        use_g_for_attn: bool = False,
+        lattn_use_qk_l2norm_in_kernel: bool = True,
+):
+    """Decode step(s) of the hybrid layer (src/nats/ops/mixed_ops/mixed_attn_gdn.py:443-591): masked attention
+    of the new queries over the cached keys/values, and the gated delta rule token by token on the cached
+    state. -> (o_gated_delta_net, o_attn, final_state, initial_state_in_current_block).
+
+    Built for the modes whose linear operator also runs on the incomplete block ('all', 'gated_delta_net');
+    the reference's 'attn' mode (state advanced in block-sized pieces, :504-589) is not."""
+    if scale_attn is None:
+        scale_attn = k_attn.shape[-1] ** -0.5
+    if scale_lattn is None:
+        scale_lattn = k_lattn.shape[-1] ** -0.5
+    strategy = all_incomplete_ops[ops_for_incomplete_chunks]
+    if not strategy.gated_delta_net:
+        raise NotImplementedError("the recurrent (decode) operator is built for ops_for_incomplete_chunks 'all' and "
+                                  "'gated_delta_net' only")
+    if cu_seqlens is not None or cu_seqlens_nats is not None:
+        raise NotImplementedError("packed sequences are not supported by the recurrent (decode) operator")
+    if attn_sw_size is not None or use_g_for_attn:
+        raise NotImplementedError("attn_sw_size / use_g_for_attn are not built")
+    if not q_lattn.is_cuda:
+        from . import _capi
+        raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
+    with torch.no_grad():
+        o_attn = masked_attention(q_attn, k_attn, v_attn, attn_msk, scale_attn)
+        o_gdn, final_state, start = fused_recurrent_gated_delta_rule_nats_fwd(
+            q_lattn, k_lattn, v_lattn, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block, nats_block_size,
+            scale_lattn, initial_state_gated_delta, initial_state_gated_delta_chunk_start, output_final_state=True,
+            use_qk_l2norm_in_kernel=lattn_use_qk_l2norm_in_kernel, decay_for_non_gdn_blocks=decay_for_non_gdn_blocks)
+    return o_gdn, o_attn, final_state, start

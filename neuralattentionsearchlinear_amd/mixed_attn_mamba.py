@@ -93,3 +93,95 @@ def nats_mixed_attn_mamba_chunk_inference(
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
         qk_l2norm=False, inference=True, op_type_last_chunk=op_type_last_chunk,
         n_tokens_in_current_block=n_tokens_in_current_block)
+
+
+def fused_recurrent_mamba_nats_fwd(q, k, v, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale,
+                                   initial_state, initial_state_in_current_block, output_final_state=True,
+                                   decay_for_non_mamba_blocks=False):
+    """The SSD recurrence token by token on a cached state, for tokens that continue the current selector block
+    (src/nats/ops/mamba/fused_recurrent.py with update_hs_for_each_iter=True).
+    -> (o, final_state or None, initial_state_in_current_block), the last updated in place when the tokens
+    complete the block."""
+    from . import _capi
+    N, T, H, K = q.shape
+    V = v.shape[-1]
+    if nats_block_types.shape[1] != 1:
+        raise AssertionError("the recurrent form only continues the current selector block: nats_block_types must hold one block")
+    HN = nats_block_types.shape[2]
+    dev = q.device
+    q, k, v = (t.contiguous() for t in (q, k, v))
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+    g = g.to(torch.float32).contiguous()
+    types = nats_block_types if nats_block_types.dtype in (torch.float32, torch.bfloat16) else nats_block_types.float()
+    types = types.contiguous()
+    if initial_state is not None:
+        initial_state = initial_state.to(torch.float32).contiguous()
+    if initial_state_in_current_block is None:
+        initial_state_in_current_block = (initial_state.clone() if initial_state is not None
+                                          else torch.zeros(N, H, K, V, dtype=torch.float32, device=dev))
+    if initial_state_in_current_block.dtype != torch.float32 or not initial_state_in_current_block.is_contiguous():
+        raise ValueError("initial_state_in_current_block must be a contiguous fp32 tensor (it is updated in place)")
+    if g_cumsum is not None:
+        g_cumsum = g_cumsum.to(torch.float32).reshape(N, H).contiguous()
+    if torch.is_tensor(n_tokens_in_current_block):
+        n_ptr, n_scalar = n_tokens_in_current_block.to(device=dev, dtype=torch.int32).contiguous(), 0
+    else:
+        n_ptr, n_scalar = None, int(n_tokens_in_current_block)
+    o = torch.empty(N, T, H, V, dtype=q.dtype, device=dev)
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
+    flags = _capi.DECAY_NON_LINEAR if decay_for_non_mamba_blocks else 0
+    rc = _capi.lib().natsl_mamba_recurrent_fwd(
+        _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), _capi.ptr(g_cumsum), _capi.ptr(initial_state),
+        _capi.ptr(initial_state_in_current_block), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype),
+        _capi.ptr(n_ptr), n_scalar, N, T, H, HN, K, V, int(nats_block_size), float(scale), flags, _capi.dtype_code(q.dtype),
+        _capi.stream_ptr(dev))
+    _capi.check(rc, "natsl_mamba_recurrent_fwd")
+    return o, ht, initial_state_in_current_block
+
+
+def nats_mixed_attn_mamba_recurrent(
+        q_attn: torch.Tensor, k_attn: torch.Tensor, v_attn: torch.Tensor,
+        q_lattn: torch.Tensor, k_lattn: torch.Tensor, v_lattn: torch.Tensor,
+        attn_msk: torch.Tensor,
+        initial_state_mamba: torch.Tensor,
+        initial_state_mamba_chunk_start: torch.Tensor,
+        g: torch.Tensor,
+        g_cumsum: torch.Tensor,
+        nats_block_types: torch.Tensor,
+        n_tokens_in_current_block: int = 0,
+        scale_attn=None, scale_lattn=None,
+        cu_seqlens=None, cu_seqlens_nats=None,
+        nats_block_size: int = 64,
+        ops_for_incomplete_chunks: str = 'all',
+        output_final_state_mamba: bool = False,
+        decay_for_non_mamba_blocks: bool = False,
+        incomplete_block_start_with_ht: bool = True,
+        use_g_for_attn: bool = False,
+):
+    """Decode step(s) of the Mamba hybrid layer (src/nats/ops/mixed_ops/mixed_attn_mamba.py:460-593).
+    -> (o_mamba, o_attn, final_state, initial_state_in_current_block).  As in the reference, scale_lattn
+    defaults to K**-0.5 here.  Built for 'all' and 'mamba' (the linear operator also runs on the incomplete
+    block); the 'attn' mode's block-wise state update (:516-591) is not."""
+    from .mixed_attn_gdn import masked_attention
+    if scale_attn is None:
+        scale_attn = k_attn.shape[-1] ** -0.5
+    if scale_lattn is None:
+        scale_lattn = k_lattn.shape[-1] ** -0.5
+    strategy = all_incomplete_ops[ops_for_incomplete_chunks]
+    if not strategy.mamba:
+        raise NotImplementedError("the recurrent (decode) operator is built for ops_for_incomplete_chunks 'all' and 'mamba' only")
+    if cu_seqlens is not None or cu_seqlens_nats is not None:
+        raise NotImplementedError("packed sequences are not supported by the recurrent (decode) operator")
+    if use_g_for_attn:
+        raise NotImplementedError("use_g_for_attn is not built")
+    if not q_lattn.is_cuda:
+        from . import _capi
+        raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
+    with torch.no_grad():
+        o_attn = masked_attention(q_attn, k_attn, v_attn, attn_msk, scale_attn)
+        o_mamba, final_state, start = fused_recurrent_mamba_nats_fwd(
+            q_lattn, k_lattn, v_lattn, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale_lattn,
+            initial_state_mamba, initial_state_mamba_chunk_start, output_final_state=True,
+            decay_for_non_mamba_blocks=decay_for_non_mamba_blocks)
+    return o_mamba, o_attn, final_state, start
