@@ -152,7 +152,7 @@ def main():
     ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
-    ap.add_argument("--cpu-batch", type=int, default=4, help="sequences of the slice timed on the CPU")
+    ap.add_argument("--cpu-batch", type=int, default=8, help="sequences of the slice timed on the CPU")
     ap.add_argument("--serial-branches", action="store_true",
                     help="force the softmax and the linear branch onto one stream, one after the other (default: the operator decides)")
     ap.add_argument("--concurrent-branches", action="store_true", help="force the softmax branch onto a side stream")
