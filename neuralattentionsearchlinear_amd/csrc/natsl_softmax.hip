@@ -338,7 +338,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   }
 
   // ---- global -> register -> LDS staging of one 64-key chunk -----------------------------
-  // 256 threads stage K (thread = row, 16-byte segments; stored row-major), 256 threads stage V
+  // 256 threads stage K (16-byte segments, whole rows per load instruction; stored row-major), 256 threads stage V
   // (thread = group of 4 keys x 8 value columns; the 4x8 block is transposed in registers and
   // stored as 8 rows of 4 keys).  With 4 waves every thread does both.
   static_assert(NTHREADS == 256 || NTHREADS == 512, "staging is written for 4 or 8 waves");
@@ -347,20 +347,24 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   const int st = SPLIT ? (tid & 255) : tid;
   const bool do_k = !SPLIT || tid < 256, do_v_role = !SPLIT || tid >= 256;
   u32x4 kreg[KL], vreg[4];
-  const int ld_row = st >> 2, ld_seg = st & 3;
+  // K: KSEGS lanes share a row, so one load instruction covers whole rows (full cache lines): a wave's loads
+  // return in order, and an instruction that touches many half-used lines holds back everything behind it
+  constexpr int KSEGS = DK / 8, KROWS = 256 / KSEGS;   // 16-byte segments per row; rows per pass (KL passes)
+  const int ld_row = st / KSEGS, ld_seg = st % KSEGS;
   constexpr int VSEGS = DV / 8;                    // 8-column segments per V row
   const int v_seg = (st & 3) + 4 * (st >> 6);      // 64 contiguous bytes per row per wave
   const int v_kg = (st >> 2) & 15;                 // keys 4*v_kg .. 4*v_kg+3
   const bool v_on = do_v_role && v_seg < VSEGS;
   // per-thread byte offsets inside a chunk; the chunk's base address is wave-uniform
   const unsigned k_off = (unsigned)(((size_t)ld_row * krow + ld_seg * 8) * sizeof(bf16_t));
+  const size_t k_pass = (size_t)KROWS * krow * sizeof(bf16_t);
   const unsigned v_off = (unsigned)(((size_t)(4 * v_kg) * vrow + 8 * v_seg) * sizeof(bf16_t));
   auto gload_full = [&](int ks) {
     // a chunk that lies wholly inside the sequence (every prior attention block): scalar base + lane offset
     if (do_k) {
       const char* kb = reinterpret_cast<const char*>(kp + (size_t)ks * krow) + k_off;
 #pragma unroll
-      for (int i = 0; i < KL; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(kb + 64 * i);
+      for (int i = 0; i < KL; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(kb + i * k_pass);
     }
     if (v_on) {
 #pragma unroll
@@ -372,10 +376,11 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
     // Rows past the end of the sequence are clamped to its last row: such keys are always hidden
     // by the causal rule (a valid query precedes them), so only finite values are needed there.
     if (do_k) {
-      const int tok = min(ks + ld_row, len - 1);
-      const u32x4* kr = reinterpret_cast<const u32x4*>(kp + (size_t)tok * krow);
 #pragma unroll
-      for (int i = 0; i < KL; ++i) kreg[i] = kr[ld_seg + 4 * i];
+      for (int i = 0; i < KL; ++i) {
+        const int tok = min(ks + ld_row + KROWS * i, len - 1);
+        kreg[i] = *reinterpret_cast<const u32x4*>(kp + (size_t)tok * krow + 8 * ld_seg);
+      }
     }
     if (v_on) {
 #pragma unroll
@@ -391,9 +396,9 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   };
   auto lstore = [&](int buf) {
     if (do_k) {
-      bf16_t* kd = Ks + (buf * 64 + ld_row) * KP;
+      bf16_t* kd = Ks + (buf * 64 + ld_row) * KP + 8 * ld_seg;
 #pragma unroll
-      for (int i = 0; i < KL; ++i) *reinterpret_cast<u32x4*>(kd + (ld_seg + 4 * i) * 8) = kreg[i];
+      for (int i = 0; i < KL; ++i) *reinterpret_cast<u32x4*>(kd + KROWS * i * KP) = kreg[i];
     }
     if (v_on) {
       bf16_t* vd = Vs + (buf * DV + 8 * v_seg) * TP + 4 * v_kg;
