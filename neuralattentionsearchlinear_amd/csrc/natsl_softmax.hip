@@ -163,9 +163,10 @@ NATSL_DEVICE void exp_pv(const bf16_t* VTb, f32x16 (&s)[2][NQ], f32x16 (&acc)[DV
       for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(e[2 * j], e[2 * j + 1]);
       PB[qt] = __builtin_bit_cast(bf16x8, w);
     }
-    const int kbase = 32 * kt + 16 * ss + 4 * hf;  // this lane's keys: kbase..kbase+3 and kbase+8..kbase+11
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
+      // this lane's keys: kbase..kbase+3 and kbase+8..kbase+11; 16-key groups of odd value tiles are stored swapped
+      const int kbase = 16 * (sidx ^ (vt & 1)) + 4 * hf;
       const bf16_t* vr = VTb + (32 * vt + l32) * TP + kbase;
       const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
       const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
@@ -236,9 +237,9 @@ NATSL_DEVICE void pv_half(const bf16_t* VTb, const int kt, const bf16x8 (&PB)[2]
   const int l32 = lane & 31, hf = lane >> 5;
 #pragma unroll
   for (int ss = 0; ss < 2; ++ss) {
-    const int kbase = 32 * kt + 16 * ss + 4 * hf;
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
+      const int kbase = 16 * ((2 * kt + ss) ^ (vt & 1)) + 4 * hf;  // 16-key groups of odd value tiles are stored swapped
       const bf16_t* vr = VTb + (32 * vt + l32) * TP + kbase;
       const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
       const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
@@ -352,9 +353,12 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
   constexpr int KSEGS = DK / 8, KROWS = 256 / KSEGS;   // 16-byte segments per row; rows per pass (KL passes)
   const int ld_row = st / KSEGS, ld_seg = st % KSEGS;
   constexpr int VSEGS = DV / 8;                    // 8-column segments per V row
-  const int v_seg = (st & 3) + 4 * (st >> 6);      // 64 contiguous bytes per row per wave
-  const int v_kg = (st >> 2) & 15;                 // keys 4*v_kg .. 4*v_kg+3
-  const bool v_on = do_v_role && v_seg < VSEGS;
+  // V: 8 lanes share 128 bytes (a full line) of a row; a thread owns keys 4*v_kg .. 4*v_kg+3 of one 8-column
+  // segment.  In the transposed tile the 16-key groups of value rows with bit 5 set are swapped pairwise
+  // (group ^ 1), which keeps the 8-byte transposed stores of one instruction on distinct banks.
+  const int v_seg = VSEGS == 16 ? (st & 7) + 8 * ((st >> 6) & 1) : (st & 7);
+  const int v_kg = VSEGS == 16 ? ((st >> 3) & 7) + 8 * (st >> 7) : (st >> 3);
+  const bool v_on = do_v_role && v_seg < VSEGS && v_kg < 16;
   // per-thread byte offsets inside a chunk; the chunk's base address is wave-uniform
   const unsigned k_off = (unsigned)(((size_t)ld_row * krow + ld_seg * 8) * sizeof(bf16_t));
   const size_t k_pass = (size_t)KROWS * krow * sizeof(bf16_t);
@@ -401,7 +405,7 @@ __global__ __launch_bounds__(64 * NWAVES, (NQ == 1 && NWAVES == 4) ? 2 : 1) void
       for (int i = 0; i < KL; ++i) *reinterpret_cast<u32x4*>(kd + KROWS * i * KP) = kreg[i];
     }
     if (v_on) {
-      bf16_t* vd = Vs + (buf * DV + 8 * v_seg) * TP + 4 * v_kg;
+      bf16_t* vd = Vs + (buf * DV + 8 * v_seg) * TP + 4 * (v_kg ^ (4 * ((v_seg >> 2) & 1)));
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         // value columns 2d (low halves) and 2d+1 (high halves) of the four keys
