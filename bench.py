@@ -27,6 +27,10 @@ WORKLOADS = {
 DECODE_WORKLOADS = {
     "decode_gdn_B8_ctx8192_H16_d128_p25": dict(B=8, ctx=8192, H=16, K=128, V=128, p_attn=0.25, block=64, n_in_block=17),
 }
+# cache hand-off after a prefill: keep the attention-typed blocks of every (sequence, head); not the headline metric
+CACHE_WORKLOADS = {
+    "kv_compact_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
+}
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 
@@ -144,12 +148,59 @@ def bench_decode(args):
                       algorithmic_bytes=nbytes, note="whole step incl. launch overheads of two kernels"))))
 
 
+def bench_kv_compact(args):
+    """The K/V hand-off of one prefill into the generation cache: gather the attention-typed blocks of every
+    (sequence, head) into a buffer sized for them.  Pure byte movement: kept bytes read once and written once."""
+    import torch
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd.cache import NAtSLayerCache
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    w = CACHE_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    B, T, H, K, V, block = w["B"], w["T"], w["H"], w["K"], w["V"], w["block"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    k = torch.randn(B, T, H, K, device=dev, generator=g).bfloat16()
+    v = torch.randn(B, T, H, V, device=dev, generator=g).bfloat16()
+    attn = (torch.rand(B, T // block, H, device=dev, generator=g) < w["p_attn"]).float()
+    types = torch.stack([attn, 1 - attn], -1).bfloat16()
+    kept = int(attn.sum())
+    nbytes = 2 * kept * block * (K + V) * 2                    # kept blocks read once and written once
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    times = []
+    for i in range(args.warmup + args.steps):
+        cache = NAtSLayerCache(nats_block_size=block, op_for_incomplete_chunk="all")
+        cache.update_attn_cache((k, v), types)
+        cache._compact(types, (k, v), T // block, 0)           # allocates the cache, then one kernel launch: warm the allocator first
+        torch.cuda.synchronize()
+        dst_k, dst_v = cache.attn_k, cache.attn_v
+        ev[0].record()
+        rc = _capi.lib().natsl_kv_compact(_capi.ptr(k), _capi.ptr(v), T, 0, _capi.ptr(dst_k), _capi.ptr(dst_v), dst_k.shape[1],
+                                          _capi.ptr(types), _capi.BF16, None, B, H, H, K, V, _capi.BF16, block, T // block,
+                                          T // block, -1, 0, _capi.stream_ptr(dev))
+        ev[1].record()
+        _capi.check(rc, "natsl_kv_compact")
+        torch.cuda.synchronize()
+        if i >= args.warmup:
+            times.append(ev[0].elapsed_time(ev[1]))
+    ms = sum(times) / len(times)
+    print(json.dumps(dict(
+        metric="prefill K/V hand-off into the generation cache, tokens/sec @T=8192,H=16,d=128 bf16", value=B * T / (ms * 1e-3),
+        unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak",
+        vs_baseline=None, dtype="u8", data="synthetic", config=dict(workload=args.workload, **w, kept_blocks=kept,
+                                                                   cache_tokens=int(dst_k.shape[1])),
+        roofline=dict(bound="hbm", kernel="kv_compact_kernel", achieved=nbytes / (ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s",
+                      frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, traffic=None, algorithmic_bytes=nbytes, launch_ms=ms))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS))
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
     ap.add_argument("--cpu-batch", type=int, default=8, help="sequences of the slice timed on the CPU")
@@ -167,6 +218,8 @@ def main():
 
     if args.workload in DECODE_WORKLOADS:
         return bench_decode(args)
+    if args.workload in CACHE_WORKLOADS:
+        return bench_kv_compact(args)
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn

@@ -183,6 +183,23 @@ int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uin
                           int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
                           size_t workspace_bytes, natsl_stream_t stream);
 
+/* KV cache of the softmax branch: keep the attention-typed blocks of a region of new tokens, per (sequence, kv
+ * head), back to back behind the blocks already kept, and put the tokens of the incomplete last block at block
+ * index tail_dst (the same for every head; pass -1 when the region ends on a block boundary).
+ * src_k/src_v [B, src_tokens, HKV, K|V] hold the region from block src_block0 on: NB blocks of `block` tokens,
+ * the first n_complete complete (n_complete = NB, or NB-1 with an incomplete block of tail_tokens tokens).
+ * dst_k/dst_v [B, dst_tokens, HKV, K|V] is the cache; it may be the source itself (in place: same pointers and
+ * sizes), since a kept block never moves towards the back.  types [B, NB, HN, 2] (f32 or bf16): column 0 equal to
+ * 1 marks an attention-typed block; kv head h follows selector head h/(HKV/HN).  n_before int64 [B, HN] = blocks
+ * already kept per (sequence, selector head), NULL = none.  The caller sizes the destination for the largest new
+ * count (stores past dst_tokens are dropped, never issued).  The rest of the block at tail_dst is zero filled when
+ * the block is moved or copied.
+ * Replaces the gather/scatter at src/nats/models/utils.py:509-588 (NAtSLayerCache.update). */
+int natsl_kv_compact(const void* src_k, const void* src_v, long long src_tokens, int src_block0, void* dst_k, void* dst_v,
+                     long long dst_tokens, const void* types, int types_dtype, const int64_t* n_before, int B, int HKV,
+                     int HN, int K, int V, int dtype, int block, int NB, int n_complete, int tail_dst, int tail_tokens,
+                     natsl_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

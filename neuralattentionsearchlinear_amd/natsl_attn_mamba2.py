@@ -1,6 +1,7 @@
 """Mamba2-SSD / softmax hybrid token mixer with the forward signature, returns and parameter names of
 the reference layer (src/nats/layers/natsl_attn_mamba2.py:100-599).  Same scope as the Gated-DeltaNet
-layer: forward only, no cache, no decode."""
+layer: forward only; with a cache, one chunked prefill on the empty cache and then decode steps of fewer
+than 64 tokens."""
 from __future__ import annotations
 
 import math
@@ -11,7 +12,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import nats_util
-from .mixed_attn_mamba import nats_mixed_attn_mamba, nats_mixed_attn_mamba_chunk_inference
+from .cache import NAtSLayerCache
+from .mixed_attn_mamba import (nats_mixed_attn_mamba, nats_mixed_attn_mamba_chunk_inference,
+                               nats_mixed_attn_mamba_recurrent)
 from .modules import FusedMultiInputRMSNormGated, L2Norm, RMSNorm, ShortConvolution
 
 
@@ -80,43 +83,73 @@ class NeuralAttentionSearchLinearAttnMamba(nn.Module):
         self.o_proj = nn.Linear(self.value_dim, hidden_size, bias=False)
         self.attn_fraction = torch.zeros(1)
 
-    def select_ops(self, hidden_states: torch.Tensor, cu_seqlens=None):
+    def select_ops(self, hidden_states: torch.Tensor, cu_seqlens=None, force_last_block: bool = True):
         B, _, dim = hidden_states.shape
         pooled = nats_util.mean_pooling(hidden_states.unsqueeze(-2), self.nats_block_size, cu_seqlens=cu_seqlens)
         logits = self.nats_layer(pooled.view(B, pooled.shape[1], dim)).unflatten(-1, (self.num_nats_head, self.n_ops))
         types, n_blocks = nats_util.hard_select(logits, force_last_block=False)
         last = types[:, -1].clone()
-        n_blocks = n_blocks + (1 - last.to(torch.int32))
-        types[:, -1] = 1
+        if force_last_block:
+            n_blocks = n_blocks + (1 - last.to(torch.int32))
+            types[:, -1] = 1
         return types, n_blocks, last
+
+    def _layer_cache(self, cache_params) -> Optional[NAtSLayerCache]:
+        """The layer's own cache in cache_params.nats_cache, created on first use (reference :332-343)."""
+        if cache_params is None:
+            return None
+        if self.layer_idx not in cache_params.nats_cache:
+            cache_params.add_natsl_layer_cache(self.layer_idx, 0, n_tokens_in_nats_block=0, n_attn_blocks=None,
+                                               nats_block_size=self.nats_block_size,
+                                               op_for_incomplete_chunk=self.ops_for_incomplete_chunks)
+        return cache_params.nats_cache[self.layer_idx]
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, cache_params=None,
                 use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False, **kwargs):
         if attention_mask is not None:
             assert len(attention_mask.shape) == 2, "Expected attention_mask as a 0-1 matrix with shape [batch_size, seq_len]"
-        if cache_params is not None:
-            raise NotImplementedError("the NAtS KV/state cache (decode and chunked prefill continuation) is not built")
         B, q_len, _ = hidden_states.shape
-        if q_len < 64:
-            raise NotImplementedError("the token-recurrent decode path (q_len < 64) is not built")
+        mode = 'fused_recurrent' if q_len < 64 else self.mode                  # reference :328
+        if self.training:
+            assert mode == 'chunk', "Only chunk mode is supported in training."
         cu_seqlens = kwargs.get('cu_seqlens', None)
-        types, n_nats_blocks, last_type = self.select_ops(hidden_states, cu_seqlens)
+        cache = self._layer_cache(cache_params)
+        if cache is not None:
+            use_cache = True
+        if cache is None and mode != 'chunk':
+            raise ValueError("fewer than 64 tokens are decoded on a cache: pass cache_params")
+        if cache is not None and mode == 'chunk' and cache.n_observed_tokens > 0:
+            raise NotImplementedError("a chunked forward that continues a non-empty cache is not built: prefill once, then "
+                                      "decode in steps of fewer than 64 tokens")
+        if cache is not None and cu_seqlens is not None:
+            raise NotImplementedError("packed sequences are not supported together with a cache")
 
-        def conv_or_act(x, conv):
+        selector_input = cache.update_attn_types(input_hidden_states=hidden_states) if cache is not None else hidden_states
+        if selector_input is not None:
+            raw_types, _, _ = self.select_ops(selector_input, cu_seqlens, force_last_block=False)
+        else:
+            raw_types = torch.ones(B, 1, self.num_nats_head, self.n_ops, device=hidden_states.device, dtype=hidden_states.dtype)
+
+        conv_states = cache.conv_state if cache is not None and cache.conv_state is not None else (None, None, None)
+        new_conv_states = []
+
+        def conv_or_act(x, conv, state):
             if self.use_short_conv:
-                return conv(x=x, cache=None, output_final_state=False, cu_seqlens=cu_seqlens)[0]
+                y, final = conv(x=x, cache=state, output_final_state=bool(use_cache), cu_seqlens=cu_seqlens)
+                new_conv_states.append(final)
+                return y
             return F.silu(x)
 
         if self.attn_with_short_conv:
-            q = conv_or_act(self.q_proj(hidden_states), getattr(self, 'q_conv1d', None))
-            k = conv_or_act(self.k_proj(hidden_states), getattr(self, 'k_conv1d', None))
-            v = conv_or_act(self.v_proj(hidden_states), getattr(self, 'v_conv1d', None))
+            q = conv_or_act(self.q_proj(hidden_states), getattr(self, 'q_conv1d', None), conv_states[0])
+            k = conv_or_act(self.k_proj(hidden_states), getattr(self, 'k_conv1d', None), conv_states[1])
+            v = conv_or_act(self.v_proj(hidden_states), getattr(self, 'v_conv1d', None), conv_states[2])
             q_attn, k_attn, v_attn = q, k, v
         else:
             q_attn, k_attn, v_attn = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
-            q = conv_or_act(q_attn, getattr(self, 'q_conv1d', None))
-            k = conv_or_act(k_attn, getattr(self, 'k_conv1d', None))
-            v = conv_or_act(v_attn, getattr(self, 'v_conv1d', None))
+            q = conv_or_act(q_attn, getattr(self, 'q_conv1d', None), conv_states[0])
+            k = conv_or_act(k_attn, getattr(self, 'k_conv1d', None), conv_states[1])
+            v = conv_or_act(v_attn, getattr(self, 'v_conv1d', None), conv_states[2])
         o_weights = self.nats_out_weights_layer(q).unflatten(-1, (self.num_attn_heads, self.n_ops)).softmax(-1)
         q, k = (x.unflatten(-1, (-1, self.head_k_dim)) for x in (q, k))
         v = v.unflatten(-1, (-1, self.head_v_dim))
@@ -131,19 +164,46 @@ class NeuralAttentionSearchLinearAttnMamba(nn.Module):
         v = (v * dt.unsqueeze(-1)).to(v.dtype)                 # the attention view keeps the un-scaled v (:391-393, :473)
         g = -self.A_log.float().exp() * dt
 
-        self.attn_fraction = (n_nats_blocks.float()[..., 0] / types.shape[1]).mean(0).detach()
+        state, state_block_start, g_cumsum = None, None, None
+        k_new, v_new, g_new = k_attn, v_attn, g
+        if cache is not None:
+            k_attn, v_attn = cache.update_attn_cache((k_attn, v_attn), nats_block_types=raw_types)
+            k, v, _, g = cache.update_lattn_cache((k, v), None, g, mode, self.ops_for_incomplete_chunks)
+            state, state_block_start, g_cumsum = cache.recurrent_state, cache.recurrent_state_block_start, cache.g_cumsum
+
         common = dict(q_attn=q_attn, k_attn=k_attn, v_attn=v_attn, q_lattn=q, k_lattn=k, v_lattn=v, g=g,
-                      nats_block_types=types, n_nats_blocks=n_nats_blocks, scale_attn=k_attn.shape[-1] ** -0.5, scale_lattn=1,
+                      scale_attn=k_attn.shape[-1] ** -0.5, scale_lattn=1,
                       cu_seqlens=cu_seqlens, cu_seqlens_nats=None, nats_block_size=self.nats_block_size,
                       ops_for_incomplete_chunks=self.ops_for_incomplete_chunks, output_final_state_mamba=bool(use_cache),
                       incomplete_block_start_with_ht=self.incomplete_block_start_with_ht,
                       decay_for_non_mamba_blocks=self.decay_for_non_mamba_blocks, use_g_for_attn=False)
-        if self.training:
-            o_lin, o_attn, self.last_recurrent_state = nats_mixed_attn_mamba(initial_state_mamba=None, **common)
+        if mode == 'chunk':
+            types = raw_types.clone()
+            last_type = types[:, -1].clone()
+            types[:, -1] = 1
+            n_nats_blocks = types.to(torch.int32).sum(1)
+            self.attn_fraction = (n_nats_blocks.float()[..., 0] / types.shape[1]).mean(0).detach()
+            if self.training:
+                o_lin, o_attn, state = nats_mixed_attn_mamba(initial_state_mamba=state, nats_block_types=types,
+                                                             n_nats_blocks=n_nats_blocks, **common)
+                state_block_start = None
+            else:
+                o_lin, o_attn, state, state_block_start = nats_mixed_attn_mamba_chunk_inference(
+                    initial_state_mamba_start=state_block_start, nats_block_types=types, n_nats_blocks=n_nats_blocks,
+                    op_type_last_chunk=last_type if k.shape[1] % self.nats_block_size == 0 else None, **common)
         else:
-            o_lin, o_attn, self.last_recurrent_state, self.last_block_start_state = nats_mixed_attn_mamba_chunk_inference(
-                initial_state_mamba_start=None,
-                op_type_last_chunk=last_type if q_len % self.nats_block_size == 0 else None, **common)
+            attn_msk = cache.generate_msk(n_data=q_len, nats_block_types=raw_types,
+                                          compute_incomplete_chunk=self.ops_for_incomplete_chunks != 'mamba')
+            o_lin, o_attn, state, state_block_start = nats_mixed_attn_mamba_recurrent(
+                attn_msk=attn_msk, initial_state_mamba=state, initial_state_mamba_chunk_start=state_block_start,
+                g_cumsum=g_cumsum, nats_block_types=raw_types, n_tokens_in_current_block=cache._n_tokens_in_nats_block, **common)
+        self.last_recurrent_state, self.last_block_start_state = state, state_block_start
+
+        if cache is not None:
+            cache.update(recurrent_state=state, recurrent_state_block_start=state_block_start, attn_state=(k_new, v_new),
+                         conv_state=tuple(new_conv_states) if self.use_short_conv else None, nats_block_types=raw_types,
+                         l_attn_state=(k, v), g=g_new, n_new_tokens=q_len)
+
         gate = self.g_proj(hidden_states).unflatten(-1, (-1, self.head_v_dim))
         o = self.o_norm(o_lin.reshape(o_attn.shape), o_attn, gate.reshape(o_attn.shape), o_weights)
         return self.o_proj(o.flatten(-2))

@@ -6,4 +6,4 @@ smoke check and the benchmark's CPU-baseline leg), never the thing measured or
 shipped.  Every function cites the reference file:line it restates; the
 reference itself is Triton-only and cannot run on a CPU.
 """
-from . import routing, softmax_branch, linear_branch, mixed, norm_gate, layer, decode  # noqa: F401
+from . import routing, softmax_branch, linear_branch, mixed, norm_gate, layer, decode, cache  # noqa: F401

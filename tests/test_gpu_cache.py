@@ -1,0 +1,178 @@
+"""GPU parity of the K/V cache (natsl_kv_compact behind NAtSLayerCache) against oracle/cache.py, bit-exact, and
+of generation through the hybrid layers (one prefill, then decode steps) against the same layer's forward
+over the whole sequence."""
+import pytest
+import torch
+
+from oracle import cache as C
+from tests.test_gpu_layers import _layer_case
+from tests._util import max_abs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+def _types(B, NB, HN, seed, p_attn=0.5, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    a = (torch.rand(B, NB, HN, generator=g) < p_attn).float()
+    return torch.stack([a, 1 - a], -1).to(dtype)
+
+
+def _feed(cache, k, v, ty, pieces, bs):
+    """Drive the cache the way the layers do: update_attn_cache, (the operators), update."""
+    t = 0
+    views = []
+    for n in pieces:
+        first_block = (t - t % bs) // bs
+        total = t % bs + n
+        types = ty[:, first_block:first_block + -(-total // bs)] if total >= bs else torch.ones_like(ty[:, :1])
+        kk, vv = k[:, t:t + n].contiguous(), v[:, t:t + n].contiguous()
+        views.append(cache.update_attn_cache((kk, vv), types))
+        cache.update(attn_state=(kk, vv), nats_block_types=types, n_new_tokens=n)
+        t += n
+    return views
+
+
+def _check(cache, want, bs, G, zero_tail=True):
+    nmax = want['n_max']
+    assert cache.n_attn_blocks_max == nmax and cache._n_tokens_in_nats_block == want['n_tail']
+    assert cache.n_attn_tokens_max == nmax * bs + want['n_tail']
+    assert torch.equal(cache.n_attn_blocks.cpu(), want['n_attn_blocks'])
+    valid = cache.valid_attn_tokens.cpu()
+    assert torch.equal(valid[:, :nmax + 1], want['valid']) and not bool(valid[:, nmax + 1:].any())
+    # only what the validity flags expose is compared: dropped blocks may leave stale tokens behind
+    vis = want['valid'].repeat_interleave(bs, 1).repeat_interleave(G, 2)                         # [B, tokens, HKV]
+    if not zero_tail:
+        vis[:, nmax * bs + want['n_tail']:] = False            # decode steps reuse dropped blocks' memory for the incomplete block
+    for got, ref in ((cache.attn_k, want['keys']), (cache.attn_v, want['values'])):
+        got = got[:, :(nmax + 1) * bs].cpu()
+        assert torch.equal(got * vis.unsqueeze(-1), ref * vis.unsqueeze(-1))
+    if want['n_tail'] and zero_tail:
+        tail = cache.attn_k[:, nmax * bs + want['n_tail']:(nmax + 1) * bs]
+        assert float(tail.float().abs().sum()) == 0, "the incomplete block must be zero padded"
+
+
+@pytest.mark.parametrize("dtype,tdtype", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("T,K,V,HKV,HN,bs", [(1078, 64, 128, 8, 4, 64), (1728, 128, 128, 4, 4, 64), (64, 64, 64, 2, 1, 64),
+                                             (40, 64, 64, 2, 2, 64), (1100, 128, 64, 4, 2, 256), (640, 256, 512, 2, 2, 64)])
+def test_prefill_compaction(T, K, V, HKV, HN, bs, dtype, tdtype):
+    from neuralattentionsearchlinear_amd.cache import NAtSLayerCache
+    B = 3
+    g = torch.Generator().manual_seed(T + K)
+    k, v = torch.randn(B, T, HKV, K, generator=g).to(dtype), torch.randn(B, T, HKV, V, generator=g).to(dtype)
+    ty = _types(B, -(-T // bs), HN, T, dtype=tdtype)
+    cache = NAtSLayerCache(nats_block_size=bs, op_for_incomplete_chunk='all')
+    (kv, vv), = _feed(cache, k.to(DEV), v.to(DEV), ty.to(DEV), [T], bs)
+    assert kv.shape[1] == T                                             # the first forward attends to its own keys
+    _check(cache, C.whole_sequence(k, v, ty.float(), bs), bs, HKV // HN)
+    assert cache.attn_k.shape[1] <= (int(cache.n_attn_blocks_max) + 2) * bs, "the cache must not keep the dropped blocks"
+
+
+@pytest.mark.parametrize("T1,T2,step", [(1728, 45, 1), (1777, 195, 1), (1078, 130, 7), (10, 200, 1), (0, 150, 3), (640, 640, 63)])
+def test_pieces_equal_whole(T1, T2, step):
+    """One prefill and then decode steps reach the cache of the whole sequence
+    (the reference states this at src/nats/models/utils.py:910-1047)."""
+    from neuralattentionsearchlinear_amd.cache import NAtSLayerCache
+    B, HKV, HN, K, V, bs = 2, 4, 2, 64, 128, 64
+    T = T1 + T2
+    g = torch.Generator().manual_seed(T)
+    k, v = torch.randn(B, T, HKV, K, generator=g).bfloat16(), torch.randn(B, T, HKV, V, generator=g).bfloat16()
+    ty = _types(B, -(-T // bs), HN, T1 + 1, dtype=torch.bfloat16)
+    if T >= 30 * bs:
+        ty[:, 29, :, 0] = 0                                             # as the reference's check does (:997)
+    pieces, t = ([T1] if T1 else []), T1
+    while t < T:                                                        # decode steps never cross a block boundary
+        n = min(step, T - t, bs - t % bs)
+        pieces.append(n); t += n
+    cache = NAtSLayerCache(nats_block_size=bs, op_for_incomplete_chunk='all')
+    kd, vd = k.to(DEV), v.to(DEV)
+    views = _feed(cache, kd, vd, ty.to(DEV), pieces, bs)
+    want = C.whole_sequence(k, v, ty.float(), bs)
+    _check(cache, want, bs, HKV // HN, zero_tail=False)
+    # what the last step's attention saw: the kept blocks, the incomplete block and its own token(s)
+    kv, _ = views[-1]
+    before = C.whole_sequence(k[:, :T - pieces[-1]], v[:, :T - pieces[-1]], ty[:, :-(-(T - pieces[-1]) // bs) or 1].float(), bs) \
+        if T - pieces[-1] > 0 else None
+    if before is not None and len(pieces) > 1:
+        assert kv.shape[1] == before['n_max'] * bs + before['n_tail'] + pieces[-1]
+        assert torch.equal(kv[:, -pieces[-1]:].cpu(), k[:, T - pieces[-1]:])
+
+
+def test_mask_of_the_next_token():
+    from neuralattentionsearchlinear_amd.cache import NAtSLayerCache
+    B, HKV, HN, K, bs, T = 2, 4, 2, 64, 64, 64 * 6 + 9
+    g = torch.Generator().manual_seed(9)
+    k = torch.randn(B, T + 3, HKV, K, generator=g).bfloat16()
+    ty = _types(B, 7, HN, 2)
+    cache = NAtSLayerCache(nats_block_size=bs, op_for_incomplete_chunk='all')
+    kd = k.to(DEV)
+    _feed(cache, kd[:, :T], kd[:, :T], ty.to(DEV), [T], bs)
+    want = C.whole_sequence(k[:, :T], k[:, :T], ty, bs)
+    one = torch.ones(B, 1, HN, 2, device=DEV)
+    kv, _ = cache.update_attn_cache((kd[:, T:T + 1].contiguous(), kd[:, T:T + 1].contiguous()), one)
+    m = cache.generate_msk(1, one, True)
+    assert m.dtype == torch.bool and m.shape[-1] == kv.shape[1]
+    assert torch.equal(m.cpu(), C.next_query_mask(want, bs))
+    cache.update(attn_state=(kd[:, T:T + 1], kd[:, T:T + 1]), nats_block_types=one, n_new_tokens=1)
+    # three tokens at once, still inside the block: kept blocks, then causal inside the block
+    kv, _ = cache.update_attn_cache((kd[:, T + 1:T + 3].contiguous(), kd[:, T + 1:T + 3].contiguous()), one)
+    m = cache.generate_msk(2, one, True).cpu()
+    assert m.shape == (B, HN, 2, kv.shape[1])
+    base = C.next_query_mask(want, bs)[:, :, 0]                           # columns up to token T included
+    assert torch.equal(m[:, :, 0, :-1], torch.cat([base, torch.ones(B, HN, 1, dtype=torch.bool)], -1))
+    assert not bool(m[:, :, 0, -1].any()) and bool(m[:, :, 1, -2:].all())
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+@pytest.mark.parametrize("T0,T", [(320, 420), (266, 400), (64, 130)])
+def test_layer_generation_matches_whole_forward(kind, T0, T):
+    """Prefill T0 tokens with a cache, decode up to T token by token (two tokens at a time where the block allows
+    it): every output must match the layer's forward over the first T0 tokens resp. the whole sequence at the same
+    positions; the selector decisions of the two runs must be identical."""
+    from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
+    layer, cfg, w, _ = _layer_case(kind)
+    layer.layer_idx = 0
+    layer = layer.to(DEV).to(torch.bfloat16).eval()
+    bs = layer.nats_block_size
+    torch.manual_seed(T)
+    x = torch.randn(2, T, 256).to(DEV).to(torch.bfloat16)
+    first = lambda out: out[0] if isinstance(out, tuple) else out
+    with torch.no_grad():
+        whole = first(layer(x))
+        types_whole, _, _ = layer.select_ops(x, force_last_block=False)
+        holder = NAtSCache() if kind == 'gdn' else NAtSMamba2Cache()
+        kw = dict(past_key_values=holder, use_cache=True) if kind == 'gdn' else dict(cache_params=holder, use_cache=True)
+        outs = [first(layer(x[:, :T0], **kw))]
+        t = T0
+        while t < T:
+            n = 2 if (t % bs) in (10, 20) and t + 2 <= T else 1
+            outs.append(first(layer(x[:, t:t + n], **kw)))
+            t += n
+    cache = holder[0] if kind == 'gdn' else holder.nats_cache[0]
+    # same selector decisions: the kept-block counts follow from them
+    n_complete = T // bs
+    want_counts = (types_whole[:, :n_complete, :, 0] == 1).sum(1)
+    assert torch.equal(cache.n_attn_blocks, want_counts), "the cached run typed a block differently from the whole forward"
+    assert cache.n_observed_tokens == T and cache._n_tokens_in_nats_block == T % bs
+    got = torch.cat(outs, 1).float()
+    # the prefill part is compared with a forward over exactly those tokens only where no later token matters:
+    # a whole-sequence forward types complete blocks only, so positions in blocks completed by the prefill agree
+    ma, rl = max_abs(got[:, T0:], whole[:, T0:].float()), rel_l2(got[:, T0:], whole[:, T0:].float())
+    assert rl <= 2e-2, f"decoded tokens: rel-L2 {rl:.3e}, max-abs {ma:.3e}"
+    rl0 = rel_l2(got[:, :T0], whole[:, :T0].float())
+    assert rl0 <= 2e-2, f"prefilled tokens: rel-L2 {rl0:.3e}"
+
+
+def test_layer_rejects_what_the_cache_cannot_do():
+    from neuralattentionsearchlinear_amd.cache import NAtSCache
+    layer, cfg, w, x = _layer_case('gdn')
+    layer.layer_idx = 0
+    layer = layer.to(DEV).to(torch.bfloat16).eval()
+    xd = x.to(DEV).bfloat16()
+    cache = NAtSCache()
+    with torch.no_grad():
+        layer(xd[:, :100], past_key_values=cache, use_cache=True)
+        with pytest.raises(NotImplementedError):
+            layer(xd[:, 100:200], past_key_values=cache, use_cache=True)      # a second chunked forward
+        with pytest.raises(NotImplementedError):
+            layer(xd[:, 100:140], past_key_values=cache, use_cache=True)      # 36 + 40 tokens cross a block boundary

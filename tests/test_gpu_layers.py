@@ -81,7 +81,5 @@ def test_layer_forward(kind, train):
 def test_layer_rejects_unbuilt_paths():
     layer, cfg, w, x = _layer_case('gdn')
     layer = layer.to(DEV).to(torch.bfloat16).eval()
-    with pytest.raises(NotImplementedError):
-        layer(x[:, :32].to(DEV).bfloat16())                       # decode
-    with pytest.raises(NotImplementedError):
-        layer(x.to(DEV).bfloat16(), past_key_values=object())     # cache
+    with pytest.raises(ValueError):
+        layer(x[:, :32].to(DEV).bfloat16())                       # decoding needs a cache
