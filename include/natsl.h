@@ -103,6 +103,23 @@ int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* 
                              int V, int TN, int block, float scale, int same_block_visible, int dtype,
                              const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
 
+
+/* Backward of the softmax branch: dq [B,T,HQ,K], dk [B,T,HKV,K], dv [B,T,HKV,V] (bf16, summed over the query heads of
+ * a kv head) and dnats fp32 [B,TN,HQ], which must be ZERO on entry: per block typed "attention" and query head, the sum
+ * of the score gradients dS = P (dP - delta) over (keys of the block) x (queries of later blocks), i.e. the gradient
+ * with respect to a bias on that block's scores as later blocks see them; blocks not typed attention keep 0 (the
+ * reference's default compute_dnats_for_invalid_blocks_attn = False).  The caller sums dnats over the query heads of a
+ * selector head.  o, lse are the forward's outputs, d_o the gradient of o.  workspace: natsl_softmax_bwd_workspace_bytes()
+ * bytes (delta = rowsum(d_o * o)).  Regular batches only (no packed-sequence table yet).
+ * Replaces parallel_attn_nats_bwd (src/nats/ops/attns/attns.py:1562-1759; kernels :357-372, :383-708, :719-983) as
+ * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:226-243. */
+size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ);
+int natsl_softmax_sparse_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* d_o,
+                             void* dq, void* dk, void* dv, float* dnats, const void* types, int types_dtype,
+                             const int32_t* nats_block_indices, const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV,
+                             int HN, int K, int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                             void* workspace, size_t workspace_bytes, natsl_stream_t stream);
+
 /* Bytes of scratch the two linear-branch entry points need for `total_chunks` 64-token chunks
  * (sum over sequences of ceil(len/64)) and H heads. */
 size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H);

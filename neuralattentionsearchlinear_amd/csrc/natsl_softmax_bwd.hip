@@ -1,0 +1,548 @@
+// Backward of the softmax branch for gfx950 (first version: correct and on the matrix cores, not yet pipelined).
+//
+//   delta_kernel   delta[t] = sum_v dO[t,v] O[t,v]                                  (attns.py:357-372)
+//   dq_kernel      one workgroup per tile of 128 queries, the forward's walk over the visible key chunks:
+//                  S^T = K Q^T, P = exp2(S c - lse), dP^T = V dO^T, dS = P (dP - delta), dQ^T += K^T dS^T (attns.py:383-708)
+//   dkdv_kernel    one workgroup per 64-key chunk of a kv head, walking the query chunks that see it (the rest of its own
+//                  block, and every later chunk when the block is typed attention), for every query head of the group:
+//                  S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS, dnats += sum dS over later blocks (attns.py:719-983)
+//
+// Layouts follow the forward kernel: the stationary operand of a workgroup (Q, dO there; K, V here) sits in registers
+// as the B operand (lane = its row), the streamed tiles are row-major in LDS, the accumulators' own layout is the B
+// operand of the second product, and the transposed A operands (K^T, dO^T, Q^T) come out of the row-major tiles with
+// the transposing LDS read.
+#include "natsl_device.h"
+#include "natsl_host.h"
+
+namespace natsl {
+
+struct SoftmaxBwdParams {
+  const bf16_t *q, *k, *v, *o, *dout;
+  const float* lse;
+  bf16_t *dq, *dk, *dv;
+  float* dnats;   // [B, TN, HQ], zero on entry
+  float* delta;   // [B, T, HQ] workspace
+  const void* types;
+  int types_dtype;
+  const int32_t* idx;
+  const int32_t* nblk;
+  int B, T, HQ, HKV, HN, TN, block;
+  float scale, scale_log2;
+  int same_block;
+};
+
+NATSL_DEVICE bool bwd_type_is_one(const void* types, int dtype, size_t i) {
+  float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i] : bf16_to_f32(reinterpret_cast<const bf16_t*>(types)[i]);
+  return rintf(x) == 1.0f;
+}
+
+constexpr int BWD_MAX_LDS_LIST = 2048;
+
+// A operand of a 32x32x16 product taken TRANSPOSED from a row-major LDS tile: A[m = lane%32][k-slot (hf, j)] =
+// tile[row_base + 8(j/4) + 4hf + j%4][col_base + m].  ds_read_b64_tr_b16: within each group of 16 lanes, lane i supplies
+// the address of a 4-element row R_i and receives { R_{4j + i/4}[i%4] : j < 4 }.
+NATSL_DEVICE bf16x8 tr_operand(const bf16_t* tile, const int pitch, const int row_base, const int col_base, const int lane) {
+  const int i16 = lane & 15, colsel = 16 * ((lane >> 4) & 1), hf = lane >> 5;
+  const bf16_t* p = tile + (row_base + 4 * hf + (i16 >> 2)) * pitch + col_base + colsel + 4 * (i16 & 3);
+  return join4(lds_tr4(p), lds_tr4(p + 8 * pitch));
+}
+
+NATSL_DEVICE bf16x8 pack8(const f32x16& x, const int ss) {
+  u32x4 w;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(x[8 * ss + 2 * j], x[8 * ss + 2 * j + 1]);
+  return __builtin_bit_cast(bf16x8, w);
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int DV>
+__global__ __launch_bounds__(256) void delta_kernel(const SoftmaxBwdParams p) {
+  constexpr int LPR = DV / 8, RPB = 256 / LPR;   // lanes per row, rows per workgroup
+  const long long rows = (long long)p.B * p.T * p.HQ;
+  const long long row = (long long)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int seg = threadIdx.x % LPR;
+  float acc = 0.f;
+  if (row < rows) {
+    const u32x4 a = *reinterpret_cast<const u32x4*>(p.o + row * DV + 8 * seg);
+    const u32x4 b = *reinterpret_cast<const u32x4*>(p.dout + row * DV + 8 * seg);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc += __uint_as_float(a[j] << 16) * __uint_as_float(b[j] << 16);
+      acc += __uint_as_float(a[j] & 0xffff0000u) * __uint_as_float(b[j] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
+  if (row < rows && seg == 0) p.delta[row] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// 256 threads stage a [64][D] tile row-major (pitch D+8) from rows tok0.. of a [T][stride] tensor, rows clamped to len-1
+template <int D>
+struct RowStage {
+  static constexpr int SEGS = D / 8, ROWS = 256 / SEGS, PASSES = 64 / ROWS, PITCH = D + 8;
+  u32x4 r[PASSES];
+  NATSL_DEVICE void load(const bf16_t* base, const size_t row_stride, const int tok0, const int len, const int tid) {
+    const int row = tid / SEGS, seg = tid % SEGS;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int tok = min(tok0 + row + ROWS * i, len - 1);
+      r[i] = *reinterpret_cast<const u32x4*>(base + (size_t)tok * row_stride + 8 * seg);
+    }
+  }
+  NATSL_DEVICE void store(bf16_t* tile, const int tid) const {
+    const int row = tid / SEGS, seg = tid % SEGS;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) *reinterpret_cast<u32x4*>(tile + (row + ROWS * i) * PITCH + 8 * seg) = r[i];
+  }
+};
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void dq_kernel(const SoftmaxBwdParams p) {
+  constexpr int KP = DK + 8, VP = DV + 8, KS = DK / 16, VS = DV / 16, DT = DK / 32, QTILE = 128;
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);  // [2][64][KP]
+  bf16_t* Vs = Ks + 2 * 64 * KP;                 // [2][64][VP]
+  __shared__ int lds_list[BWD_MAX_LDS_LIST];
+  __shared__ int lds_count;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hf = lane >> 5;
+  const int nq_tiles = (p.T + QTILE - 1) / QTILE;
+  const int pair = (int)blockIdx.x / nq_tiles, tile = nq_tiles - 1 - (int)blockIdx.x % nq_tiles;
+  const int n = pair / p.HQ, hq = pair % p.HQ;
+  const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
+  const int Bs = p.block, per_blk = Bs >> 6;
+  const int hkv = hq / (p.HQ / p.HKV), hn = hq / (p.HQ / p.HN);
+  const int tile_start = tile * QTILE;
+  const int q0 = tile_start + wave * 32;
+  const int my_chunk = q0 >> 6, qloc0 = q0 & 63;
+  const int dstart = (tile_start / p.block) * p.block;
+  const bool wave_valid = q0 < len;
+
+  const bf16_t* kp = p.k + ((size_t)bos * p.HKV + hkv) * DK;
+  const bf16_t* vp = p.v + ((size_t)bos * p.HKV + hkv) * DV;
+  const size_t krow = (size_t)p.HKV * DK, vrow = (size_t)p.HKV * DV;
+  const int32_t* list = p.idx + ((size_t)bos_nats * p.HN + hn) * 2;
+  const size_t list_stride = (size_t)p.HN * 2;
+  const int n_attn = p.nblk[((size_t)n * p.HN + hn) * 2];
+
+  // Q and dO as B operands (lane = query), lse and delta of the lane's query
+  bf16x8 QB[KS], DOB[VS];
+  const int qi = min(q0 + l32, len - 1);
+  {
+    const bf16_t* qr = p.q + ((size_t)(bos + qi) * p.HQ + hq) * DK + 8 * hf;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) QB[s] = ld8(qr + 16 * s);
+    const bf16_t* dr = p.dout + ((size_t)(bos + qi) * p.HQ + hq) * DV + 8 * hf;
+#pragma unroll
+    for (int s = 0; s < VS; ++s) DOB[s] = ld8(dr + 16 * s);
+  }
+  const float lse_q = p.lse[(size_t)(bos + qi) * p.HQ + hq], delta_q = p.delta[(size_t)(bos + qi) * p.HQ + hq];
+
+  f32x16 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+
+  RowStage<DK> sk;
+  RowStage<DV> sv;
+  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;
+  sk.load(kp, krow, dstart, len, tid);
+  sv.load(vp, vrow, dstart, len, tid);
+  if (tid == 0) lds_count = 0;
+  __syncthreads();
+  {
+    const int jmax = min(dstart / Bs, p.TN);
+    int cnt = 0;
+    for (int j = tid; j < jmax; j += 256) {
+      const int e = list[j * list_stride];
+      if (j < n_attn && (e + 1) * Bs <= dstart) {
+        ++cnt;
+        if (j < BWD_MAX_LDS_LIST) lds_list[j] = e;
+      }
+    }
+    if (cnt) atomicAdd(&lds_count, cnt);
+  }
+  unsigned long long diag_attn;
+  {
+    const int blk = dstart / Bs + lane;
+    const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
+    diag_attn = __ballot(in_range && bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
+  }
+  sk.store(Ks, tid);
+  sv.store(Vs, tid);
+  __syncthreads();
+  const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
+  const int n_iters = n_diag + n_prior_chunks;
+  int nx_it = 1, nx_j = 0, nx_sub = 0;
+  auto next_key_start = [&]() -> int {
+    int ks;
+    if (nx_it < n_diag) {
+      ks = dstart + nx_it * 64;
+    } else {
+      int e;
+      if (nx_j < BWD_MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+      else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
+      ks = e * Bs + nx_sub * 64;
+      if (++nx_sub == per_blk) {
+        nx_sub = 0;
+        ++nx_j;
+      }
+    }
+    ++nx_it;
+    return ks;
+  };
+  int ks_fetch = dstart;
+  if (n_iters > 1) ks_fetch = next_key_start();
+  const float c = p.scale_log2;
+  const int my_blk = q0 / Bs;
+
+  for (int it = 0; it < n_iters; ++it) {
+    const int buf = it & 1;
+    if (it + 1 < n_iters) {
+      sk.load(kp, krow, ks_fetch, len, tid);
+      sv.load(vp, vrow, ks_fetch, len, tid);
+    }
+    bool active = wave_valid, causal = false;
+    if (it < n_diag) {
+      const int jc = (dstart >> 6) + it;
+      const int kblk = (jc * 64) / Bs;
+      if (p.same_block) {
+        if (jc > my_chunk) active = false;
+        else if (jc == my_chunk) causal = true;
+        else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dstart / Bs)) & 1ull));
+      } else {
+        active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dstart / Bs)) & 1ull);
+      }
+    }
+    if (active) {
+      const bf16_t* Kb = Ks + buf * 64 * KP;
+      const bf16_t* Vb = Vs + buf * 64 * VP;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) s = mfma32(ld8(Kb + (32 * kt + l32) * KP + 16 * st + 8 * hf), QB[st], s);
+#pragma unroll
+        for (int st = 0; st < VS; ++st) dp = mfma32(ld8(Vb + (32 * kt + l32) * VP + 16 * st + 8 * hf), DOB[st], dp);
+        f32x16 ds;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3);
+          const bool vis = !causal || kloc <= qloc0 + l32;
+          const float pr = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse_q)) : 0.f;
+          ds[r] = pr * (dp[r] - delta_q);
+        }
+#pragma unroll
+        for (int ss = 0; ss < 2; ++ss) {
+          const bf16x8 PB = pack8(ds, ss);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(tr_operand(Kb, KP, 32 * kt + 16 * ss, 32 * dt, lane), PB, acc[dt]);
+        }
+      }
+    }
+    if (it + 1 < n_iters) {
+      sk.store(Ks + (buf ^ 1) * 64 * KP, tid);
+      sv.store(Vs + (buf ^ 1) * 64 * VP, tid);
+    }
+    if (it + 2 < n_iters) ks_fetch = next_key_start();
+    __syncthreads();
+  }
+
+  // epilogue: dQ = scale * acc, transposed through LDS, coalesced stores
+  bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + wave * 32 * KP;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      u32x2 w;
+      w[0] = pack_bf16x2(acc[dt][4 * rg] * p.scale, acc[dt][4 * rg + 1] * p.scale);
+      w[1] = pack_bf16x2(acc[dt][4 * rg + 2] * p.scale, acc[dt][4 * rg + 3] * p.scale);
+      *reinterpret_cast<u32x2*>(Os + l32 * KP + 32 * dt + 8 * rg + 4 * hf) = w;
+    }
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+  constexpr int SEGS = DK / 8, RPP = 64 / SEGS;
+#pragma unroll
+  for (int pass = 0; pass < 32 / RPP; ++pass) {
+    const int row = pass * RPP + lane / SEGS, seg = lane % SEGS;
+    const int t = q0 + row;
+    if (t < len) {
+      const u32x4 w = *reinterpret_cast<const u32x4*>(Os + row * KP + seg * 8);
+      *reinterpret_cast<u32x4*>(p.dq + ((size_t)(bos + t) * p.HQ + hq) * DK + seg * 8) = w;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int DK, int DV>
+__global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) {
+  constexpr int KP = DK + 8, VP = DV + 8, KS = DK / 16, VS = DV / 16, DT = DK / 32, VT = DV / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* Qs = reinterpret_cast<bf16_t*>(smem);     // [2][64][KP]
+  bf16_t* DOs = Qs + 2 * 64 * KP;                   // [2][64][VP]
+  float* Ls = reinterpret_cast<float*>(DOs + 2 * 64 * VP);  // [2][2][64]: lse, delta
+  __shared__ float red[4];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hf = lane >> 5;
+  const int kh = wave & 1, qh = wave >> 1;
+  const int NTc = (p.T + 63) >> 6;
+  const int n_pairs = p.B * p.HKV;
+  const int pair = (int)blockIdx.x % n_pairs, jc = (int)blockIdx.x / n_pairs;   // earliest (heaviest) chunks first
+  const int n = pair / p.HKV, hkv = pair % p.HKV;
+  const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
+  const int Bs = p.block, per_blk = Bs >> 6;
+  const int G = p.HQ / p.HKV, GN = p.HQ / p.HN;
+  const int kb = (jc * 64) / Bs;
+  const int blk_end_chunk = min((kb + 1) * per_blk, NTc);    // one past the last chunk of the key block
+
+  // K and V of the wave's 32 keys as B operands (lane = key)
+  bf16x8 KB[KS], VB[VS];
+  {
+    const int ki = min(jc * 64 + 32 * kh + l32, len - 1);
+    const bf16_t* kr = p.k + ((size_t)(bos + ki) * p.HKV + hkv) * DK + 8 * hf;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) KB[s] = ld8(kr + 16 * s);
+    const bf16_t* vr = p.v + ((size_t)(bos + ki) * p.HKV + hkv) * DV + 8 * hf;
+#pragma unroll
+    for (int s = 0; s < VS; ++s) VB[s] = ld8(vr + 16 * s);
+  }
+  f32x16 dv[VT], dk[DT];
+#pragma unroll
+  for (int t = 0; t < VT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dv[t][r] = 0.f;
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[t][r] = 0.f;
+
+  const float c = p.scale_log2;
+  RowStage<DK> sq;
+  RowStage<DV> sd;
+  float sl = 0.f;  // staged lse (threads 0..63) or delta (threads 64..127)
+  auto gload = [&](const int hq, const int jq) {
+    sq.load(p.q + ((size_t)bos * p.HQ + hq) * DK, (size_t)p.HQ * DK, jq * 64, len, tid);
+    sd.load(p.dout + ((size_t)bos * p.HQ + hq) * DV, (size_t)p.HQ * DV, jq * 64, len, tid);
+    if (tid < 128) {
+      const int t = min(jq * 64 + (tid & 63), len - 1);
+      const float* src = tid < 64 ? p.lse : p.delta;
+      sl = src[(size_t)(bos + t) * p.HQ + hq];
+    }
+  };
+  auto lstore = [&](const int buf) {
+    sq.store(Qs + buf * 64 * KP, tid);
+    sd.store(DOs + buf * 64 * VP, tid);
+    if (tid < 128) Ls[buf * 128 + tid] = sl;
+  };
+
+  for (int g = 0; g < G; ++g) {
+    const int hq = hkv * G + g, hn = hq / GN;
+    const bool attn = bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + kb) * p.HN + hn) * 2);
+    const int n_same = p.same_block ? blk_end_chunk - jc : 0;
+    const int n_later = attn ? max(NTc - blk_end_chunk, 0) : 0;
+    const int n_it = n_same + n_later;
+    float dn = 0.f;
+    auto chunk_of = [&](const int it) { return it < n_same ? jc + it : blk_end_chunk + (it - n_same); };
+    if (n_it > 0) {
+      gload(hq, chunk_of(0));
+      __syncthreads();   // the previous head's last reads of buffer 0 are done
+      lstore(0);
+      __syncthreads();
+    }
+    for (int it = 0; it < n_it; ++it) {
+      const int buf = it & 1;
+      const int jq = chunk_of(it);
+      if (it + 1 < n_it) gload(hq, chunk_of(it + 1));
+      const bf16_t* Qb = Qs + buf * 64 * KP;
+      const bf16_t* Db = DOs + buf * 64 * VP;
+      const float* Lb = Ls + buf * 128;
+      f32x16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+      for (int st = 0; st < KS; ++st) s = mfma32(ld8(Qb + (32 * qh + l32) * KP + 16 * st + 8 * hf), KB[st], s);
+#pragma unroll
+      for (int st = 0; st < VS; ++st) dp = mfma32(ld8(Db + (32 * qh + l32) * VP + 16 * st + 8 * hf), VB[st], dp);
+      f32x16 pr, ds;
+      const bool own = jq == jc;
+      float dsum = 0.f;
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Lb + 32 * qh + 8 * rg + 4 * hf);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Lb + 64 + 32 * qh + 8 * rg + 4 * hf);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int r = 4 * rg + j;
+          const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
+          const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
+          const float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[j])) : 0.f;
+          pr[r] = e;
+          ds[r] = e * (dp[r] - d4[j]);
+          dsum += ds[r];
+        }
+      }
+      if (it >= n_same && jc * 64 + 32 * kh + l32 < len) dn += dsum;
+#pragma unroll
+      for (int ss = 0; ss < 2; ++ss) {
+        const bf16x8 PBp = pack8(pr, ss), PBs = pack8(ds, ss);
+#pragma unroll
+        for (int t = 0; t < VT; ++t) dv[t] = mfma32(tr_operand(Db, VP, 32 * qh + 16 * ss, 32 * t, lane), PBp, dv[t]);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) dk[t] = mfma32(tr_operand(Qb, KP, 32 * qh + 16 * ss, 32 * t, lane), PBs, dk[t]);
+      }
+      if (it + 1 < n_it) lstore(buf ^ 1);
+      __syncthreads();
+    }
+    // dnats of this (key block, query head): the four waves' sums
+    if (n_later > 0) {
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) dn += __shfl_xor(dn, m);
+      if (lane == 0) red[wave] = dn;
+      __syncthreads();
+      if (tid == 0) atomicAdd(p.dnats + ((size_t)(bos_nats + kb)) * p.HQ + hq, red[0] + red[1] + red[2] + red[3]);
+      __syncthreads();
+    }
+  }
+
+  // ---- the two query halves of a key half are summed through LDS, then the tiles are transposed and stored
+  __syncthreads();
+  float* Rs = reinterpret_cast<float*>(smem);   // [2 key halves][(VT + DT) * 16][64 lanes]
+  if (qh == 1) {
+    float* dst = Rs + (size_t)kh * (VT + DT) * 16 * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[(t * 16 + r) * 64] = dv[t][r];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[((VT + t) * 16 + r) * 64] = dk[t][r];
+  }
+  __syncthreads();
+  if (qh == 0) {
+    const float* src = Rs + (size_t)kh * (VT + DT) * 16 * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dv[t][r] += src[(t * 16 + r) * 64];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dk[t][r] = (dk[t][r] + src[((VT + t) * 16 + r) * 64]) * p.scale;
+  }
+  __syncthreads();
+  if (qh == 0) {
+    // accumulators are [value or dim rows x key columns]: write [key][value|dim] rows to LDS, then coalesced stores
+    constexpr int OP = DV + DK + 8;
+    bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + kh * 32 * OP;
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 w;
+        w[0] = pack_bf16x2(dv[t][4 * rg], dv[t][4 * rg + 1]);
+        w[1] = pack_bf16x2(dv[t][4 * rg + 2], dv[t][4 * rg + 3]);
+        *reinterpret_cast<u32x2*>(Os + l32 * OP + 32 * t + 8 * rg + 4 * hf) = w;
+      }
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 w;
+        w[0] = pack_bf16x2(dk[t][4 * rg], dk[t][4 * rg + 1]);
+        w[1] = pack_bf16x2(dk[t][4 * rg + 2], dk[t][4 * rg + 3]);
+        *reinterpret_cast<u32x2*>(Os + l32 * OP + DV + 32 * t + 8 * rg + 4 * hf) = w;
+      }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    for (int i = lane; i < 32 * (DV / 8); i += 64) {
+      const int row = i / (DV / 8), seg = i % (DV / 8);
+      const int t = jc * 64 + 32 * kh + row;
+      if (t < len)
+        *reinterpret_cast<u32x4*>(p.dv + ((size_t)(bos + t) * p.HKV + hkv) * DV + seg * 8) =
+            *reinterpret_cast<const u32x4*>(Os + row * OP + seg * 8);
+    }
+    for (int i = lane; i < 32 * (DK / 8); i += 64) {
+      const int row = i / (DK / 8), seg = i % (DK / 8);
+      const int t = jc * 64 + 32 * kh + row;
+      if (t < len)
+        *reinterpret_cast<u32x4*>(p.dk + ((size_t)(bos + t) * p.HKV + hkv) * DK + seg * 8) =
+            *reinterpret_cast<const u32x4*>(Os + row * OP + DV + seg * 8);
+    }
+  }
+}
+
+template <int DK, int DV>
+static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
+  constexpr int KP = DK + 8, VP = DV + 8;
+  const long long rows = (long long)p.B * p.T * p.HQ;
+  constexpr int RPB = 256 / (DV / 8);
+  hipLaunchKernelGGL((delta_kernel<DV>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream, p);
+  {
+    size_t lds = (size_t)2 * 64 * (KP + VP) * sizeof(bf16_t);
+    auto kern = dq_kernel<DK, DV>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    const long long grid = (long long)p.B * p.HQ * ((p.T + 127) / 128);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
+  }
+  {
+    size_t lds = (size_t)2 * 64 * (KP + VP) * sizeof(bf16_t) + 2 * 128 * sizeof(float);
+    const size_t red = (size_t)2 * (DV / 32 + DK / 32) * 16 * 64 * sizeof(float);
+    if (red > lds) lds = red;
+    auto kern = dkdv_kernel<DK, DV>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    const long long grid = (long long)p.B * p.HKV * ((p.T + 63) / 64);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
+  }
+  return check_launch("natsl_softmax_sparse_bwd");
+}
+
+}  // namespace natsl
+
+using namespace natsl;
+
+extern "C" size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ) { return (size_t)B * T * HQ * sizeof(float); }
+
+extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
+                                        const void* d_o, void* dq, void* dk, void* dv, float* dnats, const void* types,
+                                        int types_dtype, const int32_t* nats_block_indices, const int32_t* n_nats_blocks,
+                                        int B, int T, int HQ, int HKV, int HN, int K, int V, int TN, int block, float scale,
+                                        int same_block_visible, int dtype, void* workspace, size_t workspace_bytes,
+                                        natsl_stream_t stream) {
+  const char* what = "natsl_softmax_sparse_bwd";
+  if (!q || !k || !v || !o || !lse || !d_o || !dq || !dk || !dv || !dnats || !types || !nats_block_indices || !n_nats_blocks)
+    return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
+  if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
+  if (B <= 0 || T <= 0 || HQ <= 0 || HKV <= 0 || HN <= 0 || TN <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
+  if (HQ % HKV || HQ % HN) return fail(NATSL_ERR_INVALID, "%s: HQ=%d must be a multiple of HKV=%d and HN=%d", what, HQ, HKV, HN);
+  if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
+  if (TN != cdiv(T, block)) return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d", what, TN, T, block);
+  if (!workspace || workspace_bytes < natsl_softmax_bwd_workspace_bytes(B, T, HQ))
+    return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", what, natsl_softmax_bwd_workspace_bytes(B, T, HQ));
+  SoftmaxBwdParams p;
+  p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (const bf16_t*)o; p.dout = (const bf16_t*)d_o;
+  p.lse = lse; p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dv = (bf16_t*)dv; p.dnats = dnats; p.delta = (float*)workspace;
+  p.types = types; p.types_dtype = types_dtype; p.idx = nats_block_indices; p.nblk = n_nats_blocks;
+  p.B = B; p.T = T; p.HQ = HQ; p.HKV = HKV; p.HN = HN; p.TN = TN; p.block = block;
+  p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f; p.same_block = same_block_visible ? 1 : 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define NATSL_SB(KK, VV) \
+  if (K == KK && V == VV) return launch_bwd<KK, VV>(p, s);
+  NATSL_SB(128, 128)
+  NATSL_SB(64, 64)
+  NATSL_SB(64, 128)
+  NATSL_SB(128, 64)
+#undef NATSL_SB
+  return fail(NATSL_ERR_UNSUPPORTED, "%s: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", what, K, V);
+}

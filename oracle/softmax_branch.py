@@ -104,3 +104,56 @@ def flops(types: torch.Tensor, T: int, block: int, K: int, V: int, heads_per_sel
         n = min(block, T - c * block)
         tot += float((n * (n + 1) / 2 + n * block * prior[:, c]).sum())
     return 2.0 * (K + V) * tot * heads_per_selector
+
+
+def softmax_branch_bwd(q, k, v, types, do, scale, block, same_block_visible=True, dtype=torch.float64, with_magnitude=False):
+    """Gradients of the softmax branch in closed form (parallel_attn_nats_bwd, src/nats/ops/attns/attns.py:1562-1759;
+    kernels :383-708 for dq, :719-983 for dk, dv and dnats):
+        P = softmax(masked scores), delta = rowsum(dO * O) (:357-372), dP = dO V^T, dS = P * (dP - delta)
+        dq = scale dS K (:704), dk = scale dS^T Q (:966, summed over the query heads of a kv head :1746),
+        dv = P^T dO (:1747)
+        dnats[b, j, hn] = sum of dS over (keys of block j) x (queries of LATER blocks), summed over the query heads of
+        selector head hn, for blocks typed attention (:946-961, :1755); 0 for the other blocks (the default
+        compute_dnats_for_invalid_blocks_attn=False).  It is the gradient with respect to a bias added to the
+        (natural-log scale) scores of a block's keys as later blocks see them.
+    -> (dq [B,T,HQ,K], dk [B,T,HKV,K], dv [B,T,HKV,V], dnats [B,NB,HN]); with_magnitude adds the same sums over |dS|
+    (the scale rounding errors of dnats are measured against: the signed sums cancel, down to exactly 0 when a query
+    sees a single earlier block and nothing else).
+
+    What pins it: torch.autograd through the same dense masked softmax with that bias as a zero tensor
+    (tests/test_oracle_branches.py)."""
+    B, T, HQ, K = q.shape
+    HKV, V = k.shape[2], v.shape[-1]
+    NB, HN = types.shape[1], types.shape[2]
+    G, GN = HQ // HKV, HQ // HN
+    dq = torch.zeros(B, T, HQ, K, dtype=dtype)
+    dk = torch.zeros(B, T, HKV, K, dtype=dtype)
+    dv = torch.zeros(B, T, HKV, V, dtype=dtype)
+    dnats = torch.zeros(B, NB, HN, dtype=dtype)
+    dnats_mag = torch.zeros(B, NB, HN, dtype=dtype)
+    a = torch.round(types[..., 0].float())
+    blk = torch.arange(T) // block
+    later = blk.view(-1, 1) > blk.view(1, -1)                                  # [query, key]: the key's block is an earlier one
+    for b in range(B):
+        for hq in range(HQ):
+            hn, hk = hq // GN, hq // G
+            m = visibility_mask(a[b, :, hn], T, block, same_block_visible)
+            qq, kk, vv, dd = (x.to(dtype) for x in (q[b, :, hq], k[b, :, hk], v[b, :, hk], do[b, :, hq]))
+            s = (qq @ kk.T) * scale
+            s = s.masked_fill(~m, float('-inf'))
+            valid = m.any(-1, keepdim=True)
+            p = torch.where(valid, torch.softmax(torch.where(valid, s, torch.zeros_like(s)), -1), torch.zeros_like(s))
+            p = p * m
+            o = p @ vv
+            delta = (dd * o).sum(-1, keepdim=True)
+            ds = p * (dd @ vv.T - delta)
+            dq[b, :, hq] = scale * ds @ kk
+            dk[b, :, hk] += scale * ds.T @ qq
+            dv[b, :, hk] += p.T @ dd
+            inter = ds * later                                                  # [query, key]
+            per_block = torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter.sum(0))
+            dnats[b, :, hn] += per_block * a[b, :, hn].to(dtype)
+            dnats_mag[b, :, hn] += torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter.abs().sum(0)) * a[b, :, hn].to(dtype)
+    if with_magnitude:
+        return dq, dk, dv, dnats, dnats_mag
+    return dq, dk, dv, dnats

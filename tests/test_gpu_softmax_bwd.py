@@ -1,0 +1,83 @@
+"""GPU parity: backward of the softmax branch through the C ABI vs oracle/softmax_branch.softmax_branch_bwd
+(fp64 on the same bf16-rounded inputs).  Tolerance for gradients: rel-L2 5e-3 as for the outputs; the absolute part of
+the outputs' tolerance does not transfer (gradients are not O(1)), so max-abs is checked against 2e-2 of the
+reference's largest magnitude."""
+import pytest
+import torch
+
+from oracle import softmax_branch as sb
+from tests._util import make_qkv, make_types, max_abs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+def _close(a, b, what):
+    rl, ma, top = rel_l2(a, b), max_abs(a, b), float(b.abs().max())
+    assert rl <= 5e-3 and ma <= 2e-2 * max(top, 1.0), f"{what}: rel-L2 {rl:.3e}, max-abs {ma:.3e} (largest reference value {top:.3e})"
+
+
+def _run(B, T, HQ, H, HN, K, V, block, p_attn, same_block, seed, through_autograd=False):
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_bwd, parallel_attn_nats_fwd, parallel_nats_attn
+    q, k, v = make_qkv(B, T, H, K, V, seed, HQ=HQ)
+    do = torch.randn(B, T, HQ, V, generator=torch.Generator().manual_seed(seed + 7)).bfloat16()
+    ty = make_types(B, -(-T // block), HN, p_attn, seed + 1, torch.bfloat16)
+    scale = K ** -0.5
+    dq_r, dk_r, dv_r, dn_r, dn_mag = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block, with_magnitude=True)
+    qd, kd, vd, dod, tyd = (t.to(DEV) for t in (q, k, v, do, ty))
+    r = nats_util.route(tyd, T, block)
+    if through_autograd:
+        qd, kd, vd = (t.requires_grad_() for t in (qd, kd, vd))
+        tyd = tyd.requires_grad_()
+        o, _ = parallel_nats_attn(qd, kd, vd, None, tyd, r['nats_block_indices'], r['n_nats_blocks'], scale,
+                                  NAtS_block_size=block, compute_incomplete_chunk_scores=same_block)
+        o.backward(dod)
+        dq, dk, dv, dn = qd.grad, kd.grad, vd.grad, tyd.grad[..., 0]
+        assert float(tyd.grad[..., 1:].abs().max()) == 0.0
+    else:
+        o, lse, _ = parallel_attn_nats_fwd(qd, kd, vd, tyd, r['nats_block_indices'], None, scale, block,
+                                           compute_incomplete_chunk_scores=same_block, n_nats_blocks=r['n_nats_blocks'])
+        dq, dk, dv, _, dn = parallel_attn_nats_bwd(qd, kd, vd, o, tyd, r['nats_block_indices'], r['n_nats_blocks'], None, lse, dod,
+                                                   scale=scale, NAtS_block_size=block, compute_incomplete_chunk_scores=same_block)
+    torch.cuda.synchronize()
+    _close(dq.float(), dq_r, "dq")
+    _close(dk.float(), dk_r, "dk")
+    _close(dv.float(), dv_r, "dv")
+    # dnats sums thousands of signed terms that largely cancel (to exactly 0 when a query sees one earlier block and
+    # nothing else): the error is measured against the sum of their magnitudes
+    err = (dn.float().cpu().double() - dn_r).abs()
+    assert bool((err <= 2e-3 * dn_mag + 1e-6).all()), f"dnats: error {float(err.max()):.3e} against a magnitude of {float(dn_mag.max()):.3e}"
+    lin = torch.round(ty[..., 0].float()) == 0
+    assert float(dn.float().cpu()[lin].abs().max() if lin.any() else 0.0) == 0.0, "blocks not typed attention get no gradient"
+
+
+@pytest.mark.parametrize("same_block", [True, False])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
+def test_softmax_bwd_small(K, V, same_block):
+    _run(2, 512, 4, 4, 4, K, V, 64, 0.4, same_block, seed=0)
+
+
+def test_softmax_bwd_gqa_and_selector_groups():
+    _run(1, 768, 8, 4, 2, 128, 128, 64, 0.5, True, seed=3)
+    _run(1, 512, 8, 2, 8, 64, 64, 64, 0.5, True, seed=4)       # more selector heads than kv heads
+
+
+def test_softmax_bwd_ragged_length():
+    _run(2, 600, 2, 2, 2, 128, 128, 64, 0.5, True, seed=5)
+    _run(1, 100, 2, 2, 2, 64, 64, 64, 0.5, True, seed=6)
+
+
+@pytest.mark.parametrize("block", [128, 256])
+def test_softmax_bwd_large_blocks(block):
+    _run(1, 1024, 2, 2, 2, 128, 64, block, 0.5, True, seed=7)
+    _run(1, 1024, 2, 2, 2, 128, 64, block, 0.5, False, seed=8)
+
+
+def test_softmax_bwd_all_attention_and_all_linear():
+    _run(1, 512, 2, 2, 2, 128, 128, 64, 1.0, True, seed=9)
+    _run(1, 512, 2, 2, 2, 128, 128, 64, 0.0, True, seed=10)
+
+
+def test_softmax_bwd_through_autograd():
+    _run(2, 384, 4, 2, 2, 128, 128, 64, 0.5, True, seed=11, through_autograd=True)

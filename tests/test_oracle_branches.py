@@ -211,3 +211,37 @@ def test_norm_gate_closed_form():
     y = norm_gate.two_input_rmsnorm_gated(x1, x2, gate, xw, w1, w2, eps=1e-5)
     ref = (F.rms_norm(x1, (16,), w1, 1e-5) * xw[..., :1] + F.rms_norm(x2, (16,), w2, 1e-5) * xw[..., 1:]) * F.silu(gate)
     _close(y, ref, 1e-5)
+
+
+@pytest.mark.parametrize("same_block", [True, False])
+def test_softmax_backward_closed_form_equals_autograd(same_block):
+    """oracle/softmax_branch.softmax_branch_bwd against torch.autograd through a dense masked softmax in which every
+    block's keys carry a bias (a zero tensor) as LATER blocks see them: d/d(bias) is what the reference calls dnats."""
+    from oracle import softmax_branch as sb
+    from tests._util import make_types
+    torch.manual_seed(3)
+    B, T, HQ, HKV, HN, K, V, block = 2, 200, 4, 2, 2, 16, 8, 64
+    NB = -(-T // block)
+    q = torch.randn(B, T, HQ, K, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(B, T, HKV, K, dtype=torch.float64, requires_grad=True)
+    v = torch.randn(B, T, HKV, V, dtype=torch.float64, requires_grad=True)
+    do = torch.randn(B, T, HQ, V, dtype=torch.float64)
+    ty = make_types(B, NB, HN, 0.5, 4, force_last=False)
+    bias = torch.zeros(B, NB, HQ, dtype=torch.float64, requires_grad=True)
+    scale = K ** -0.5
+    blk = torch.arange(T) // block
+    later = (blk.view(-1, 1) > blk.view(1, -1)).double()
+    loss = 0
+    for b in range(B):
+        for hq in range(HQ):
+            m = sb.visibility_mask(torch.round(ty[b, :, hq // (HQ // HN), 0]), T, block, same_block)
+            s = (q[b, :, hq] @ k[b, :, hq // (HQ // HKV)].T) * scale + bias[b, blk, hq].view(1, -1) * later
+            s = s.masked_fill(~m, -1e300)
+            p = torch.softmax(s, -1) * m
+            loss = loss + ((p @ v[b, :, hq // (HQ // HKV)]) * do[b, :, hq]).sum()
+    gq, gk, gv, gb = torch.autograd.grad(loss, (q, k, v, bias))
+    dq, dk, dv, dnats = sb.softmax_branch_bwd(q.detach(), k.detach(), v.detach(), ty, do, scale, block, same_block)
+    a = torch.round(ty[..., 0]).double()
+    want_dnats = (gb.view(B, NB, HN, HQ // HN).sum(-1)) * a                     # attention-typed blocks only
+    for got, want, name in ((dq, gq, 'dq'), (dk, gk, 'dk'), (dv, gv, 'dv'), (dnats, want_dnats, 'dnats')):
+        assert float((got - want).abs().max()) < 1e-9, name
