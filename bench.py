@@ -31,6 +31,10 @@ DECODE_WORKLOADS = {
 CACHE_WORKLOADS = {
     "kv_compact_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
 }
+# backward of the softmax branch at the headline shape (training); not the headline metric
+BACKWARD_WORKLOADS = {
+    "softmax_bwd_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
+}
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 
@@ -195,12 +199,54 @@ def bench_kv_compact(args):
                       frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, traffic=None, algorithmic_bytes=nbytes, launch_ms=ms))))
 
 
+def bench_softmax_bwd(args):
+    """Backward of the softmax branch: dq, dk, dv and the selector's gradient from (q, k, v, o, lse, do).  Five products
+    per (query, visible key) pair -- S, dP, dV, dK, dQ -- so 2.5x the forward's FLOPs; the two kernels form S and dP
+    twice (once per kernel), which is not counted."""
+    import torch
+    from neuralattentionsearchlinear_amd import _capi, nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_bwd, parallel_attn_nats_fwd
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    w = BACKWARD_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    host, d = make_inputs(w, torch, dev)
+    ty, nb = nats_util.hard_select(d["logits"], force_last_block=True)
+    r = nats_util.route(ty, w["T"], w["block"])
+    scale = w["K"] ** -0.5
+    o, lse, _ = parallel_attn_nats_fwd(d["q"], d["k"], d["v"], ty, r["nats_block_indices"], None, scale, w["block"],
+                                       compute_incomplete_chunk_scores=True, n_nats_blocks=r["n_nats_blocks"])
+    do = torch.randn(o.shape, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).bfloat16()
+
+    def step():
+        return parallel_attn_nats_bwd(d["q"], d["k"], d["v"], o, ty, r["nats_block_indices"], r["n_nats_blocks"], None, lse, do,
+                                      scale=scale, NAtS_block_size=w["block"], compute_incomplete_chunk_scores=True)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    flops = 2.5 * softmax_flops(ty.cpu(), w["T"], w["block"], w["K"], w["V"])
+    print(json.dumps(dict(
+        metric="softmax-branch backward tokens/sec @T=8192,H=16,d=128 bf16", value=w["B"] * w["T"] / (ms * 1e-3), unit="tokens/s",
+        n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w),
+        roofline=dict(bound="mfma", kernel="dq_kernel+dkdv_kernel", achieved=flops / (ms * 1e-3) / 1e12, peak=PEAK_BF16_MFMA_TFLOPS,
+                      unit="TFLOP/s", frac=flops / (ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS, traffic=None, algorithmic_flops=flops,
+                      note="whole step: delta, dq and dk/dv kernels"))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS))
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
     ap.add_argument("--cpu-batch", type=int, default=8, help="sequences of the slice timed on the CPU")
@@ -220,6 +266,8 @@ def main():
         return bench_decode(args)
     if args.workload in CACHE_WORKLOADS:
         return bench_kv_compact(args)
+    if args.workload in BACKWARD_WORKLOADS:
+        return bench_softmax_bwd(args)
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn

@@ -98,7 +98,7 @@ struct RowStage {
 };
 
 template <int DK, int DV>
-__global__ __launch_bounds__(256) void dq_kernel(const SoftmaxBwdParams p) {
+__global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
   constexpr int KP = DK + 8, VP = DV + 8, KS = DK / 16, VS = DV / 16, DT = DK / 32, QTILE = 128;
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);  // [2][64][KP]
@@ -223,13 +223,20 @@ __global__ __launch_bounds__(256) void dq_kernel(const SoftmaxBwdParams p) {
       const bf16_t* Vb = Vs + buf * 64 * VP;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
+        // the LDS operands of the first two products are requested ahead of the matrix instructions that use them
+        bf16x8 ak[KS], av[VS];
+#pragma unroll
+        for (int st = 0; st < KS; ++st) ak[st] = ld8(Kb + (32 * kt + l32) * KP + 16 * st + 8 * hf);
+#pragma unroll
+        for (int st = 0; st < VS; ++st) av[st] = ld8(Vb + (32 * kt + l32) * VP + 16 * st + 8 * hf);
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-        for (int st = 0; st < KS; ++st) s = mfma32(ld8(Kb + (32 * kt + l32) * KP + 16 * st + 8 * hf), QB[st], s);
-#pragma unroll
-        for (int st = 0; st < VS; ++st) dp = mfma32(ld8(Vb + (32 * kt + l32) * VP + 16 * st + 8 * hf), DOB[st], dp);
+        for (int st = 0; st < (KS > VS ? KS : VS); ++st) {   // the two chains alternate
+          if (st < KS) s = mfma32(ak[st], QB[st], s);
+          if (st < VS) dp = mfma32(av[st], DOB[st], dp);
+        }
         f32x16 ds;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -240,9 +247,12 @@ __global__ __launch_bounds__(256) void dq_kernel(const SoftmaxBwdParams p) {
         }
 #pragma unroll
         for (int ss = 0; ss < 2; ++ss) {
+          bf16x8 at[DT];
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) at[dt] = tr_operand(Kb, KP, 32 * kt + 16 * ss, 32 * dt, lane);
           const bf16x8 PB = pack8(ds, ss);
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(tr_operand(Kb, KP, 32 * kt + 16 * ss, 32 * dt, lane), PB, acc[dt]);
+          for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(at[dt], PB, acc[dt]);
         }
       }
     }
@@ -368,9 +378,10 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-      for (int st = 0; st < KS; ++st) s = mfma32(ld8(Qb + (32 * qh + l32) * KP + 16 * st + 8 * hf), KB[st], s);
-#pragma unroll
-      for (int st = 0; st < VS; ++st) dp = mfma32(ld8(Db + (32 * qh + l32) * VP + 16 * st + 8 * hf), VB[st], dp);
+      for (int st = 0; st < (KS > VS ? KS : VS); ++st) {   // the two chains alternate
+        if (st < KS) s = mfma32(ld8(Qb + (32 * qh + l32) * KP + 16 * st + 8 * hf), KB[st], s);
+        if (st < VS) dp = mfma32(ld8(Db + (32 * qh + l32) * VP + 16 * st + 8 * hf), VB[st], dp);
+      }
       f32x16 pr, ds;
       const bool own = jq == jc;
       float dsum = 0.f;
