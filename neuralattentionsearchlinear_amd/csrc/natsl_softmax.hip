@@ -67,12 +67,24 @@ NATSL_DEVICE void mask_half(f32x16& s, const int kt, const int lane, const int q
     if (8 * (r >> 2) + (r & 3) > d) s[r] = -INFINITY;
 }
 
+// max(a, b, c) as ONE instruction.  fmaxf() costs three here: the compiler first quiets possible signalling NaNs of
+// each operand (v_mul by 1.0) because it cannot know that matrix-instruction results are canonical.  The scores hold
+// no NaNs (masked entries are -inf), so the plain instruction gives the same result.
+NATSL_DEVICE float max3_plain(const float a, const float b, const float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // scaled row maximum of one half (both lane halves joined)
 NATSL_DEVICE float half_max(const f32x16& s, const float c) {
-  float m = -INFINITY;
+  float m0 = -INFINITY, m1 = -INFINITY;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) m = fmaxf(m, s[r]);
-  return xhalf_max(m) * c;
+  for (int r = 0; r < 16; r += 4) {
+    m0 = max3_plain(m0, s[r], s[r + 1]);
+    m1 = max3_plain(m1, s[r + 2], s[r + 3]);
+  }
+  return xhalf_max(max3_plain(m0, m1, m1)) * c;
 }
 
 // P = exp2(S*c - m_ref) for one half, packed to bf16 in the B-operand order; adds the row sums
@@ -209,6 +221,154 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
   l_run += rs;  // partial over this lane's keys; the lane halves are joined in the epilogue
 }
 
+// ---- the 8-wave schedule: one chunk as three phases ----------------------------------------------------------------
+// K chunks go from global memory straight into LDS (global_load_lds_dwordx4: every lane names 16 source bytes, the
+// wave's 1 KiB lands contiguously at the LDS address in M0): no staging registers, no LDS store instructions.  The K
+// tile is row-major, [64 keys][DK] without padding; bank conflicts are avoided by an XOR swizzle of the 16-byte
+// segments of a row (segment s of row r sits at s ^ (r & 7): the operand read is ds_read_b128, 8 lanes = 8 rows per
+// clock), applied on the way in by letting each lane fetch the segment that belongs at its LDS position.
+// V has to be transposed on the way (the matrix instruction wants 8 consecutive keys per lane, memory has 8
+// consecutive value columns), which the DMA cannot do: it passes through registers (4x8 transposes with v_perm_b32).
+// The two waves that share a SIMD run half a chunk apart (see the kernel), so a wave's vector phase (softmax_phase)
+// meets the other wave's matrix phases (pv_phase, qk_phase).
+
+// one DMA instruction: lane l copies 16 bytes from base + voff to LDS byte address lds + 16 l
+NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+}
+
+// S^T = K Q^T - m_ref for both key halves of one chunk: the accumulators start from minus the reference maximum of the
+// lane's query, so the scores come out of the matrix pipe already shifted.  The halves alternate so that consecutive
+// instructions are independent.  kaddr: LDS byte address of this lane's row (lane%32) in the tile, plus 16*((lane>>5) ^
+// (lane & 7)): XOR-ing it with 32*(k-step & 3) gives the swizzled position of the lane's 16 bytes of that k-step.
+template <int DK>
+NATSL_DEVICE void qk_phase(const unsigned kaddr, const bf16x8 (&QB)[DK / 16], const float m_ref, f32x16& s0, f32x16& s1) {
+  constexpr int N = DK / 8, A = OPERANDS_AHEAD;
+  typedef __attribute__((address_space(3))) const bf16x8* lds_op;
+  unsigned base[4];  // one register per swizzle value, opaque to the compiler (see pv_phase)
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    base[q] = kaddr ^ (32u * q);
+    asm("" : "+v"(base[q]));
+  }
+  auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+    const int st = j >> 1, half = j & 1;
+    return *reinterpret_cast<lds_op>(base[st & 3] + 128u * (st >> 2) + half * 32u * (2u * DK));
+  };
+  bf16x8 op[N + A];
+#pragma unroll
+  for (int j = 0; j < A; ++j) op[j] = ld_op(j);
+  f32x16 start;  // short-lived: the first instruction of each chain reads it
+#pragma unroll
+  for (int r = 0; r < 16; ++r) start[r] = -m_ref;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    if (j + A < N) op[j + A] = ld_op(j + A);
+    if (j & 1) s1 = mfma32(op[j], QB[j >> 1], j == 1 ? start : s1);
+    else s0 = mfma32(op[j], QB[j >> 1], j == 0 ? start : s0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, A, 0);
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    if (j + A < N) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  }
+}
+
+// sum of the two bf16 halves of w, added to acc in fp32
+NATSL_DEVICE float dot2_ones(const unsigned w, const float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+}
+
+// O^T += V^T P^T for one chunk: PB[g] holds the probabilities of keys 16 g .. 16 g + 15.  V is staged transposed,
+// [DV][VTP] with the keys of a 16-key group stored in the order the probabilities are held (a lane's 8 k-slots are 16
+// contiguous bytes), so an operand is ONE ds_read_b128: the LDS pipe takes as long for an 8-byte read instruction as
+// for a 16-byte one, and two reads per operand made this phase LDS-bound.  vaddr: LDS byte address of the lane's row
+// (lane%32) of the tile plus 16*(lane>>5).  The row sums are taken from the same rounded probabilities, one v_dot2
+// under each matrix instruction.
+constexpr int VTP = 72;  // elements per row of that tile (64 keys + 8): conflict-free 16-byte reads and 8-byte transposed stores
+template <int DV>
+NATSL_DEVICE void pv_phase(const unsigned vaddr, const bf16x8 (&PB)[4], f32x16 (&acc)[DV / 32], float& l_run) {
+  constexpr int VT = DV / 32, N = 4 * VT, A = OPERANDS_AHEAD, DOTS = 16 / N;  // 16 packed words per lane
+  static_assert(16 % N == 0, "row sums ride on the matrix instructions");
+  typedef __attribute__((address_space(3))) const bf16x8* lds_op;
+  // (opaque to the compiler: it must stay ONE base register with the tile offsets in the instructions' offset fields;
+  // re-associated with the ring arithmetic of the caller, half of the offsets came out negative, each read got an
+  // address computation of its own and the reads were no longer issued ahead of their use)
+  unsigned base = vaddr;
+  asm("" : "+v"(base));
+  auto ld_op = [&](const int i) __attribute__((always_inline)) -> bf16x8 {
+    const int g = i / VT, vt = i % VT;
+    return *reinterpret_cast<lds_op>(base + 32u * vt * (2u * VTP) + 32u * g);
+  };
+  bf16x8 op[N + A];
+#pragma unroll
+  for (int j = 0; j < A; ++j) op[j] = ld_op(j);
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (i + A < N) op[i + A] = ld_op(i + A);
+    acc[i % VT] = mfma32(op[i], PB[i / VT], acc[i % VT]);
+#pragma unroll
+    for (int d = 0; d < DOTS; ++d) l_run = dot2_ones(__builtin_bit_cast(u32x4, PB[(i * DOTS + d) / 4])[(i * DOTS + d) % 4], l_run);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, A, 0);
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (i + A < N) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  }
+}
+
+// Shifted scores of one chunk (s = score - m_ref, straight from the matrix pipe) -> probabilities in the B-operand
+// order.  The common path is a maximum (for the check), 32 exp2 and the packing.  The reference moves, in a side
+// block, when a score outgrows it by more than `thr`: -inf while the row has seen no key yet (m_ref is then still the
+// arbitrary 0 and the first visible score sets the real one), RESCALE_SLACK afterwards.
+template <int DV>
+NATSL_DEVICE void softmax_phase(f32x16& s0, f32x16& s1, f32x16 (&acc)[DV / 32], float& m_ref, float& l_run, float& thr,
+                                const int lane, const bool causal, const int qloc0, bf16x8 (&PB)[4]) {
+  if (causal) {
+    mask_half(s0, 0, lane, qloc0);
+    mask_half(s1, 1, lane, qloc0);
+  }
+  float m0 = -INFINITY, m1 = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 16; r += 2) {
+    m0 = max3_plain(m0, s0[r], s0[r + 1]);
+    m1 = max3_plain(m1, s1[r], s1[r + 1]);
+  }
+  const float mx = xhalf_max(max3_plain(m0, m1, m1));
+  if (__any(mx > thr)) {
+    const bool unset = thr < 0.f;
+    float m_new = unset ? m_ref + mx : fmaxf(m_ref, m_ref + mx);
+    if (mx == -INFINITY) m_new = m_ref;  // still nothing visible: keep whatever reference there is
+    else thr = RESCALE_SLACK;
+    const float delta = m_new - m_ref;
+    const float alpha = unset ? 1.f : __builtin_amdgcn_exp2f(-delta);  // unset: nothing accumulated yet
+    m_ref = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int vt = 0; vt < DV / 32; ++vt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[vt][r] *= alpha;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s0[r] -= delta;
+      s1[r] -= delta;
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x16& s = g < 2 ? s0 : s1;
+    u32x4 w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      w[j] = pack_bf16x2(__builtin_amdgcn_exp2f(s[8 * (g & 1) + 2 * j]), __builtin_amdgcn_exp2f(s[8 * (g & 1) + 2 * j + 1]));
+    PB[g] = __builtin_bit_cast(bf16x8, w);
+  }
+}
+
 // NWAVES waves of 32 queries: the workgroup owns QTILE = 32*NWAVES queries.
 template <int DK, int DV, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES, NWAVES == 4 ? 2 : 1) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -279,8 +439,18 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   {
     const int qi = min(q0 + l32, len - 1);  // rows past the end are computed on a copy and never stored
     const bf16_t* qr = qp + (size_t)qi * p.HQ * DK + 8 * hf;
+    // The queries carry the softmax scale (and log2 e) from here on, rounded to bf16 like the reference's scaled
+    // queries: the matrix pipe then delivers the scores in log2 units.
+    const float qscale = p.scale_log2;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) QB[s] = ld8(qr + 16 * s);
+    for (int s = 0; s < KSTEPS; ++s) {
+      const u32x4 w = *reinterpret_cast<const u32x4*>(qr + 16 * s);
+      u32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = pack_bf16x2(__uint_as_float(w[j] << 16) * qscale, __uint_as_float(w[j] & 0xffff0000u) * qscale);
+      QB[s] = __builtin_bit_cast(bf16x8, r);
+    }
   }
 
   if (tile_start >= len) return;  // packed input: a sequence's last 256-row table slot may hold no tile of this size
@@ -299,7 +469,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   // two chunks are in flight per thread (two register sets of 4 loads) at the same register cost.
   static_assert(NTHREADS == 256 || NTHREADS == 512, "staging is written for 4 or 8 waves");
   constexpr bool SPLIT = NTHREADS == 512;
-  constexpr int NSETS = SPLIT ? 2 : 1;
+  constexpr int NSETS = 1;
   constexpr int KL = DK / 32;
   const int st = SPLIT ? (tid & 255) : tid;
   const bool do_k = !SPLIT || tid < 256, do_v_role = !SPLIT || tid >= 256;
@@ -381,134 +551,342 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
     }
   };
 
-  // ---- prologue: everything the tile needs first is requested at once -----------------------
-  // The chunks from dstart on (same-block / causal rules) come FIRST: their addresses need no
-  // routing table, so their loads, the Q loads above and the reads of the block list are all in
-  // flight together.  The chunks of the prior attention blocks follow.
-  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;  // >= 1
-  // Only a sequence's last tile can hold chunks that reach past its end; it takes the plain loop further down.
-  const bool ragged_tile = dstart + 64 * n_diag > len;
-  if (ragged_tile) {
-    gload(std::false_type{}, dstart, sreg[0]);
-  } else {
-    gload(std::true_type{}, dstart, sreg[0]);
-    if (SPLIT && n_diag >= 2) gload(std::true_type{}, dstart + 64, sreg[NSETS - 1]);  // the second chunk too: its address needs no list
-  }
-  if (tid == 0) lds_count = 0;
-  __syncthreads();
-  {
-    // attention blocks that end at or before dstart: ids into LDS, count.  The list is sorted and
-    // holds distinct block ids, so entry j >= j: only the first dstart/Bs entries can qualify.
-    const int jmax = min(dstart / Bs, p.TN);
-    int cnt = 0;
-    for (int j = tid; j < jmax; j += NTHREADS) {
-      const int e = list[j * list_stride];
-      if (j < n_attn && (e + 1) * Bs <= dstart) {
-        ++cnt;
-        if (j < MAX_LDS_LIST) lds_list[j] = e;
-      }
-    }
-    if (cnt) atomicAdd(&lds_count, cnt);
-  }
-  // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
-  unsigned long long diag_attn;
-  {
-    const int blk = dstart / Bs + lane;
-    const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
-    diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
-  }
-  lstore(0, sreg[0]);
-  __syncthreads();
-  const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
-  const int n_iters = n_diag + n_prior_chunks;
-
-  // Chunk iterator, all wave-uniform (scalar registers): the chunks from dstart on, then the
-  // 64-key chunks of the prior attention blocks in list order.
-  int nx_it = 1, nx_j = 0, nx_sub = 0;  // chunk 0 is already staged
-  auto next_key_start = [&]() -> int {
-    int ks;
-    if (nx_it < n_diag) {
-      ks = dstart + nx_it * 64;
-    } else {
-      int e;
-      if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
-      else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
-      ks = e * Bs + nx_sub * 64;
-      if (++nx_sub == per_blk) {
-        nx_sub = 0;
-        ++nx_j;
-      }
-    }
-    ++nx_it;
-    return ks;
-  };
-
-  const float c = p.scale_log2;
+  const int n_diag = (min(len, tile_start + QTILE) - dstart + 63) >> 6;  // chunks from dstart to the end of the tile, >= 1
+  // Only a sequence's last tile can hold chunks that reach past its end (or a block so large that there are more such
+  // chunks than a lane mask holds): it takes the plain loop further down.
+  const bool ragged_tile = dstart + 64 * n_diag > len || n_diag > 63;
   const int my_blk = q0 / Bs;
-  // one chunk for this wave: the chunks from dstart on follow the same-block and causal rules, the prior attention
-  // blocks are seen whole
-  auto compute = [&](const int it, const int buf) __attribute__((always_inline)) {
-    bool active = wave_valid, causal = false;
-    if (it < n_diag) {
-      const int jc = (dstart >> 6) + it;  // absolute chunk index of the keys
-      const int kblk = (jc * 64) / Bs;
-      if (p.same_block) {
-        if (jc > my_chunk) active = false;
-        else if (jc == my_chunk) causal = true;
-        else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dstart / Bs)) & 1ull));
-      } else {
-        active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dstart / Bs)) & 1ull);
+  bool dma_done = false;
+  if constexpr (SPLIT) {
+    if (!ragged_tile) {
+      // ================= 8 waves, full tile: two wave groups half a chunk apart ===================================
+      // Waves w and w+4 share a SIMD.  Every wave runs, per chunk `it`:  softmax(it) | PV(it) | QK(it+1).  Waves 0-3
+      // ("early") meet the workgroup barrier at the end of that body, waves 4-7 ("late") in its middle, after softmax:
+      // between two barriers one wave of a SIMD does softmax, PV, QK and the other PV, QK, softmax, so the vector work of
+      // one meets the matrix work of the other.  Call sync(k) the barrier that ends the early group's body k.  Then
+      // keys of chunk c are read in (sync(c-2), sync(c)) and its values in (sync(c-1), sync(c+1)).
+      //  * K(c) lives in ring buffer c % 4.  The early waves request K(k+4) by DMA right after sync(k): the buffer it
+      //    overwrites, K(k), was last read before sync(k); it must have landed when they arrive at sync(k+2), so their
+      //    wait before a barrier leaves exactly the newest request in flight.
+      //  * V(c) lives, transposed, in ring buffer c % 3.  The late waves load V(k+3) into registers right after sync(k)
+      //    and, at the same point one chunk later, write it to LDS: V(k+2) is stored
+      //    after sync(k), into the buffer of V(k-1), last read before sync(k), and is visible from sync(k+1) on.
+      constexpr int KRING = 4, KTILE = 64 * DK * 2, VRING = 3, VTILE = DV * VTP * 2;     // bytes
+      constexpr int KI = DK / 32;                                                        // DMA instructions per early wave and chunk
+      constexpr int KROWS_I = 512 / DK;                                                  // tile rows one instruction covers
+      // (the swizzled operand addresses are formed with XOR: the ring starts on a 1 KiB boundary)
+      const unsigned lds_k = ((unsigned)(size_t)smem + 1023u) & ~1023u, lds_v = lds_k + KRING * KTILE;
+      const bool late = wave >= 4;
+      const int gw = wave & 3;  // wave within its group
+      // --- early waves: lane l of instruction i fills LDS row KROWS_I*i + l/segs, position l%segs, with the segment that belongs there
+      unsigned k_src[KI];
+#pragma unroll
+      for (int j = 0; j < KI; ++j) {
+        const int r = KROWS_I * (KI * gw + j) + lane / (DK / 8), pos = lane % (DK / 8);
+        k_src[j] = (unsigned)((size_t)r * krow * sizeof(bf16_t)) + 16u * (pos ^ (r & 7));
       }
-    }
-    if (active && !NATSL_ABL(p.dbg & 2))
-      chunk_pipelined<DK, DV>(Ks + buf * 64 * KP, Vs + buf * DV * TP, QB, acc, m_ref, l_run, c, lane, causal, qloc0);
-  };
+      auto dma_k = [&](const int ks, const int c) __attribute__((always_inline)) {
+        const char* g = reinterpret_cast<const char*>(kp + (size_t)ks * krow);
+#pragma unroll
+        for (int j = 0; j < KI; ++j) dma16(g, k_src[j], lds_k + (c & 3) * KTILE + (KI * gw + j) * 1024);
+      };
+      // --- late waves: a thread owns keys 4 kg .. 4 kg + 3 of one 8-column segment.  16 consecutive lanes take the 16
+      // key groups of one segment: their transposed 8-byte stores fill one 128-byte row, the next 16 lanes' row lies
+      // 8 rows = 1152 bytes further, on the other half of the banks.
+      const int lt = tid & 255;
+      const int v_kg = lt & 15, v_sg = lt >> 4;
+      const bool v_on = v_sg < DV / 8;   // (DV = 64: half of the late waves have nothing to stage)
+      const unsigned v_src = (unsigned)((size_t)(4 * v_kg) * vrow * sizeof(bf16_t)) + 16u * (v_on ? v_sg : 0);
+      const unsigned v_src_pitch = (unsigned)(vrow * sizeof(bf16_t));
+      // keys 4 kg .. 4 kg + 3 sit at position 4 * slot of their 16-key group, slot = 2 (q & 1) + (q >> 1), q = kg % 4:
+      // a lane of half hf then finds its k-slots (keys 4 hf .. +3 and 8 + 4 hf .. +3 of the group) in bytes 16 hf .. 16 hf + 15
+      const unsigned v_dst = (unsigned)(8 * v_sg * VTP * 2) + 32u * (v_kg >> 2) + 8u * (2 * (v_kg & 1) + ((v_kg >> 1) & 1));
+      struct VRegs { u32x4 v[4]; };
+      auto vload = [&](const int ks, VRegs& r) __attribute__((always_inline)) {
+        const char* g = reinterpret_cast<const char*>(vp + (size_t)ks * vrow) + v_src;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(g + j * v_src_pitch);
+      };
+      auto vstore = [&](const int c, const VRegs& r) __attribute__((always_inline)) {
+        if (v_on) {
+          const unsigned a = lds_v + (c % VRING) * VTILE + v_dst;
+          typedef __attribute__((address_space(3))) u32x2* lds_w;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            // value columns 2d (low halves) and 2d+1 (high halves) of the four keys
+            u32x2 lo, hi;
+            lo[0] = __builtin_amdgcn_perm(r.v[1][d], r.v[0][d], 0x05040100u);
+            lo[1] = __builtin_amdgcn_perm(r.v[3][d], r.v[2][d], 0x05040100u);
+            hi[0] = __builtin_amdgcn_perm(r.v[1][d], r.v[0][d], 0x07060302u);
+            hi[1] = __builtin_amdgcn_perm(r.v[3][d], r.v[2][d], 0x07060302u);
+            *reinterpret_cast<lds_w>(a + (2 * d) * VTP * 2) = lo;
+            *reinterpret_cast<lds_w>(a + (2 * d + 1) * VTP * 2) = hi;
+          }
+        }
+      };
+      // operand addresses of this lane inside a tile (see qk_phase / pv_phase)
+      const unsigned k_lane = (unsigned)(l32 * DK * 2) + 16u * (hf ^ (l32 & 7));
+      const unsigned v_lane = (unsigned)(l32 * VTP * 2) + 16u * hf;
 
-  if (ragged_tile) {
-    // plain loop, one chunk in flight, every row clamped to the sequence
-    int ks_fetch = dstart;
-    if (n_iters > 1) ks_fetch = next_key_start();
-    for (int it = 0; it < n_iters; ++it) {
-      const int buf = it & 1;
-      if (it + 1 < n_iters) gload(std::false_type{}, ks_fetch, sreg[0]);
-      compute(it, buf);
-      if (it + 1 < n_iters) lstore(buf ^ 1, sreg[0]);
-      if (it + 2 < n_iters) ks_fetch = next_key_start();
+      // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
+      unsigned long long diag_attn;
+      {
+        const int blk = dstart / Bs + lane;
+        const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
+        diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
+      }
+      // The first four chunks are requested before anything else when their addresses need no block list (the usual
+      // case: four or more chunks from dstart on).
+      const bool early_request = n_diag >= 4;
+      VRegs vr0, vr1;
+      if (early_request) {
+        if (!late) {
+#pragma unroll
+          for (int cc = 0; cc < 4; ++cc) dma_k(dstart + 64 * cc, cc);
+        } else {
+          vload(dstart, vr0);
+          vload(dstart + 64, vr1);
+        }
+      }
+      // attention blocks that end at or before dstart: ids into LDS.  The list is sorted and holds distinct block ids
+      // (entry j >= j), so only the first dstart/Bs entries can qualify, and those that do form a prefix.
+      __shared__ int wave_count[NWAVES];
+      {
+        const int jmax = min(dstart / Bs, p.TN);
+        int cnt = 0;
+        for (int j = tid; j < jmax; j += NTHREADS) {
+          const int e = list[j * list_stride];
+          const bool ok = j < n_attn && (e + 1) * Bs <= dstart;
+          cnt += __popcll(__ballot(ok));
+          if (ok && j < MAX_LDS_LIST) lds_list[j] = e;
+        }
+        if (lane == 0) wave_count[wave] = cnt;
+      }
       __syncthreads();
+      int n_prior = 0;
+#pragma unroll
+      for (int w2 = 0; w2 < NWAVES; ++w2) n_prior += wave_count[w2];
+      n_prior = __builtin_amdgcn_readfirstlane(n_prior);
+      const int n_iters = n_diag + n_prior * per_blk;
+
+      // chunk iterator (wave-uniform): first key of chunk nx_it, then on to the next; past the last chunk it repeats it
+      int nx_it = 0, nx_j = 0, nx_sub = 0, ks_cur = dstart;
+      auto next_chunk = [&]() __attribute__((always_inline)) -> int {
+        if (nx_it < n_iters) {
+          if (nx_it < n_diag) {
+            ks_cur = dstart + nx_it * 64;
+          } else {
+            int e;
+            if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+            else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
+            ks_cur = e * Bs + nx_sub * 64;
+            if (++nx_sub == per_blk) {
+              nx_sub = 0;
+              ++nx_j;
+            }
+          }
+        }
+        ++nx_it;
+        return ks_cur;
+      };
+      if (!late) {
+        if (early_request) {
+          nx_it = 4;
+        } else {
+#pragma unroll
+          for (int cc = 0; cc < 4; ++cc) {
+            const int ks = next_chunk();
+            if (cc < n_iters) dma_k(ks, cc);
+          }
+        }
+        // K(0) and K(1) are needed now; K(2), K(3) may stay in flight when all four were requested
+        if (n_iters >= 4) __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * KI));
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
+      } else {
+        if (early_request) {
+          nx_it = 2;
+        } else {
+          vload(next_chunk(), vr0);
+          vload(next_chunk(), vr1);
+        }
+        vstore(0, vr0);
+        vstore(1, vr1);
+        vload(next_chunk(), vr0);   // V(2): stored in the first body
+      }
+      __syncthreads();
+
+      // which of the chunks from dstart on this wave takes part in (bit it), and which one is its own, causal chunk:
+      // lane i works it out for chunk i, once
+      unsigned long long act_mask;
+      int causal_it;
+      {
+        const int jc = (dstart >> 6) + lane;  // absolute chunk index of the keys
+        const int kblk = (jc * 64) / Bs;
+        const bool typed = (diag_attn >> ((kblk - dstart / Bs) & 63)) & 1ull;
+        bool a, cz = false;
+        if (p.same_block) {
+          cz = jc == my_chunk;
+          a = cz || (jc < my_chunk && (kblk == my_blk || typed));
+        } else {
+          a = jc < my_chunk && kblk < my_blk && typed;
+        }
+        act_mask = __ballot(a && lane < n_diag);
+        const unsigned long long cm = __ballot(cz && lane < n_diag);
+        causal_it = cm ? __builtin_ctzll(cm) : -1;
+      }
+      m_ref = 0.f;       // an arbitrary finite reference until the row's first visible key sets the real one
+      float thr = -INFINITY;
+      f32x16 s0, s1;
+      bool cur_active = act_mask & 1ull;
+      if (cur_active) qk_phase<DK>(lds_k + k_lane, QB, m_ref, s0, s1);
+      auto is_active = [&](const int it) -> bool { return it < n_diag ? (act_mask >> it) & 1ull : it < n_iters; };
+
+      if (!late) {
+        for (int it = 0; it < n_iters; ++it) {
+          const bool nxt_active = is_active(it + 1);
+          bf16x8 PB[4];
+          if (cur_active) {
+            softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
+            __builtin_amdgcn_s_setprio(3);
+            pv_phase<DV>(lds_v + (it % VRING) * VTILE + v_lane, PB, acc, l_run);
+          }
+          __builtin_amdgcn_s_setprio(3);
+          if (nxt_active) qk_phase<DK>(lds_k + ((it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
+          __builtin_amdgcn_s_setprio(0);
+          // K(it+2) must have landed; the request for K(it+3) may stay in flight if there is one
+          if (it + 3 < n_iters) __builtin_amdgcn_s_waitcnt(0x0f70 | KI);
+          else __builtin_amdgcn_s_waitcnt(0x0f70);
+          __syncthreads();                                  // sync(it)
+          const int ks = next_chunk();
+          if (it + 4 < n_iters) dma_k(ks, it + 4);
+          cur_active = nxt_active;
+        }
+      } else {
+        auto body = [&](const int it, VRegs& vr) __attribute__((always_inline)) {
+          const bool nxt_active = is_active(it + 1);
+          bf16x8 PB[4];
+          if (cur_active) softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(PB[i]));   // the probabilities exist before the barrier
+          __syncthreads();                                  // sync(it)
+          __builtin_amdgcn_s_setprio(3);
+          if (cur_active) pv_phase<DV>(lds_v + (it % VRING) * VTILE + v_lane, PB, acc, l_run);
+          if (nxt_active) qk_phase<DK>(lds_k + ((it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
+          __builtin_amdgcn_s_setprio(0);
+          // the matrix phases come first, while the early waves are in their vector phase; staging follows
+          vstore(it + 2, vr);                               // V(it+2) (past the end: a repeat, into a buffer nobody reads)
+          vload(next_chunk(), vr);                          // V(it+3)
+          cur_active = nxt_active;
+        };
+        for (int it = 0; it < n_iters; ++it) body(it, vr0);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();  // the late waves finish their last PV after the early ones: the output tile below reuses the rings
+      dma_done = true;
     }
-  } else if constexpr (SPLIT) {
-    // Chunk it+2 is requested while chunk it is computed and chunk it+1 (requested one iteration earlier) is
-    // written to LDS: how long a chunk's loads take to come back no longer sets the pace of an iteration.  Every
-    // iteration issues its loads unconditionally (past the last chunk it re-reads the last one), so that the wait
-    // before the LDS writes counts exactly the loads issued after the ones it needs.
-    int ks_next = dstart;                                    // chunk 1 (a repeat of chunk 0 if there is no other)
-    if (n_iters > 1) ks_next = next_key_start();
-    if (n_diag < 2) gload(std::true_type{}, ks_next, sreg[NSETS - 1]);
-    if (n_iters > 2) ks_next = next_key_start();             // chunk 2
-    auto step = [&](auto parity, const int it) __attribute__((always_inline)) {
-      constexpr int P = decltype(parity)::value;
-      if (!NATSL_ABL(p.dbg & 1)) gload(std::true_type{}, ks_next, sreg[P % NSETS]);
-      compute(it, P);
-      if (it + 1 < n_iters && !NATSL_ABL(p.dbg & 1)) lstore(P ^ 1, sreg[(P ^ 1) % NSETS]);
-      if (it + 3 < n_iters) ks_next = next_key_start();
-      if (!NATSL_ABL(p.dbg & 4)) __syncthreads();
+  }
+  if (!dma_done) {
+    // ---- prologue: everything the tile needs first is requested at once -----------------------
+    // The chunks from dstart on (same-block / causal rules) come FIRST: their addresses need no
+    // routing table, so their loads, the Q loads above and the reads of the block list are all in
+    // flight together.  The chunks of the prior attention blocks follow.
+    if (ragged_tile) {
+      gload(std::false_type{}, dstart, sreg[0]);
+    } else {
+      gload(std::true_type{}, dstart, sreg[0]);
+    }
+    if (tid == 0) lds_count = 0;
+    __syncthreads();
+    {
+      // attention blocks that end at or before dstart: ids into LDS, count.  The list is sorted and
+      // holds distinct block ids, so entry j >= j: only the first dstart/Bs entries can qualify.
+      const int jmax = min(dstart / Bs, p.TN);
+      int cnt = 0;
+      for (int j = tid; j < jmax; j += NTHREADS) {
+        const int e = list[j * list_stride];
+        if (j < n_attn && (e + 1) * Bs <= dstart) {
+          ++cnt;
+          if (j < MAX_LDS_LIST) lds_list[j] = e;
+        }
+      }
+      if (cnt) atomicAdd(&lds_count, cnt);
+    }
+    // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
+    unsigned long long diag_attn;
+    {
+      const int blk = dstart / Bs + lane;
+      const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
+      diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
+    }
+    lstore(0, sreg[0]);
+    __syncthreads();
+    const int n_prior_chunks = __builtin_amdgcn_readfirstlane(lds_count) * per_blk;
+    const int n_iters = n_diag + n_prior_chunks;
+
+    // Chunk iterator, all wave-uniform (scalar registers): the chunks from dstart on, then the
+    // 64-key chunks of the prior attention blocks in list order.
+    int nx_it = 1, nx_j = 0, nx_sub = 0;  // chunk 0 is already staged
+    auto next_key_start = [&]() -> int {
+      int ks;
+      if (nx_it < n_diag) {
+        ks = dstart + nx_it * 64;
+      } else {
+        int e;
+        if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+        else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
+        ks = e * Bs + nx_sub * 64;
+        if (++nx_sub == per_blk) {
+          nx_sub = 0;
+          ++nx_j;
+        }
+      }
+      ++nx_it;
+      return ks;
     };
-    int it = 0;
-    for (; it + 1 < n_iters; it += 2) {
-      step(std::integral_constant<int, 0>{}, it);
-      step(std::integral_constant<int, 1>{}, it + 1);
-    }
-    if (it < n_iters) step(std::integral_constant<int, 0>{}, it);
-  } else {
-    int ks_fetch = dstart;  // key start of the chunk the next loads bring in (past the last chunk: a repeat)
-    if (n_iters > 1) ks_fetch = next_key_start();
-    for (int it = 0; it < n_iters; ++it) {
-      const int buf = it & 1;
-      gload(std::true_type{}, ks_fetch, sreg[0]);
-      compute(it, buf);
-      if (it + 1 < n_iters) lstore(buf ^ 1, sreg[0]);
-      if (it + 2 < n_iters) ks_fetch = next_key_start();
-      __syncthreads();
+
+    constexpr float c = 1.f;  // the scale is already in the queries
+    // one chunk for this wave: the chunks from dstart on follow the same-block and causal rules, the prior attention
+    // blocks are seen whole
+    auto compute = [&](const int it, const int buf) __attribute__((always_inline)) {
+      bool active = wave_valid, causal = false;
+      if (it < n_diag) {
+        const int jc = (dstart >> 6) + it;  // absolute chunk index of the keys
+        const int kblk = (jc * 64) / Bs;
+        if (p.same_block) {
+          if (jc > my_chunk) active = false;
+          else if (jc == my_chunk) causal = true;
+          else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dstart / Bs)) & 1ull));
+        } else {
+          active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dstart / Bs)) & 1ull);
+        }
+      }
+      if (active && !NATSL_ABL(p.dbg & 2))
+        chunk_pipelined<DK, DV>(Ks + buf * 64 * KP, Vs + buf * DV * TP, QB, acc, m_ref, l_run, c, lane, causal, qloc0);
+    };
+
+    if (ragged_tile) {
+      // plain loop, one chunk in flight, every row clamped to the sequence
+      int ks_fetch = dstart;
+      if (n_iters > 1) ks_fetch = next_key_start();
+      for (int it = 0; it < n_iters; ++it) {
+        const int buf = it & 1;
+        if (it + 1 < n_iters) gload(std::false_type{}, ks_fetch, sreg[0]);
+        compute(it, buf);
+        if (it + 1 < n_iters) lstore(buf ^ 1, sreg[0]);
+        if (it + 2 < n_iters) ks_fetch = next_key_start();
+        __syncthreads();
+      }
+    } else {
+      int ks_fetch = dstart;  // key start of the chunk the next loads bring in (past the last chunk: a repeat)
+      if (n_iters > 1) ks_fetch = next_key_start();
+      for (int it = 0; it < n_iters; ++it) {
+        const int buf = it & 1;
+        gload(std::true_type{}, ks_fetch, sreg[0]);
+        compute(it, buf);
+        if (it + 1 < n_iters) lstore(buf ^ 1, sreg[0]);
+        if (it + 2 < n_iters) ks_fetch = next_key_start();
+        __syncthreads();
+      }
     }
   }
 
@@ -552,6 +930,8 @@ static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   size_t lds = (size_t)2 * (64 * KP + DV * VT_PITCH) * sizeof(bf16_t);
   const size_t epi = (size_t)QTILE * VP * sizeof(bf16_t);
   if (epi > lds) lds = epi;
+  const size_t ring = ((size_t)4 * 64 * DK + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;  // 8 waves: four K tiles and three transposed V tiles, 1 KiB aligned
+  if (NWAVES == 8 && ring > lds) lds = ring;
   auto kern = softmax_sparse_fwd_kernel<DK, DV, NWAVES>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
