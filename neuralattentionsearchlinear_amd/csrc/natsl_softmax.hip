@@ -568,14 +568,15 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       //  * K(c) lives in ring buffer c % 4.  The early waves request K(k+4) by DMA right after sync(k): the buffer it
       //    overwrites, K(k), was last read before sync(k); it must have landed when they arrive at sync(k+2), so their
       //    wait before a barrier leaves exactly the newest request in flight.
-      //  * V(c) lives, transposed, in ring buffer c % 3.  The late waves load V(k+3) into registers right after sync(k)
-      //    and, at the same point one chunk later, write it to LDS: V(k+2) is stored
+      //  * V(c) first lands row-major ("raw", buffer c % 2), also by DMA from the early waves: V(k+3) is requested right
+      //    after sync(k), ahead of K(k+4), and must have landed when they arrive at sync(k+1).  The late waves then
+      //    transpose it from LDS to LDS into ring buffer c % 3: V(k+2) is stored
       //    after sync(k), into the buffer of V(k-1), last read before sync(k), and is visible from sync(k+1) on.
-      constexpr int KRING = 4, KTILE = 64 * DK * 2, VRING = 3, VTILE = DV * VTP * 2;     // bytes
-      constexpr int KI = DK / 32;                                                        // DMA instructions per early wave and chunk
-      constexpr int KROWS_I = 512 / DK;                                                  // tile rows one instruction covers
+      constexpr int KRING = 4, KTILE = 64 * DK * 2, VRING = 3, VTILE = DV * VTP * 2, RTILE = 64 * DV * 2;   // bytes
+      constexpr int KI = DK / 32, RI = DV / 32;                                          // DMA instructions per early wave and chunk
+      constexpr int KROWS_I = 512 / DK, RROWS_I = 512 / DV;                              // tile rows one instruction covers
       // (the swizzled operand addresses are formed with XOR: the ring starts on a 1 KiB boundary)
-      const unsigned lds_k = ((unsigned)(size_t)smem + 1023u) & ~1023u, lds_v = lds_k + KRING * KTILE;
+      const unsigned lds_k = ((unsigned)(size_t)smem + 1023u) & ~1023u, lds_r = lds_k + KRING * KTILE, lds_v = lds_r + 2 * RTILE;
       const bool late = wave >= 4;
       const int gw = wave & 3;  // wave within its group
       // --- early waves: lane l of instruction i fills LDS row KROWS_I*i + l/segs, position l%segs, with the segment that belongs there
@@ -585,6 +586,19 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
         const int r = KROWS_I * (KI * gw + j) + lane / (DK / 8), pos = lane % (DK / 8);
         k_src[j] = (unsigned)((size_t)r * krow * sizeof(bf16_t)) + 16u * (pos ^ (r & 7));
       }
+      // raw V: segment s of row r sits at s ^ ((r >> 2) & 15), so that the 16 lanes of a transposing thread group (16
+      // key groups = rows 4 apart, one segment) read 16 different 16-byte slots
+      unsigned r_src[RI];
+#pragma unroll
+      for (int j = 0; j < RI; ++j) {
+        const int r = RROWS_I * (RI * gw + j) + lane / (DV / 8), pos = lane % (DV / 8);
+        r_src[j] = (unsigned)((size_t)r * vrow * sizeof(bf16_t)) + 16u * (pos ^ ((r >> 2) & (DV / 8 - 1)));
+      }
+      auto dma_r = [&](const int ks, const int c) __attribute__((always_inline)) {
+        const char* g = reinterpret_cast<const char*>(vp + (size_t)ks * vrow);
+#pragma unroll
+        for (int j = 0; j < RI; ++j) dma16(g, r_src[j], lds_r + (c & 1) * RTILE + (RI * gw + j) * 1024);
+      };
       auto dma_k = [&](const int ks, const int c) __attribute__((always_inline)) {
         const char* g = reinterpret_cast<const char*>(kp + (size_t)ks * krow);
 #pragma unroll
@@ -596,29 +610,29 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       const int lt = tid & 255;
       const int v_kg = lt & 15, v_sg = lt >> 4;
       const bool v_on = v_sg < DV / 8;   // (DV = 64: half of the late waves have nothing to stage)
-      const unsigned v_src = (unsigned)((size_t)(4 * v_kg) * vrow * sizeof(bf16_t)) + 16u * (v_on ? v_sg : 0);
-      const unsigned v_src_pitch = (unsigned)(vrow * sizeof(bf16_t));
+      // raw tile: rows 4 kg .. 4 kg + 3, segment sg (swizzled)
+      const unsigned v_raw = (unsigned)(4 * v_kg * DV * 2) + 16u * ((v_on ? v_sg : 0) ^ (v_kg & (DV / 8 - 1)));
       // keys 4 kg .. 4 kg + 3 sit at position 4 * slot of their 16-key group, slot = 2 (q & 1) + (q >> 1), q = kg % 4:
       // a lane of half hf then finds its k-slots (keys 4 hf .. +3 and 8 + 4 hf .. +3 of the group) in bytes 16 hf .. 16 hf + 15
       const unsigned v_dst = (unsigned)(8 * v_sg * VTP * 2) + 32u * (v_kg >> 2) + 8u * (2 * (v_kg & 1) + ((v_kg >> 1) & 1));
-      struct VRegs { u32x4 v[4]; };
-      auto vload = [&](const int ks, VRegs& r) __attribute__((always_inline)) {
-        const char* g = reinterpret_cast<const char*>(vp + (size_t)ks * vrow) + v_src;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) r.v[j] = *reinterpret_cast<const u32x4*>(g + j * v_src_pitch);
-      };
-      auto vstore = [&](const int c, const VRegs& r) __attribute__((always_inline)) {
+      auto transpose_v = [&](const int c) __attribute__((always_inline)) {
         if (v_on) {
-          const unsigned a = lds_v + (c % VRING) * VTILE + v_dst;
+          typedef __attribute__((address_space(3))) const u32x4* lds_r4;
           typedef __attribute__((address_space(3))) u32x2* lds_w;
+          unsigned src = lds_r + (c & 1) * RTILE + v_raw;
+          asm("" : "+v"(src));
+          u32x4 rv[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) rv[j] = *reinterpret_cast<lds_r4>(src + j * DV * 2);
+          const unsigned a = lds_v + (c % VRING) * VTILE + v_dst;
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             // value columns 2d (low halves) and 2d+1 (high halves) of the four keys
             u32x2 lo, hi;
-            lo[0] = __builtin_amdgcn_perm(r.v[1][d], r.v[0][d], 0x05040100u);
-            lo[1] = __builtin_amdgcn_perm(r.v[3][d], r.v[2][d], 0x05040100u);
-            hi[0] = __builtin_amdgcn_perm(r.v[1][d], r.v[0][d], 0x07060302u);
-            hi[1] = __builtin_amdgcn_perm(r.v[3][d], r.v[2][d], 0x07060302u);
+            lo[0] = __builtin_amdgcn_perm(rv[1][d], rv[0][d], 0x05040100u);
+            lo[1] = __builtin_amdgcn_perm(rv[3][d], rv[2][d], 0x05040100u);
+            hi[0] = __builtin_amdgcn_perm(rv[1][d], rv[0][d], 0x07060302u);
+            hi[1] = __builtin_amdgcn_perm(rv[3][d], rv[2][d], 0x07060302u);
             *reinterpret_cast<lds_w>(a + (2 * d) * VTP * 2) = lo;
             *reinterpret_cast<lds_w>(a + (2 * d + 1) * VTP * 2) = hi;
           }
@@ -628,25 +642,22 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       const unsigned k_lane = (unsigned)(l32 * DK * 2) + 16u * (hf ^ (l32 & 7));
       const unsigned v_lane = (unsigned)(l32 * VTP * 2) + 16u * hf;
 
+      // The first four chunks are requested before anything else when their addresses need no block list (the usual
+      // case: four or more chunks from dstart on).
+      // Request order of the early waves: K(0), V(0), K(1), V(1); K(2) after the first barrier; V(2), K(3) after the second.
+      const bool early_request = n_diag >= 4;
+      if (early_request && !late) {
+        dma_k(dstart, 0);
+        dma_r(dstart, 0);
+        dma_k(dstart + 64, 1);
+        dma_r(dstart + 64, 1);
+      }
       // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
       unsigned long long diag_attn;
       {
         const int blk = dstart / Bs + lane;
         const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
         diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
-      }
-      // The first four chunks are requested before anything else when their addresses need no block list (the usual
-      // case: four or more chunks from dstart on).
-      const bool early_request = n_diag >= 4;
-      VRegs vr0, vr1;
-      if (early_request) {
-        if (!late) {
-#pragma unroll
-          for (int cc = 0; cc < 4; ++cc) dma_k(dstart + 64 * cc, cc);
-        } else {
-          vload(dstart, vr0);
-          vload(dstart + 64, vr1);
-        }
       }
       // attention blocks that end at or before dstart: ids into LDS.  The list is sorted and holds distinct block ids
       // (entry j >= j), so only the first dstart/Bs entries can qualify, and those that do form a prefix.
@@ -671,13 +682,16 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
 
       // chunk iterator (wave-uniform): first key of chunk nx_it, then on to the next; past the last chunk it repeats it
       int nx_it = 0, nx_j = 0, nx_sub = 0, ks_cur = dstart;
-      auto next_chunk = [&]() __attribute__((always_inline)) -> int {
+      // (in the loop the list entry is read from LDS at the top of the body, `ahead`, and used at its end: the
+      // iterator only moves in between)
+      auto list_ahead = [&]() -> int { return lds_list[min(nx_j, MAX_LDS_LIST - 1)]; };
+      auto next_chunk = [&](const int ahead = 0, const bool have_ahead = false) __attribute__((always_inline)) -> int {
         if (nx_it < n_iters) {
           if (nx_it < n_diag) {
             ks_cur = dstart + nx_it * 64;
           } else {
             int e;
-            if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(lds_list[nx_j]);
+            if (nx_j < MAX_LDS_LIST) e = __builtin_amdgcn_readfirstlane(have_ahead ? ahead : lds_list[nx_j]);
             else e = __builtin_amdgcn_readfirstlane(list[nx_j * list_stride]);
             ks_cur = e * Bs + nx_sub * 64;
             if (++nx_sub == per_blk) {
@@ -689,31 +703,39 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
         ++nx_it;
         return ks_cur;
       };
+      int ks_v = dstart;   // first key of the chunk whose raw V is requested next (one chunk behind the K requests)
       if (!late) {
-        if (early_request) {
-          nx_it = 4;
-        } else {
-#pragma unroll
-          for (int cc = 0; cc < 4; ++cc) {
-            const int ks = next_chunk();
-            if (cc < n_iters) dma_k(ks, cc);
-          }
-        }
-        // K(0) and K(1) are needed now; K(2), K(3) may stay in flight when all four were requested
-        if (n_iters >= 4) __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * KI));
-        else __builtin_amdgcn_s_waitcnt(0x0f70);
-      } else {
         if (early_request) {
           nx_it = 2;
         } else {
-          vload(next_chunk(), vr0);
-          vload(next_chunk(), vr1);
+          int ks = next_chunk();
+          dma_k(ks, 0);
+          dma_r(ks, 0);
+          ks = next_chunk();
+          if (1 < n_iters) {
+            dma_k(ks, 1);
+            dma_r(ks, 1);
+          }
         }
-        vstore(0, vr0);
-        vstore(1, vr1);
-        vload(next_chunk(), vr0);   // V(2): stored in the first body
+        // raw V(0), V(1) (and K(0), K(1)) must have landed for the transposition below
+        __builtin_amdgcn_s_waitcnt(0x0f70);
       }
       __syncthreads();
+      if (!late) {
+        ks_v = next_chunk();                      // chunk 2
+        if (2 < n_iters) dma_k(ks_v, 2);
+      } else {
+        transpose_v(0);
+        if (1 < n_iters) transpose_v(1);
+      }
+      __syncthreads();                            // "sync(-1)"
+      if (!late) {
+        // raw V(2) only now: its buffer held raw V(0) until the barrier.  Like every later request pair it is followed
+        // by the K request that may stay in flight at the next barrier.
+        if (2 < n_iters) dma_r(ks_v, 2);
+        ks_v = next_chunk();                      // chunk 3
+        if (3 < n_iters) dma_k(ks_v, 3);
+      }
 
       // which of the chunks from dstart on this wave takes part in (bit it), and which one is its own, causal chunk:
       // lane i works it out for chunk i, once
@@ -744,6 +766,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       if (!late) {
         for (int it = 0; it < n_iters; ++it) {
           const bool nxt_active = is_active(it + 1);
+          const int ahead = list_ahead();
           bf16x8 PB[4];
           if (cur_active) {
             softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
@@ -753,16 +776,17 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
           __builtin_amdgcn_s_setprio(3);
           if (nxt_active) qk_phase<DK>(lds_k + ((it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
           __builtin_amdgcn_s_setprio(0);
-          // K(it+2) must have landed; the request for K(it+3) may stay in flight if there is one
+          // K(it+2) and raw V(it+2) must have landed; the request for K(it+3), the newest, may stay in flight if there is one
           if (it + 3 < n_iters) __builtin_amdgcn_s_waitcnt(0x0f70 | KI);
           else __builtin_amdgcn_s_waitcnt(0x0f70);
           __syncthreads();                                  // sync(it)
-          const int ks = next_chunk();
-          if (it + 4 < n_iters) dma_k(ks, it + 4);
+          if (it + 3 < n_iters) dma_r(ks_v, it + 3);        // raw V first: it has one interval to land, K has two
+          ks_v = next_chunk(ahead, true);
+          if (it + 4 < n_iters) dma_k(ks_v, it + 4);
           cur_active = nxt_active;
         }
       } else {
-        auto body = [&](const int it, VRegs& vr) __attribute__((always_inline)) {
+        for (int it = 0; it < n_iters; ++it) {
           const bool nxt_active = is_active(it + 1);
           bf16x8 PB[4];
           if (cur_active) softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
@@ -773,12 +797,10 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
           if (cur_active) pv_phase<DV>(lds_v + (it % VRING) * VTILE + v_lane, PB, acc, l_run);
           if (nxt_active) qk_phase<DK>(lds_k + ((it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
           __builtin_amdgcn_s_setprio(0);
-          // the matrix phases come first, while the early waves are in their vector phase; staging follows
-          vstore(it + 2, vr);                               // V(it+2) (past the end: a repeat, into a buffer nobody reads)
-          vload(next_chunk(), vr);                          // V(it+3)
+          // the matrix phases come first, while the early waves are in their vector phase; the transposition follows
+          if (it + 2 < n_iters) transpose_v(it + 2);
           cur_active = nxt_active;
-        };
-        for (int it = 0; it < n_iters; ++it) body(it, vr0);
+        }
       }
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();  // the late waves finish their last PV after the early ones: the output tile below reuses the rings
@@ -930,7 +952,7 @@ static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   size_t lds = (size_t)2 * (64 * KP + DV * VT_PITCH) * sizeof(bf16_t);
   const size_t epi = (size_t)QTILE * VP * sizeof(bf16_t);
   if (epi > lds) lds = epi;
-  const size_t ring = ((size_t)4 * 64 * DK + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;  // 8 waves: four K tiles and three transposed V tiles, 1 KiB aligned
+  const size_t ring = ((size_t)4 * 64 * DK + (size_t)2 * 64 * DV + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;  // 8 waves: four K tiles, two raw and three transposed V tiles, 1 KiB aligned
   if (NWAVES == 8 && ring > lds) lds = ring;
   auto kern = softmax_sparse_fwd_kernel<DK, DV, NWAVES>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
