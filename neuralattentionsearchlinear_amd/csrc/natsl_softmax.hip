@@ -33,6 +33,7 @@ struct SoftmaxParams {
   float scale_log2;
   int same_block;
   int variant;  // 4: 128-query tile on 4 waves, 8: 256-query tile on 8 waves
+  int g_kv, g_n;  // query heads per kv head / per selector head
   int dbg;      // ablation bits, always 0 unless built with NATSL_ABLATE
 };
 
@@ -392,14 +393,17 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   if (p.seqs == nullptr) {
     // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD whole (batch, head) pairs,
     // heaviest tile first, so the tiles that share one pair's K/V run together on one L2.
-    const int n_pairs = p.B * p.HQ;
-    const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
-    const int nq_tiles = (p.T + QTILE - 1) / QTILE;
-    const int pair = (j / nq_tiles) * 8 + xcd;
+    // (unsigned arithmetic throughout: a signed division by a run-time value costs a third more scalar instructions,
+    // and this preamble is what every tile starts with)
+    const unsigned n_pairs = (unsigned)(p.B * p.HQ);
+    const unsigned xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const unsigned nq_tiles = ((unsigned)p.T + QTILE - 1) / QTILE;
+    const unsigned jq = j / nq_tiles;
+    const unsigned pair = jq * 8 + xcd;
     if (pair >= n_pairs) return;
-    tile = nq_tiles - 1 - j % nq_tiles;
-    n = pair / p.HQ;
-    hq = pair % p.HQ;
+    tile = (int)(nq_tiles - 1 - (j - jq * nq_tiles));
+    n = (int)(pair / (unsigned)p.HQ);
+    hq = (int)(pair - (unsigned)n * (unsigned)p.HQ);
     bos = n * p.T;
     len = p.T;
     bos_nats = n * p.TN;
@@ -416,14 +420,15 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
     bos_nats = p.seqs[n].bos_nats;
   }
   const int Bs = p.block, per_blk = Bs >> 6;
-  const int hkv = hq / (p.HQ / p.HKV), hn = hq / (p.HQ / p.HN);
+  const int hkv = (int)((unsigned)hq / (unsigned)p.g_kv), hn = (int)((unsigned)hq / (unsigned)p.g_n);
   const int tile_start = tile * QTILE;
   const int q0 = tile_start + wave * QW;      // this wave's first query
   const int my_chunk = q0 >> 6;               // the 64-key chunk of the sequence that holds them
   const int qloc0 = q0 & 63;                  // ... and where in that chunk
   // keys from here on are handled chunk by chunk with the same-block / causal rules: the start of
   // the tile, or of the selector block it falls into when blocks are larger than the tile
-  const int dstart = (tile_start / p.block) * p.block;
+  const int dstart = (int)(((unsigned)tile_start / (unsigned)p.block) * (unsigned)p.block);
+  const int dblk = (int)((unsigned)dstart / (unsigned)p.block);   // the selector block dstart begins
   const bool wave_valid = q0 < len;
 
   const bf16_t* qp = p.q + ((size_t)bos * p.HQ + hq) * DK;
@@ -555,7 +560,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   // Only a sequence's last tile can hold chunks that reach past its end (or a block so large that there are more such
   // chunks than a lane mask holds): it takes the plain loop further down.
   const bool ragged_tile = dstart + 64 * n_diag > len || n_diag > 63;
-  const int my_blk = q0 / Bs;
+  const int my_blk = (int)((unsigned)q0 / (unsigned)Bs);
   bool dma_done = false;
   if constexpr (SPLIT) {
     if (!ragged_tile) {
@@ -655,7 +660,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
       unsigned long long diag_attn;
       {
-        const int blk = dstart / Bs + lane;
+        const int blk = dblk + lane;
         const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
         diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
       }
@@ -663,7 +668,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       // (entry j >= j), so only the first dstart/Bs entries can qualify, and those that do form a prefix.
       __shared__ int wave_count[NWAVES];
       {
-        const int jmax = min(dstart / Bs, p.TN);
+        const int jmax = min(dblk, p.TN);
         int cnt = 0;
         for (int j = tid; j < jmax; j += NTHREADS) {
           const int e = list[j * list_stride];
@@ -743,8 +748,8 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       int causal_it;
       {
         const int jc = (dstart >> 6) + lane;  // absolute chunk index of the keys
-        const int kblk = (jc * 64) / Bs;
-        const bool typed = (diag_attn >> ((kblk - dstart / Bs) & 63)) & 1ull;
+        const int kblk = (int)((unsigned)(jc * 64) / (unsigned)Bs);
+        const bool typed = (diag_attn >> ((kblk - dblk) & 63)) & 1ull;
         bool a, cz = false;
         if (p.same_block) {
           cz = jc == my_chunk;
@@ -822,7 +827,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
     {
       // attention blocks that end at or before dstart: ids into LDS, count.  The list is sorted and
       // holds distinct block ids, so entry j >= j: only the first dstart/Bs entries can qualify.
-      const int jmax = min(dstart / Bs, p.TN);
+      const int jmax = min(dblk, p.TN);
       int cnt = 0;
       for (int j = tid; j < jmax; j += NTHREADS) {
         const int e = list[j * list_stride];
@@ -836,7 +841,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
     // types of the blocks the chunks from dstart on fall into, as a bit mask (bit i = block dstart/Bs + i)
     unsigned long long diag_attn;
     {
-      const int blk = dstart / Bs + lane;
+      const int blk = dblk + lane;
       const bool in_range = lane < n_diag && (size_t)blk * Bs < (size_t)min(len, tile_start + QTILE);
       diag_attn = __ballot(in_range && type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + blk) * p.HN + hn) * 2));
     }
@@ -873,13 +878,13 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       bool active = wave_valid, causal = false;
       if (it < n_diag) {
         const int jc = (dstart >> 6) + it;  // absolute chunk index of the keys
-        const int kblk = (jc * 64) / Bs;
+        const int kblk = (int)((unsigned)(jc * 64) / (unsigned)Bs);
         if (p.same_block) {
           if (jc > my_chunk) active = false;
           else if (jc == my_chunk) causal = true;
-          else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dstart / Bs)) & 1ull));
+          else active = active && (kblk == my_blk || ((diag_attn >> (kblk - dblk)) & 1ull));
         } else {
-          active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dstart / Bs)) & 1ull);
+          active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dblk)) & 1ull);
         }
       }
       if (active && !NATSL_ABL(p.dbg & 2))
@@ -993,6 +998,8 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.total_tiles = seqs ? total_units : B * p.nq_tiles;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.same_block = same_block_visible ? 1 : 0;
+  p.g_kv = HQ / HKV;
+  p.g_n = HQ / HN;
   p.dbg = 0;
   // 256-query tiles on 8 waves (two chunks in flight per thread) once there are enough of them to fill the GPU twice
   p.variant = (long long)B * HQ * cdiv(T, 256) >= 512 ? 8 : 4;
