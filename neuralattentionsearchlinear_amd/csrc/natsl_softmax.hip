@@ -1,11 +1,15 @@
 // Softmax branch: sparse-KV causal flash attention for gfx950.
 //
 // One workgroup owns a tile of 32 queries per wave (4 waves: 128 queries, 8 waves: 256) of one (sequence, query
-// head).  Key/value chunks of 64 tokens stream through LDS (double buffered): first the tile's own chunks with the
-// causal / same-block rules, then every earlier block typed "attention" (taken from the sorted block list).
+// head).  Key/value chunks of 64 tokens stream through LDS: first the tile's own chunks with the causal / same-block
+// rules, then every earlier block typed "attention" (taken from the sorted block list).
 // Scores are computed transposed, S^T = K Q^T, so that a lane owns one query column: the online-softmax
 // statistics are per-lane scalars and the probabilities already sit in the B-operand layout of the second
-// product O^T = V^T P^T.  V is staged transposed in LDS, so the V^T operand is two 8-byte reads per lane.
+// product O^T = V^T P^T.  V is staged transposed in LDS.
+// Two ways through a tile: chunk_pipelined() (4 waves, and the ragged last tile of a sequence on 8 waves: K and V
+// staged through registers, double buffered, one chunk as one pipelined instruction stream per wave) and, for full
+// tiles on 8 waves, the three-phase schedule further down (K and V by LDS-DMA, the two waves of a SIMD half a chunk
+// apart).
 #include "natsl_device.h"
 #include "natsl_host.h"
 #include <type_traits>
