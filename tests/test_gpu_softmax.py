@@ -76,6 +76,20 @@ def test_softmax_wide_tiles_large_blocks(block):
     _run(4, 1024, 32, 32, 32, 128, 64, block, 0.5, False, seed=27)
 
 
+@pytest.mark.parametrize("T", [64, 128, 192, 256, 320, 576])
+def test_softmax_wide_tiles_short_sequences(T):
+    """8-wave shape on sequences of one to three tiles: fewer chunks than the staging rings hold, waves with no query
+    at all (T < 256), a full tile followed by a ragged one (320, 576)."""
+    _run(16, T, 32, 32, 32, 128, 128, 64, 0.5, True, seed=40 + T)
+    _run(16, T, 32, 16, 8, 64, 128, 64, 0.5, False, seed=41 + T)
+
+
+def test_softmax_wide_tiles_block_of_three_chunks():
+    """Selector blocks of 192 tokens: blocks do not line up with the 256-query tiles and hold an odd number of chunks."""
+    _run(4, 1536, 32, 32, 32, 128, 128, 192, 0.5, True, seed=50)
+    _run(4, 1536, 32, 8, 8, 128, 64, 192, 0.5, False, seed=51)
+
+
 def test_softmax_wide_tiles_packed():
     """Packed sequences on the 8-wave shape: every sequence attends within itself; sequence ends fall inside tiles."""
     from neuralattentionsearchlinear_amd import nats_util
