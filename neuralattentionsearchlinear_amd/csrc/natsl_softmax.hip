@@ -230,8 +230,9 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
 // K chunks go from global memory straight into LDS (global_load_lds_dwordx4: every lane names 16 source bytes, the
 // wave's 1 KiB lands contiguously at the LDS address in M0): no staging registers, no LDS store instructions.  The K
 // tile is row-major, [64 keys][DK] without padding; bank conflicts are avoided by an XOR swizzle of the 16-byte
-// segments of a row (segment s of row r sits at s ^ (r & 7): the operand read is ds_read_b128, 8 lanes = 8 rows per
-// clock), applied on the way in by letting each lane fetch the segment that belongs at its LDS position.
+// segments of a row, applied on the way in by letting each lane fetch the segment that belongs at its LDS position.
+// The operand read is ds_read_b128, 16 lanes = 16 rows = 256 bytes per clock: with DK = 128 (one row = all 64 banks)
+// segment s of row r sits at s ^ (r & 15); with DK = 64 (two rows share the banks) at s ^ ((r >> 1) & 7).
 // V has to be transposed on the way (the matrix instruction wants 8 consecutive keys per lane, memory has 8
 // consecutive value columns), which the DMA cannot do: it passes through registers (4x8 transposes with v_perm_b32).
 // The two waves that share a SIMD run half a chunk apart (see the kernel), so a wave's vector phase (softmax_phase)
@@ -245,20 +246,20 @@ NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned ld
 // S^T = K Q^T - m_ref for both key halves of one chunk: the accumulators start from minus the reference maximum of the
 // lane's query, so the scores come out of the matrix pipe already shifted.  The halves alternate so that consecutive
 // instructions are independent.  kaddr: LDS byte address of this lane's row (lane%32) in the tile, plus 16*((lane>>5) ^
-// (lane & 7)): XOR-ing it with 32*(k-step & 3) gives the swizzled position of the lane's 16 bytes of that k-step.
+// swizzle(row)): XOR-ing it with 32*(k-step) gives the swizzled position of the lane's 16 bytes of that k-step.
 template <int DK>
 NATSL_DEVICE void qk_phase(const unsigned kaddr, const bf16x8 (&QB)[DK / 16], const float m_ref, f32x16& s0, f32x16& s1) {
   constexpr int N = DK / 8, A = OPERANDS_AHEAD;
   typedef __attribute__((address_space(3))) const bf16x8* lds_op;
-  unsigned base[4];  // one register per swizzle value, opaque to the compiler (see pv_phase)
+  unsigned base[DK / 16];  // one register per k-step, opaque to the compiler (see pv_phase)
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
+  for (int q = 0; q < DK / 16; ++q) {
     base[q] = kaddr ^ (32u * q);
     asm("" : "+v"(base[q]));
   }
   auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
     const int st = j >> 1, half = j & 1;
-    return *reinterpret_cast<lds_op>(base[st & 3] + 128u * (st >> 2) + half * 32u * (2u * DK));
+    return *reinterpret_cast<lds_op>(base[st] + half * 32u * (2u * DK));
   };
   bf16x8 op[N + A];
 #pragma unroll
@@ -593,7 +594,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
 #pragma unroll
       for (int j = 0; j < KI; ++j) {
         const int r = KROWS_I * (KI * gw + j) + lane / (DK / 8), pos = lane % (DK / 8);
-        k_src[j] = (unsigned)((size_t)r * krow * sizeof(bf16_t)) + 16u * (pos ^ (r & 7));
+        k_src[j] = (unsigned)((size_t)r * krow * sizeof(bf16_t)) + 16u * (pos ^ (DK == 128 ? (r & 15) : ((r >> 1) & 7)));
       }
       // raw V: segment s of row r sits at s ^ ((r >> 2) & 15), so that the 16 lanes of a transposing thread group (16
       // key groups = rows 4 apart, one segment) read 16 different 16-byte slots
@@ -648,7 +649,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
         }
       };
       // operand addresses of this lane inside a tile (see qk_phase / pv_phase)
-      const unsigned k_lane = (unsigned)(l32 * DK * 2) + 16u * (hf ^ (l32 & 7));
+      const unsigned k_lane = (unsigned)(l32 * DK * 2) + 16u * (hf ^ (DK == 128 ? (l32 & 15) : ((l32 >> 1) & 7)));
       const unsigned v_lane = (unsigned)(l32 * VTP * 2) + 16u * hf;
 
       // The first four chunks are requested before anything else when their addresses need no block list (the usual
