@@ -1006,8 +1006,9 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.g_kv = HQ / HKV;
   p.g_n = HQ / HN;
   p.dbg = 0;
-  // 256-query tiles on 8 waves (two chunks in flight per thread) once there are enough of them to fill the GPU twice
-  p.variant = (long long)B * HQ * cdiv(T, 256) >= 512 ? 8 : 4;
+  // 256-query tiles on 8 waves once there is at least one of them per CU (measured: from there on that shape is the
+  // faster one; below, the 128-query tiles fill more CUs)
+  p.variant = (long long)B * HQ * cdiv(T, 256) >= 256 ? 8 : 4;
 #ifdef NATSL_ABLATE
   if (getenv("NATSL_DBG")) p.dbg = atoi(getenv("NATSL_DBG"));
   if (getenv("NATSL_SOFTMAX_WAVES")) p.variant = atoi(getenv("NATSL_SOFTMAX_WAVES"));

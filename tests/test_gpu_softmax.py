@@ -55,7 +55,7 @@ def test_softmax_all_attention_and_all_linear():
     _run(1, 512, 2, 2, 2, 128, 128, 64, 0.0, False, seed=11)
 
 
-# ---- the 256-query tile on 8 waves: chosen once B*HQ*ceil(T/256) >= 512, which the cases above never reach ----
+# ---- the 256-query tile on 8 waves: chosen once B*HQ*ceil(T/256) >= 256, which the cases above never reach ----
 @pytest.mark.parametrize("same_block", [True, False])
 @pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
 def test_softmax_wide_tiles(K, V, same_block):
