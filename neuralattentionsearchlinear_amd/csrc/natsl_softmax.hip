@@ -442,7 +442,9 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   const size_t krow = (size_t)p.HKV * DK, vrow = (size_t)p.HKV * DV;
   const int32_t* list = p.idx + ((size_t)bos_nats * p.HN + hn) * 2;  // element j at list[j*HN*2]
   const size_t list_stride = (size_t)p.HN * 2;
-  const int n_attn = p.nblk[((size_t)n * p.HN + hn) * 2];
+  // (read where it is used: a scalar load from global memory makes the NEXT scalar-memory wait, whatever it is for,
+  // last a full memory latency, and this one would sit in front of the tile's first requests)
+  const int32_t* n_attn_p = p.nblk + ((size_t)n * p.HN + hn) * 2;
 
   // ---- Q as the B operand of S^T = K Q^T: lane = query column ----------------------------
   bf16x8 QB[KSTEPS];
@@ -674,6 +676,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       __shared__ int wave_count[NWAVES];
       {
         const int jmax = min(dblk, p.TN);
+        const int n_attn = *n_attn_p;
         int cnt = 0;
         for (int j = tid; j < jmax; j += NTHREADS) {
           const int e = list[j * list_stride];
@@ -833,6 +836,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
       // attention blocks that end at or before dstart: ids into LDS, count.  The list is sorted and
       // holds distinct block ids, so entry j >= j: only the first dstart/Bs entries can qualify.
       const int jmax = min(dblk, p.TN);
+      const int n_attn = *n_attn_p;
       int cnt = 0;
       for (int j = tid; j < jmax; j += NTHREADS) {
         const int e = list[j * list_stride];
