@@ -223,19 +223,33 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
       const bf16_t* Vb = Vs + buf * 64 * VP;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
-        // the LDS operands of the first two products are requested ahead of the matrix instructions that use them
-        bf16x8 ak[KS], av[VS];
+        // The LDS operands of the first two products form one stream (K row piece, V row piece, K, V, ...) that is
+        // read a few instructions ahead of its use: reading all of them up front needs 64 registers and spills.
+        constexpr int NOPS = KS + VS, AHEAD = 4;
+        constexpr int NPAIR = KS < VS ? KS : VS;   // the two chains alternate while both last; the longer one ends alone
+        auto is_v = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? (j & 1) != 0 : VS > KS; };
+        auto step_of = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? j >> 1 : j - NPAIR; };
+        auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+          const int st = step_of(j);
+          return is_v(j) ? ld8(Vb + (32 * kt + l32) * VP + 16 * st + 8 * hf) : ld8(Kb + (32 * kt + l32) * KP + 16 * st + 8 * hf);
+        };
+        bf16x8 op[NOPS + AHEAD];
 #pragma unroll
-        for (int st = 0; st < KS; ++st) ak[st] = ld8(Kb + (32 * kt + l32) * KP + 16 * st + 8 * hf);
-#pragma unroll
-        for (int st = 0; st < VS; ++st) av[st] = ld8(Vb + (32 * kt + l32) * VP + 16 * st + 8 * hf);
+        for (int j = 0; j < AHEAD; ++j) op[j] = ld_op(j);
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-        for (int st = 0; st < (KS > VS ? KS : VS); ++st) {   // the two chains alternate
-          if (st < KS) s = mfma32(ak[st], QB[st], s);
-          if (st < VS) dp = mfma32(av[st], DOB[st], dp);
+        for (int j = 0; j < NOPS; ++j) {
+          if (j + AHEAD < NOPS) op[j + AHEAD] = ld_op(j + AHEAD);
+          if (is_v(j)) dp = mfma32(op[j], DOB[step_of(j)], dp);
+          else s = mfma32(op[j], QB[step_of(j)], s);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+        for (int j = 0; j < NOPS; ++j) {
+          if (j + AHEAD < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
         f32x16 ds;
 #pragma unroll
