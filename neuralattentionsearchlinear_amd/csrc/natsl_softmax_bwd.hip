@@ -1,4 +1,4 @@
-// Backward of the softmax branch for gfx950 (first version: correct and on the matrix cores, not yet pipelined).
+// Backward of the softmax branch for gfx950.
 //
 //   delta_kernel   delta[t] = sum_v dO[t,v] O[t,v]                                  (attns.py:357-372)
 //   dq_kernel      one workgroup per tile of 128 queries, the forward's walk over the visible key chunks:
@@ -6,6 +6,7 @@
 //   dkdv_kernel    one workgroup per 64-key chunk of a kv head, walking the query chunks that see it (the rest of its own
 //                  block, and every later chunk when the block is typed attention), for every query head of the group:
 //                  S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS, dnats += sum dS over later blocks (attns.py:719-983)
+//                  The query tiles (Q, dO, lse, delta) arrive by DMA in a ring of three LDS slots, two steps ahead.
 //
 // Layouts follow the forward kernel: the stationary operand of a workgroup (Q, dO there; K, V here) sits in registers
 // as the B operand (lane = its row), the streamed tiles are row-major in LDS, the accumulators' own layout is the B
@@ -37,6 +38,43 @@ NATSL_DEVICE bool bwd_type_is_one(const void* types, int dtype, size_t i) {
 }
 
 constexpr int BWD_MAX_LDS_LIST = 2048;
+
+// Position swizzle of the dkdv kernel's query tiles (rows of D bf16, unpadded): 16-byte segment s of row r is stored at
+// s ^ bwd_swizzle<D>(r).  A bijection over the 16 rows that one clock of a 16-byte row read serves (conflict-free), and
+// two of four consecutive rows never differ by 1, so the 4 rows x 2 segments of a transposing read's 16 lanes
+// fall on different banks as well.
+template <int D>
+NATSL_DEVICE int bwd_swizzle(const int r) {
+  if constexpr (D == 128) return ((r & 7) << 1) | ((r >> 3) & 1);
+  const int y = (r >> 1) & 7;
+  return ((y & 3) << 1) | (y >> 2);
+}
+
+// one DMA instruction: lane l copies 16 (4) bytes from base + voff to LDS byte address lds + 16 l (4 l)
+NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+}
+NATSL_DEVICE void dma4(const void* base, const unsigned voff, const unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+}
+// ... under a wave-uniform condition (non-zero or zero, held in a scalar register): with no lane enabled the instruction
+// requests nothing, which lets a request sit in straight-line code between matrix instructions and still be conditional.
+NATSL_DEVICE void dma16_if(const void* base, const unsigned voff, const unsigned lds, const unsigned on) {
+  unsigned long long saved;
+  asm volatile(
+      "s_mov_b32 m0, %3\n\ts_mov_b64 %0, exec\n\ts_cmp_lg_u32 %4, 0\n\ts_cselect_b64 exec, exec, 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "v"(voff), "s"(base), "s"(lds), "s"(__builtin_amdgcn_readfirstlane(on))
+      : "memory", "m0", "scc");
+}
+NATSL_DEVICE void dma4_if(const void* base, const unsigned voff, const unsigned lds, const unsigned on) {
+  unsigned long long saved;
+  asm volatile(
+      "s_mov_b32 m0, %3\n\ts_mov_b64 %0, exec\n\ts_cmp_lg_u32 %4, 0\n\ts_cselect_b64 exec, exec, 0\n\tglobal_load_lds_dword %1, %2\n\ts_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "v"(voff), "s"(base), "s"(lds), "s"(__builtin_amdgcn_readfirstlane(on))
+      : "memory", "m0", "scc");
+}
 
 // A operand of a 32x32x16 product taken TRANSPOSED from a row-major LDS tile: A[m = lane%32][k-slot (hf, j)] =
 // tile[row_base + 8(j/4) + 4hf + j%4][col_base + m].  ds_read_b64_tr_b16: within each group of 16 lanes, lane i supplies
@@ -306,11 +344,8 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
 // ---------------------------------------------------------------------------------------------
 template <int DK, int DV>
 __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) {
-  constexpr int KP = DK + 8, VP = DV + 8, KS = DK / 16, VS = DV / 16, DT = DK / 32, VT = DV / 32;
+  constexpr int KS = DK / 16, VS = DV / 16, DT = DK / 32, VT = DV / 32;
   extern __shared__ __align__(16) unsigned char smem[];
-  bf16_t* Qs = reinterpret_cast<bf16_t*>(smem);     // [2][64][KP]
-  bf16_t* DOs = Qs + 2 * 64 * KP;                   // [2][64][VP]
-  float* Ls = reinterpret_cast<float*>(DOs + 2 * 64 * VP);  // [2][2][64]: lse, delta
   __shared__ float red[4];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -319,7 +354,18 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
   const int kh = wave & 1, qh = wave >> 1;
   const int NTc = (p.T + 63) >> 6;
   const int n_pairs = p.B * p.HKV;
-  const int pair = (int)blockIdx.x % n_pairs, jc = (int)blockIdx.x / n_pairs;   // earliest (heaviest) chunks first
+  // Workgroups that run at the same time should stream the same queries: consecutive workgroups of one XCD (every 8th
+  // block index) take the key chunks of one (sequence, kv head) in turn, earliest (heaviest) first, and every one
+  // walks the later query chunks from the last one down, so those started together stay together in L2.
+  int pair, jc;
+  if (n_pairs % 8 == 0) {
+    const int xcd = (int)blockIdx.x & 7, i = (int)blockIdx.x >> 3;
+    pair = (i / NTc) * 8 + xcd;
+    jc = i % NTc;
+  } else {
+    pair = (int)blockIdx.x / NTc;
+    jc = (int)blockIdx.x % NTc;
+  }
   const int n = pair / p.HKV, hkv = pair % p.HKV;
   const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
   const int Bs = p.block, per_blk = Bs >> 6;
@@ -349,82 +395,261 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
     for (int r = 0; r < 16; ++r) dk[t][r] = 0.f;
 
   const float c = p.scale_log2;
-  RowStage<DK> sq;
-  RowStage<DV> sd;
-  float sl = 0.f;  // staged lse (threads 0..63) or delta (threads 64..127)
-  auto gload = [&](const int hq, const int jq) {
-    sq.load(p.q + ((size_t)bos * p.HQ + hq) * DK, (size_t)p.HQ * DK, jq * 64, len, tid);
-    sd.load(p.dout + ((size_t)bos * p.HQ + hq) * DV, (size_t)p.HQ * DV, jq * 64, len, tid);
-    if (tid < 128) {
-      const int t = min(jq * 64 + (tid & 63), len - 1);
-      const float* src = tid < 64 ? p.lse : p.delta;
-      sl = src[(size_t)(bos + t) * p.HQ + hq];
+
+  // ---- the ring of query tiles.  Slot layout: Q [64][DK], dO [64][DV], lse [64], delta [64]; rows are unpadded and
+  // the 16-byte segment s of row r sits at position s ^ bwd_swizzle(r).  Tiles arrive by DMA (global -> LDS, no
+  // registers): each instruction fills 1 KiB of a tile, and the swizzle is applied on the global side.
+  constexpr int QROWB = DK * 2, DROWB = DV * 2;
+  constexpr unsigned DOFF = 64 * QROWB, LOFF = DOFF + 64 * DROWB, SLOT = LOFF + 512;
+  constexpr int QI = DK / 32, DI = DV / 32;              // DMA instructions per wave and tile
+  const unsigned lds0 = (unsigned)(size_t)smem;
+  unsigned q_row[QI], q_seg[QI], d_row[DI], d_seg[DI];   // per DMA instruction: the lane's tile row and global byte offset in the row
+#pragma unroll
+  for (int j = 0; j < QI; ++j) {
+    const int pos = lane % (DK / 8), row = (QI * wave + j) * (1024 / QROWB) + lane / (DK / 8);
+    q_row[j] = row;
+    q_seg[j] = 16u * (pos ^ bwd_swizzle<DK>(row));
+  }
+#pragma unroll
+  for (int j = 0; j < DI; ++j) {
+    const int pos = lane % (DV / 8), row = (DI * wave + j) * (1024 / DROWB) + lane / (DV / 8);
+    d_row[j] = row;
+    d_seg[j] = 16u * (pos ^ bwd_swizzle<DV>(row));
+  }
+  // waves 0 and 2 fetch lse, waves 1 and 3 delta (twice the same bytes: every wave then has the same number of requests)
+  const float* l_src = (wave & 1) ? p.delta : p.lse;
+  constexpr int NREQ = QI + DI + 1;   // requests per wave and tile
+  // request piece r of tile jq of head hq into a slot
+  auto piece = [&](const int r, const int hq, const int jq, const int slot, const void*& g, unsigned& voff, unsigned& dst) __attribute__((always_inline)) {
+    const unsigned sl = lds0 + slot * SLOT;
+    if (r < QI) {
+      g = p.q + ((size_t)bos * p.HQ + hq) * DK;
+      voff = (unsigned)min(jq * 64 + (int)q_row[r < QI ? r : 0], len - 1) * ((unsigned)p.HQ * QROWB) + q_seg[r < QI ? r : 0];
+      dst = sl + (QI * wave + r) * 1024;
+    } else if (r < QI + DI) {
+      const int j = r < QI ? 0 : (r < QI + DI ? r - QI : 0);
+      g = p.dout + ((size_t)bos * p.HQ + hq) * DV;
+      voff = (unsigned)min(jq * 64 + (int)d_row[j], len - 1) * ((unsigned)p.HQ * DROWB) + d_seg[j];
+      dst = sl + DOFF + (DI * wave + j) * 1024;
+    } else {
+      g = l_src + (size_t)bos * p.HQ + hq;
+      voff = (unsigned)min(jq * 64 + lane, len - 1) * (unsigned)(p.HQ * 4);
+      dst = sl + LOFF + 256 * (wave & 1);
     }
   };
-  auto lstore = [&](const int buf) {
-    sq.store(Qs + buf * 64 * KP, tid);
-    sd.store(DOs + buf * 64 * VP, tid);
-    if (tid < 128) Ls[buf * 128 + tid] = sl;
+  auto request = [&](const int hq, const int jq, const int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < NREQ; ++r) {
+      const void* g;
+      unsigned voff, dst;
+      piece(r, hq, jq, slot, g, voff, dst);
+      if (r < QI + DI) dma16(g, voff, dst);
+      else dma4(g, voff, dst);
+    }
   };
+  auto request_piece_if = [&](const int r, const int hq, const int jq, const int slot, const unsigned on) __attribute__((always_inline)) {
+    const void* g;
+    unsigned voff, dst;
+    piece(r, hq, jq, slot, g, voff, dst);
+    if (r < QI + DI) dma16_if(g, voff, dst, on);
+    else dma4_if(g, voff, dst, on);
+  };
+
+  // ---- LDS byte offsets of the lane's operands inside a slot
+  typedef __attribute__((address_space(3))) const bf16x8* lds_op;
+  typedef __attribute__((address_space(3))) s16x4* lds_tr;
+  unsigned aq[KS], ad[VS];              // first two products: the lane's query row, k-step st
+  {
+    const int row = 32 * qh + l32;
+#pragma unroll
+    for (int st = 0; st < KS; ++st) aq[st] = row * QROWB + 16u * ((2 * st + hf) ^ bwd_swizzle<DK>(row));
+#pragma unroll
+    for (int st = 0; st < VS; ++st) ad[st] = DOFF + row * DROWB + 16u * ((2 * st + hf) ^ bwd_swizzle<DV>(row));
+  }
+  // last two products: transposing reads.  Within 16 lanes, lane i addresses 4 elements of row 4 hf + i/4 (+ 8 for the
+  // second read) at column 32 t + 16 (lane/16 % 2) + 4 (i % 4).
+  unsigned tq[2][DT][2], td[2][VT][2];
+  {
+    const int i16 = lane & 15;
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int rd = 0; rd < 2; ++rd) {
+        const int row = 32 * qh + 16 * ss + 8 * rd + 4 * hf + (i16 >> 2);
+        const int seg0 = 2 * ((lane >> 4) & 1) + ((i16 >> 1) & 1);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) tq[ss][t][rd] = row * QROWB + 16u * ((4 * t + seg0) ^ bwd_swizzle<DK>(row)) + 8u * (i16 & 1);
+#pragma unroll
+        for (int t = 0; t < VT; ++t) td[ss][t][rd] = DOFF + row * DROWB + 16u * ((4 * t + seg0) ^ bwd_swizzle<DV>(row)) + 8u * (i16 & 1);
+      }
+  }
 
   for (int g = 0; g < G; ++g) {
     const int hq = hkv * G + g, hn = hq / GN;
     const bool attn = bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + kb) * p.HN + hn) * 2);
     const int n_same = p.same_block ? blk_end_chunk - jc : 0;
-    const int n_later = attn ? max(NTc - blk_end_chunk, 0) : 0;
+    const int n_later = __builtin_amdgcn_readfirstlane(attn ? max(NTc - blk_end_chunk, 0) : 0);   // (the type was read by a vector load)
     const int n_it = n_same + n_later;
     float dn = 0.f;
-    auto chunk_of = [&](const int it) { return it < n_same ? jc + it : blk_end_chunk + (it - n_same); };
+    auto chunk_of = [&](const int it) { return it < n_same ? jc + it : NTc - 1 - (it - n_same); };
     if (n_it > 0) {
-      gload(hq, chunk_of(0));
-      __syncthreads();   // the previous head's last reads of buffer 0 are done
-      lstore(0);
+      __syncthreads();   // the previous head's last reads of the ring are done
+      request(hq, chunk_of(0), 0);
+      if (n_it > 1) {
+        request(hq, chunk_of(1), 1);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | NREQ);   // vmcnt: all but the newest tile's requests
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+      }
       __syncthreads();
     }
+    int slot = 0;
     for (int it = 0; it < n_it; ++it) {
-      const int buf = it & 1;
       const int jq = chunk_of(it);
-      if (it + 1 < n_it) gload(hq, chunk_of(it + 1));
-      const bf16_t* Qb = Qs + buf * 64 * KP;
-      const bf16_t* Db = DOs + buf * 64 * VP;
-      const float* Lb = Ls + buf * 128;
+      const unsigned sb = lds0 + slot * SLOT;
+      // ---- S^T = Q K^T and dP^T = dO V^T for (32 queries) x (32 keys): one stream of LDS operands, read ahead
+      constexpr int NOPS = KS + VS, AHEAD = 6;
+      constexpr int NPAIR = KS < VS ? KS : VS;
+      auto is_v = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? (j & 1) != 0 : VS > KS; };
+      auto step_of = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? j >> 1 : j - NPAIR; };
+      // (equal head dims: the dO tile has the Q tile's layout DOFF bytes further, an immediate offset of the read)
+      constexpr bool SAME = DK == DV;
+      unsigned cq[KS], cd[SAME ? 1 : VS];
+#pragma unroll
+      for (int st = 0; st < KS; ++st) { cq[st] = sb + aq[st]; asm("" : "+v"(cq[st])); }
+      if constexpr (!SAME) {
+#pragma unroll
+        for (int st = 0; st < VS; ++st) { cd[st] = sb + ad[st]; asm("" : "+v"(cd[st])); }
+      }
+      auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+        if constexpr (SAME) return *reinterpret_cast<lds_op>(cq[step_of(j)] + (is_v(j) ? DOFF : 0u));
+        else return *reinterpret_cast<lds_op>(is_v(j) ? cd[step_of(j)] : cq[step_of(j)]);
+      };
       f32x16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+      {
+        bf16x8 op[NOPS + AHEAD];
 #pragma unroll
-      for (int st = 0; st < (KS > VS ? KS : VS); ++st) {   // the two chains alternate
-        if (st < KS) s = mfma32(ld8(Qb + (32 * qh + l32) * KP + 16 * st + 8 * hf), KB[st], s);
-        if (st < VS) dp = mfma32(ld8(Db + (32 * qh + l32) * VP + 16 * st + 8 * hf), VB[st], dp);
+        for (int j = 0; j < AHEAD; ++j) op[j] = ld_op(j);
+#pragma unroll
+        for (int j = 0; j < NOPS; ++j) {
+          if (j + AHEAD < NOPS) op[j + AHEAD] = ld_op(j + AHEAD);
+          if (is_v(j)) dp = mfma32(op[j], VB[step_of(j)], dp);
+          else s = mfma32(op[j], KB[step_of(j)], s);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+        for (int j = 0; j < NOPS; ++j) {
+          if (j + AHEAD < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
       }
+      // ---- the tile of the next step has been requested a whole step ago: once every wave has seen its own requests
+      // land it is complete, and the slot of the previous step is free for the tile two steps ahead
+      __builtin_amdgcn_sched_barrier(0);   // (all matrix instructions are issued first: they drain while the wave waits)
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      const bool ask = it + 2 < n_it;   // the tile two steps ahead goes into the slot of the previous step
+      const int ask_jq = ask ? chunk_of(it + 2) : 0, ask_slot = slot == 0 ? 2 : slot - 1;
+      // no tile left to ask for: the requests run with no lane enabled (read through a lane so that it sits in scalar registers)
+      const unsigned ask_mask = __builtin_amdgcn_readfirstlane(ask ? 1u : 0u);
+      // ---- dV^T += dO^T P and dK^T += Q^T dS: 16 operands of two transposing reads each, read ahead.  The first of
+      // them and the rows' lse and delta are requested before the exponentials, which then run under the LDS latency.
+      constexpr int N2 = 2 * (VT + DT), A2 = 4;   // operand j: ss = j / (VT + DT); within it the VT value tiles, then the DT key-dim tiles
+      unsigned ct[SAME ? 2 * DT : N2][2];   // equal head dims: one address per (ss, tile) serves both tiles
+      if constexpr (SAME) {
+#pragma unroll
+        for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+          for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int rd = 0; rd < 2; ++rd) {
+              ct[ss * DT + t][rd] = sb + tq[ss][t][rd];
+              asm("" : "+v"(ct[ss * DT + t][rd]));
+            }
+      } else {
+#pragma unroll
+        for (int j = 0; j < N2; ++j) {
+          const int ss = j / (VT + DT), u = j % (VT + DT);
+#pragma unroll
+          for (int rd = 0; rd < 2; ++rd) {
+            ct[j][rd] = sb + (u < VT ? td[ss][u < VT ? u : 0][rd] : tq[ss][u < VT ? 0 : u - VT][rd]);
+            asm("" : "+v"(ct[j][rd]));
+          }
+        }
+      }
+      auto tr_read = [&](const int j, const int rd) __attribute__((always_inline)) -> s16x4 {
+        if constexpr (SAME) {
+          const int ss = j / (VT + DT), u = j % (VT + DT);
+          return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr>(ct[ss * DT + (u < VT ? u : u - VT)][rd] + (u < VT ? DOFF : 0u)));
+        } else {
+          return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr>(ct[j][rd]));
+        }
+      };
+      const float* Lb = reinterpret_cast<const float*>(smem + slot * SLOT + LOFF);
+      f32x4 l4[4], d4[4];
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        l4[rg] = *reinterpret_cast<const f32x4*>(Lb + 32 * qh + 8 * rg + 4 * hf);
+        d4[rg] = *reinterpret_cast<const f32x4*>(Lb + 64 + 32 * qh + 8 * rg + 4 * hf);
+      }
+      s16x4 lo[N2 + A2], hi[N2 + A2];
+#pragma unroll
+      for (int j = 0; j < A2; ++j) {
+        lo[j] = tr_read(j, 0);
+        hi[j] = tr_read(j, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
       f32x16 pr, ds;
       const bool own = jq == jc;
       float dsum = 0.f;
+      if (!own && jq * 64 + 64 <= len) {   // every (query, key) pair of the tile is visible: no masks
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Lb + 32 * qh + 8 * rg + 4 * hf);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Lb + 64 + 32 * qh + 8 * rg + 4 * hf);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int r = 4 * rg + j;
-          const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
-          const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
-          const float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[j])) : 0.f;
+        for (int r = 0; r < 16; ++r) {
+          const float e = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[r >> 2][r & 3]));
           pr[r] = e;
-          ds[r] = e * (dp[r] - d4[j]);
+          ds[r] = e * (dp[r] - d4[r >> 2][r & 3]);
           dsum += ds[r];
+        }
+      } else {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = 4 * rg + j;
+            const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
+            const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
+            const float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[rg][j])) : 0.f;
+            pr[r] = e;
+            ds[r] = e * (dp[r] - d4[rg][j]);
+            dsum += ds[r];
+          }
         }
       }
       if (it >= n_same && jc * 64 + 32 * kh + l32 < len) dn += dsum;
+      bf16x8 PB[2][2];
 #pragma unroll
-      for (int ss = 0; ss < 2; ++ss) {
-        const bf16x8 PBp = pack8(pr, ss), PBs = pack8(ds, ss);
+      for (int ss = 0; ss < 2; ++ss) { PB[ss][0] = pack8(pr, ss); PB[ss][1] = pack8(ds, ss); }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < VT; ++t) dv[t] = mfma32(tr_operand(Db, VP, 32 * qh + 16 * ss, 32 * t, lane), PBp, dv[t]);
-#pragma unroll
-        for (int t = 0; t < DT; ++t) dk[t] = mfma32(tr_operand(Qb, KP, 32 * qh + 16 * ss, 32 * t, lane), PBs, dk[t]);
+      for (int j = 0; j < N2; ++j) {
+        if (j + A2 < N2) {
+          lo[j + A2] = tr_read(j + A2, 0);
+          hi[j + A2] = tr_read(j + A2, 1);
+        }
+        const int ss = j / (VT + DT), u = j % (VT + DT);
+        if (u < VT) dv[u < VT ? u : 0] = mfma32(join4(lo[j], hi[j]), PB[ss][0], dv[u < VT ? u : 0]);
+        else dk[u < VT ? 0 : u - VT] = mfma32(join4(lo[j], hi[j]), PB[ss][1], dk[u < VT ? 0 : u - VT]);
+        if (j < NREQ) request_piece_if(j, hq, ask_jq, ask_slot, ask_mask);   // one request under each matrix instruction
       }
-      if (it + 1 < n_it) lstore(buf ^ 1);
-      __syncthreads();
+      static_assert(NREQ <= N2, "requests are issued under the matrix instructions");
+#pragma unroll
+      for (int j = 0; j < N2; ++j) {
+        if (j + A2 < N2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      slot = slot == 2 ? 0 : slot + 1;
     }
     // dnats of this (key block, query head): the four waves' sums
     if (n_later > 0) {
@@ -520,9 +745,12 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
   }
   {
-    size_t lds = (size_t)2 * 64 * (KP + VP) * sizeof(bf16_t) + 2 * 128 * sizeof(float);
+    size_t lds = (size_t)3 * (64 * (DK + DV) * sizeof(bf16_t) + 512);   // the ring of three query tiles
     const size_t red = (size_t)2 * (DV / 32 + DK / 32) * 16 * 64 * sizeof(float);
     if (red > lds) lds = red;
+    // the DMA requests address a sequence's rows with 32-bit byte offsets
+    if ((long long)p.T * p.HQ * (DK > DV ? DK : DV) * 2 >= (1ll << 32))
+      return fail(NATSL_ERR_UNSUPPORTED, "softmax bwd: T * HQ = %lld rows of one sequence exceed the 32-bit offsets of the dk/dv kernel", (long long)p.T * p.HQ);
     auto kern = dkdv_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
@@ -571,3 +799,4 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
 #undef NATSL_SB
   return fail(NATSL_ERR_UNSUPPORTED, "%s: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", what, K, V);
 }
+
