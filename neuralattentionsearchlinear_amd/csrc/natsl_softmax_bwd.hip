@@ -148,7 +148,11 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hf = lane >> 5;
   const int nq_tiles = (p.T + QTILE - 1) / QTILE;
-  const int pair = (int)blockIdx.x / nq_tiles, tile = nq_tiles - 1 - (int)blockIdx.x % nq_tiles;
+  // every 8th block index lands on the same XCD: an XCD takes the tiles of one (sequence, head) in turn, last tile
+  // first, so the workgroups that share an L2 walk the same key blocks
+  const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
+  const int pair = (j / nq_tiles) * 8 + xcd, tile = nq_tiles - 1 - j % nq_tiles;
+  if (pair >= p.B * p.HQ) return;   // (the grid is rounded up to whole groups of 8 pairs)
   const int n = pair / p.HQ, hq = pair % p.HQ;
   const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
   const int Bs = p.block, per_blk = Bs >> 6;
@@ -741,7 +745,7 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     auto kern = dq_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    const long long grid = (long long)p.B * p.HQ * ((p.T + 127) / 128);
+    const long long grid = ((long long)p.B * p.HQ + 7) / 8 * 8 * ((p.T + 127) / 128);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
   }
   {
