@@ -92,6 +92,50 @@ def test_c2_softmax_slices_against_dense_fp32(c2, same_block):
         assert float((lse[b, :, h] - lse_ref).abs().max()) <= 2e-2, "lse (log2 units)"
 
 
+def test_c2_softmax_backward_slices_against_dense_fp32(c2):
+    """dq, dk, dv and the selector's gradient at the full c2 shape, on single (sequence, head) slices, against
+    torch.autograd through the dense fp32 masked softmax (the oracle's visibility rule).  Gradient tolerance as in the
+    backward's own tests: rel-L2 5e-3, max-abs 2e-2 of the reference's largest magnitude."""
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_bwd, parallel_attn_nats_fwd
+    w = C2
+    scale = w['K'] ** -0.5
+    r = nats_util.route(c2['ty'], w['T'], w['block'])
+    with torch.no_grad():
+        o, lse, _ = parallel_attn_nats_fwd(c2['q'], c2['k'], c2['v'], c2['ty'], r['nats_block_indices'], None, scale, w['block'],
+                                           compute_incomplete_chunk_scores=True, n_nats_blocks=r['n_nats_blocks'])
+        do = _randn(o.shape, 55)
+        dq, dk, dv, _, dn = parallel_attn_nats_bwd(c2['q'], c2['k'], c2['v'], o, c2['ty'], r['nats_block_indices'], r['n_nats_blocks'],
+                                                   None, lse, do, scale=scale, NAtS_block_size=w['block'],
+                                                   compute_incomplete_chunk_scores=True)
+    for b, h in ((0, 0), (5, 9)):
+        typ = c2['ty'][b, :, h, 0].float().cpu()
+        mask = SB.visibility_mask(typ, w['T'], w['block'], True).to(DEV)
+        qf, kf, vf = (c2[n][b, :, h].float().requires_grad_() for n in ('q', 'k', 'v'))
+        s = ((qf @ kf.T) * scale).masked_fill(~mask, float('-inf'))
+        p = torch.softmax(s, -1)
+        (p @ vf).backward(do[b, :, h].float())
+        for name, got, ref in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+            g_, r_ = got[b, :, h].float(), ref
+            rl = float((g_ - r_).norm() / r_.norm())
+            ma, top = float((g_ - r_).abs().max()), float(r_.abs().max())
+            assert rl <= 5e-3 and ma <= 2e-2 * max(top, 1.0), f"{name}[{b},:,{h}]: rel-L2 {rl:.3e}, max-abs {ma:.3e} of {top:.3e}"
+        # selector gradient of block j: sum of dS over (queries of later blocks) x (keys of block j), for blocks typed attention
+        with torch.no_grad():
+            dp = do[b, :, h].float() @ vf.detach().T
+            delta = (do[b, :, h].float() * o[b, :, h].float()).sum(-1, keepdim=True)
+            dS = p.detach() * (dp - delta)
+            NB, Bs = w['T'] // w['block'], w['block']
+            blk = torch.arange(w['T'], device=DEV) // Bs
+            later = blk[:, None] > blk[None, :]
+            dS_l = torch.where(later, dS, torch.zeros_like(dS))
+            ref_dn = dS_l.sum(0).view(NB, Bs).sum(-1)
+            mag = dS_l.abs().sum(0).view(NB, Bs).sum(-1)
+            attn = (torch.round(typ) == 1).to(DEV)
+            err = (dn[b, :, h].float() - torch.where(attn, ref_dn, torch.zeros_like(ref_dn))).abs()
+            assert bool((err <= 2e-3 * mag + 1e-5).all()), f"dnats[{b},:,{h}]: error {float(err.max()):.3e} against magnitude {float(mag.max()):.3e}"
+
+
 def test_c2_outputs_are_exactly_homogeneous_in_v(c2):
     w = C2
     scale = w['K'] ** -0.5

@@ -81,3 +81,11 @@ def test_softmax_bwd_all_attention_and_all_linear():
 
 def test_softmax_bwd_through_autograd():
     _run(2, 384, 4, 2, 2, 128, 128, 64, 0.5, True, seed=11, through_autograd=True)
+
+
+def test_softmax_bwd_many_pairs_and_long_walks():
+    """More (sequence, kv head) pairs than XCDs and walks of tens of query tiles: the dk/dv kernel's ring of tiles in its
+    steady state, several pairs per XCD; then grouped query heads (the ring restarts for every head of the group)."""
+    _run(2, 2048, 16, 16, 16, 128, 128, 64, 0.3, True, seed=20)
+    _run(2, 1024, 16, 8, 4, 64, 128, 64, 0.4, False, seed=21)
+    _run(1, 1000, 8, 8, 8, 128, 64, 128, 0.5, True, seed=22)     # ragged last tile, blocks of two chunks
