@@ -23,6 +23,7 @@ struct SoftmaxBwdParams {
   bf16_t *dq, *dk, *dv;
   float* dnats;   // [B, TN, HQ], zero on entry
   float* delta;   // [B, T, HQ] workspace
+  int* queue;     // [8] workspace: next unit of each XCD's list for the dk/dv kernel, zeroed by the delta kernel
   const void* types;
   int types_dtype;
   const int32_t* idx;
@@ -99,6 +100,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const SoftmaxBwdParams p) {
   const long long rows = (long long)p.B * p.T * p.HQ;
   const long long row = (long long)blockIdx.x * RPB + threadIdx.x / LPR;
   const int seg = threadIdx.x % LPR;
+  if (blockIdx.x == 0 && threadIdx.x < 8) p.queue[threadIdx.x] = 0;   // the dk/dv kernel's work queues (it runs after this kernel)
   float acc = 0.f;
   if (row < rows) {
     const u32x4 a = *reinterpret_cast<const u32x4*>(p.o + row * DV + 8 * seg);
@@ -358,18 +360,37 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
   const int kh = wave & 1, qh = wave >> 1;
   const int NTc = (p.T + 63) >> 6;
   const int n_pairs = p.B * p.HKV;
-  // Workgroups that run at the same time should stream the same queries: consecutive workgroups of one XCD (every 8th
-  // block index) take the key chunks of one (sequence, kv head) in turn, earliest (heaviest) first, and every one
-  // walks the later query chunks from the last one down, so those started together stay together in L2.
-  int pair, jc;
-  if (n_pairs % 8 == 0) {
-    const int xcd = (int)blockIdx.x & 7, i = (int)blockIdx.x >> 3;
-    pair = (i / NTc) * 8 + xcd;
-    jc = i % NTc;
-  } else {
-    pair = (int)blockIdx.x / NTc;
-    jc = (int)blockIdx.x % NTc;
-  }
+  // ---- Persistent workgroups (one per CU; the kernel's registers and LDS admit no more) take units = (sequence, kv
+  // head, key chunk) from work queues: starting a workgroup per unit left the CUs idle a quarter of the time.
+  // Workgroups that run at the same time should stream the same queries, so every XCD (block index mod 8) has a queue
+  // of its own with the key chunks of one (sequence, kv head) after the other, earliest (heaviest) chunk first, and
+  // every unit walks the later query chunks from the last one down: units started together stay together in L2.  A
+  // workgroup whose queue is empty takes from the other XCDs' queues.
+  __shared__ int unit_pair, unit_jc;
+  const bool per_xcd = n_pairs % 8 == 0;
+  const int n_queues = per_xcd ? 8 : 1;
+  const int queue_len = (per_xcd ? n_pairs / 8 : n_pairs) * NTc;
+  int q_probe = 0;   // queues found empty so far (they stay empty)
+  for (;;) {
+    if (tid == 0) {
+      int pr = -1, jj = 0;
+      while (q_probe < n_queues) {
+        const int x = per_xcd ? ((int)blockIdx.x + q_probe) & 7 : 0;
+        const int i = atomicAdd(p.queue + x, 1);
+        if (i < queue_len) {
+          pr = per_xcd ? (i / NTc) * 8 + x : i / NTc;
+          jj = i % NTc;
+          break;
+        }
+        ++q_probe;
+      }
+      unit_pair = pr;
+      unit_jc = jj;
+    }
+    __syncthreads();
+    const int pair = unit_pair, jc = unit_jc;
+    __syncthreads();   // (read before the next round's write)
+    if (pair < 0) break;
   const int n = pair / p.HKV, hkv = pair % p.HKV;
   const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
   const int Bs = p.block, per_blk = Bs >> 6;
@@ -732,6 +753,21 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
             *reinterpret_cast<const u32x4*>(Os + row * OP + DV + seg * 8);
     }
   }
+  __syncthreads();   // the staging area is the next unit's tile ring
+  }  // units
+}
+
+// number of CUs of the current device (one persistent dk/dv workgroup each)
+static int cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
 }
 
 template <int DK, int DV>
@@ -758,7 +794,9 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     auto kern = dkdv_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    const long long grid = (long long)p.B * p.HKV * ((p.T + 63) / 64);
+    const long long units = (long long)p.B * p.HKV * ((p.T + 63) / 64);
+    long long grid = (cu_count() + 7) / 8 * 8;   // whole groups of 8: block index mod 8 names the XCD and its queue
+    if (grid > units) grid = units;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
   }
   return check_launch("natsl_softmax_sparse_bwd");
@@ -768,7 +806,9 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
 
 using namespace natsl;
 
-extern "C" size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ) { return (size_t)B * T * HQ * sizeof(float); }
+// delta [B, T, HQ] fp32, then the dk/dv kernel's 8 work-queue counters
+static size_t bwd_queue_offset(int B, int T, int HQ) { return ((size_t)B * T * HQ * sizeof(float) + 255) / 256 * 256; }
+extern "C" size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ) { return bwd_queue_offset(B, T, HQ) + 256; }
 
 extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
                                         const void* d_o, void* dq, void* dk, void* dv, float* dnats, const void* types,
@@ -790,6 +830,7 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
   SoftmaxBwdParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (const bf16_t*)o; p.dout = (const bf16_t*)d_o;
   p.lse = lse; p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dv = (bf16_t*)dv; p.dnats = dnats; p.delta = (float*)workspace;
+  p.queue = reinterpret_cast<int*>(static_cast<char*>(workspace) + bwd_queue_offset(B, T, HQ));
   p.types = types; p.types_dtype = types_dtype; p.idx = nats_block_indices; p.nblk = n_nats_blocks;
   p.B = B; p.T = T; p.HQ = HQ; p.HKV = HKV; p.HN = HN; p.TN = TN; p.block = block;
   p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f; p.same_block = same_block_visible ? 1 : 0;
