@@ -295,22 +295,41 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
           if (j + AHEAD < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
-        f32x16 ds;
+        // dQ^T += K^T dS^T: the transposed K operands are read ahead as well, the first of them before the exponentials
+        constexpr int N3 = 2 * DT, A3 = 4 < N3 ? 4 : N3;
+        auto tr_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+          return tr_operand(Kb, KP, 32 * kt + 16 * (j / DT), 32 * (j % DT), lane);
+        };
+        bf16x8 at[N3 + A3];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3);
-          const bool vis = !causal || kloc <= qloc0 + l32;
-          const float pr = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse_q)) : 0.f;
-          ds[r] = pr * (dp[r] - delta_q);
+        for (int j = 0; j < A3; ++j) at[j] = tr_op(j);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x16 ds;
+        if (!causal) {   // every key of the chunk is visible to every query of the wave: no masks
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse_q)) * (dp[r] - delta_q);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kloc = 32 * kt + 8 * (r >> 2) + 4 * hf + (r & 3);
+            const bool vis = kloc <= qloc0 + l32;
+            const float pr = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse_q)) : 0.f;
+            ds[r] = pr * (dp[r] - delta_q);
+          }
+        }
+        bf16x8 PB[2];
+#pragma unroll
+        for (int ss = 0; ss < 2; ++ss) PB[ss] = pack8(ds, ss);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < N3; ++j) {
+          if (j + A3 < N3) at[j + A3] = tr_op(j + A3);
+          acc[j % DT] = mfma32(at[j], PB[j / DT], acc[j % DT]);
         }
 #pragma unroll
-        for (int ss = 0; ss < 2; ++ss) {
-          bf16x8 at[DT];
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) at[dt] = tr_operand(Kb, KP, 32 * kt + 16 * ss, 32 * dt, lane);
-          const bf16x8 PB = pack8(ds, ss);
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(at[dt], PB, acc[dt]);
+        for (int j = 0; j < N3; ++j) {
+          if (j + A3 < N3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
       }
     }
