@@ -708,29 +708,33 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
 
   // ---- the two query halves of a key half are summed through LDS, then the tiles are transposed and stored
   __syncthreads();
-  float* Rs = reinterpret_cast<float*>(smem);   // [2 key halves][(VT + DT) * 16][64 lanes]
+  f32x4* Rs = reinterpret_cast<f32x4*>(smem);   // [2 key halves][(VT + DT) * 4 register groups][64 lanes] of 4 floats
   if (qh == 1) {
-    float* dst = Rs + (size_t)kh * (VT + DT) * 16 * 64 + lane;
+    f32x4* dst = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
 #pragma unroll
     for (int t = 0; t < VT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dst[(t * 16 + r) * 64] = dv[t][r];
+      for (int rg = 0; rg < 4; ++rg) dst[(t * 4 + rg) * 64] = f32x4{dv[t][4 * rg], dv[t][4 * rg + 1], dv[t][4 * rg + 2], dv[t][4 * rg + 3]};
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dst[((VT + t) * 16 + r) * 64] = dk[t][r];
+      for (int rg = 0; rg < 4; ++rg) dst[((VT + t) * 4 + rg) * 64] = f32x4{dk[t][4 * rg], dk[t][4 * rg + 1], dk[t][4 * rg + 2], dk[t][4 * rg + 3]};
   }
   __syncthreads();
   if (qh == 0) {
-    const float* src = Rs + (size_t)kh * (VT + DT) * 16 * 64 + lane;
+    // (all reads first, then the sums: a read-wait-add sequence per value took 5000 cycles)
+    const f32x4* src = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
+    f32x4 x[(VT + DT) * 4];
+#pragma unroll
+    for (int i = 0; i < (VT + DT) * 4; ++i) x[i] = src[i * 64];
 #pragma unroll
     for (int t = 0; t < VT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dv[t][r] += src[(t * 16 + r) * 64];
+      for (int r = 0; r < 16; ++r) dv[t][r] += x[t * 4 + (r >> 2)][r & 3];
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dk[t][r] = (dk[t][r] + src[((VT + t) * 16 + r) * 64]) * p.scale;
+      for (int r = 0; r < 16; ++r) dk[t][r] = (dk[t][r] + x[(VT + t) * 4 + (r >> 2)][r & 3]) * p.scale;
   }
   __syncthreads();
   if (qh == 0) {
@@ -757,19 +761,29 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
       }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
-    for (int i = lane; i < 32 * (DV / 8); i += 64) {
-      const int row = i / (DV / 8), seg = i % (DV / 8);
-      const int t = jc * 64 + 32 * kh + row;
-      if (t < len)
-        *reinterpret_cast<u32x4*>(p.dv + ((size_t)(bos + t) * p.HKV + hkv) * DV + seg * 8) =
-            *reinterpret_cast<const u32x4*>(Os + row * OP + seg * 8);
+    // all LDS reads first, then the stores (a read-wait-store sequence per piece took 4000 cycles)
+    constexpr int NV = 32 * (DV / 8) / 64, NK = 32 * (DK / 8) / 64;
+    u32x4 wv[NV], wk[NK];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = lane + 64 * i, row = e / (DV / 8), seg = e % (DV / 8);
+      wv[i] = *reinterpret_cast<const u32x4*>(Os + row * OP + seg * 8);
     }
-    for (int i = lane; i < 32 * (DK / 8); i += 64) {
-      const int row = i / (DK / 8), seg = i % (DK / 8);
-      const int t = jc * 64 + 32 * kh + row;
-      if (t < len)
-        *reinterpret_cast<u32x4*>(p.dk + ((size_t)(bos + t) * p.HKV + hkv) * DK + seg * 8) =
-            *reinterpret_cast<const u32x4*>(Os + row * OP + DV + seg * 8);
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int e = lane + 64 * i, row = e / (DK / 8), seg = e % (DK / 8);
+      wk[i] = *reinterpret_cast<const u32x4*>(Os + row * OP + DV + seg * 8);
+    }
+    const int t_base = jc * 64 + 32 * kh;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = lane + 64 * i, row = e / (DV / 8), seg = e % (DV / 8);
+      if (t_base + row < len) *reinterpret_cast<u32x4*>(p.dv + ((size_t)(bos + t_base + row) * p.HKV + hkv) * DV + seg * 8) = wv[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int e = lane + 64 * i, row = e / (DK / 8), seg = e % (DK / 8);
+      if (t_base + row < len) *reinterpret_cast<u32x4*>(p.dk + ((size_t)(bos + t_base + row) * p.HKV + hkv) * DK + seg * 8) = wk[i];
     }
   }
   __syncthreads();   // the staging area is the next unit's tile ring
