@@ -89,3 +89,41 @@ def test_softmax_bwd_many_pairs_and_long_walks():
     _run(2, 2048, 16, 16, 16, 128, 128, 64, 0.3, True, seed=20)
     _run(2, 1024, 16, 8, 4, 64, 128, 64, 0.4, False, seed=21)
     _run(1, 1000, 8, 8, 8, 128, 64, 128, 0.5, True, seed=22)     # ragged last tile, blocks of two chunks
+
+
+def test_softmax_bwd_repeatable_and_workspace_reuse():
+    """The dk/dv kernel takes its units from work queues in whatever order the workgroups arrive: dq, dk, dv must not
+    depend on it (bit-identical from launch to launch; dnats is summed with float atomics and may differ in the last
+    bits).  The queue counters live in the caller's workspace and are reset by every call: the same buffer, dirty from
+    the previous call and then filled with ones, serves the next."""
+    from neuralattentionsearchlinear_amd import _capi, nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_fwd
+    B, T, HQ, H, HN, K, V, block = 2, 1536, 16, 8, 8, 128, 128, 64
+    q, k, v = (t.to(DEV) for t in make_qkv(B, T, H, K, V, 31, HQ=HQ))
+    do = torch.randn(B, T, HQ, V, generator=torch.Generator().manual_seed(32)).bfloat16().to(DEV)
+    ty = make_types(B, T // block, HN, 0.4, 33, torch.bfloat16).to(DEV)
+    scale = K ** -0.5
+    r = nats_util.route(ty, T, block)
+    o, lse, _ = parallel_attn_nats_fwd(q, k, v, ty, r['nats_block_indices'], None, scale, block,
+                                       compute_incomplete_chunk_scores=True, n_nats_blocks=r['n_nats_blocks'])
+    L = _capi.lib()
+    ws_bytes = L.natsl_softmax_bwd_workspace_bytes(B, T, HQ)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    outs = []
+    for rep in range(3):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dn = torch.zeros(B, T // block, HQ, dtype=torch.float32, device=DEV)
+        if rep == 2:
+            ws.fill_(1)
+        rc = L.natsl_softmax_sparse_bwd(
+            _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(o), _capi.ptr(lse), _capi.ptr(do), _capi.ptr(dq), _capi.ptr(dk),
+            _capi.ptr(dv), _capi.ptr(dn), _capi.ptr(ty), _capi.dtype_code(ty.dtype), _capi.ptr(r['nats_block_indices']),
+            _capi.ptr(r['n_nats_blocks']), B, T, HQ, H, HN, K, V, T // block, block, float(scale), 1, _capi.dtype_code(q.dtype),
+            _capi.ptr(ws), ws_bytes, _capi.stream_ptr(q.device))
+        _capi.check(rc, "natsl_softmax_sparse_bwd")
+        torch.cuda.synchronize()
+        outs.append((dq, dk, dv, dn))
+    for rep in (1, 2):
+        for name, a, b in zip(("dq", "dk", "dv"), outs[0], outs[rep]):
+            assert torch.equal(a, b), f"{name} differs between launches 0 and {rep}"
+        assert float((outs[0][3] - outs[rep][3]).abs().max()) <= 1e-3 * float(outs[0][3].abs().max() + 1.0)
