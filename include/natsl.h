@@ -110,7 +110,9 @@ int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* 
  * with respect to a bias on that block's scores as later blocks see them; blocks not typed attention keep 0 (the
  * reference's default compute_dnats_for_invalid_blocks_attn = False).  The caller sums dnats over the query heads of a
  * selector head.  o, lse are the forward's outputs, d_o the gradient of o.  workspace: natsl_softmax_bwd_workspace_bytes()
- * bytes (delta = rowsum(d_o * o)).  Regular batches only (no packed-sequence table yet).
+ * bytes (delta = rowsum(d_o * o), then the work-queue counters of the dk/dv kernel; nothing to initialise: every call resets
+ * them, so calls that share a workspace must not overlap).  T * HQ * max(K, V) * 2 must stay below 2^32 (32-bit row offsets
+ * within a sequence).  Regular batches only (no packed-sequence table yet).
  * Replaces parallel_attn_nats_bwd (src/nats/ops/attns/attns.py:1562-1759; kernels :357-372, :383-708, :719-983) as
  * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:226-243. */
 size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ);
