@@ -3,10 +3,11 @@
 //   delta_kernel   delta[t] = sum_v dO[t,v] O[t,v]                                  (attns.py:357-372)
 //   dq_kernel      one workgroup per tile of 128 queries, the forward's walk over the visible key chunks:
 //                  S^T = K Q^T, P = exp2(S c - lse), dP^T = V dO^T, dS = P (dP - delta), dQ^T += K^T dS^T (attns.py:383-708)
-//   dkdv_kernel    one workgroup per 64-key chunk of a kv head, walking the query chunks that see it (the rest of its own
+//   dkdv_kernel    unit = one 64-key chunk of a kv head, walking the query chunks that see it (the rest of its own
 //                  block, and every later chunk when the block is typed attention), for every query head of the group:
 //                  S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS, dnats += sum dS over later blocks (attns.py:719-983)
 //                  The query tiles (Q, dO, lse, delta) arrive by DMA in a ring of three LDS slots, two steps ahead.
+//                  One persistent workgroup per CU takes units from per-XCD work queues.
 //
 // Layouts follow the forward kernel: the stationary operand of a workgroup (Q, dO there; K, V here) sits in registers
 // as the B operand (lane = its row), the streamed tiles are row-major in LDS, the accumulators' own layout is the B
