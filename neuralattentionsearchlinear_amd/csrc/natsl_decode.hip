@@ -156,6 +156,14 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
   float m_run = -INFINITY, l_run = 0.f, acc[CPL];
 #pragma unroll
   for (int j = 0; j < CPL; ++j) acc[j] = 0.f;
+  // bf16 values are read like the keys, 16 lanes per row and 16 (8) bytes per lane, four rows per instruction: a lane then
+  // sums DV/16 adjacent columns over every fourth row, and the four row groups are added up once, at the end.  (One row
+  // per instruction with 4 bytes per lane, the f32 path below, keeps the memory pipe well below its rate.)
+  constexpr int EV = DV / 16;
+  float acc16[EV];
+#pragma unroll
+  for (int j = 0; j < EV; ++j) acc16[j] = 0.f;
+  const bool wide_v = p.dtype == NATSL_BF16;
   for (int k0 = 64 * (split * ATTN_WAVES + wave); k0 < p.TK; k0 += 64 * ATTN_WAVES * p.nsplit) {
     // scores: 16 lanes share a key row (16 bytes = 8 (bf16) or 4 (f32) elements each, one coalesced 256/512-byte
     // read per row), four rows per pass; the 16 partial dot products are summed across the lanes and the row's
@@ -212,6 +220,35 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
     m_run = m_new;
 #pragma unroll
     for (int j = 0; j < CPL; ++j) acc[j] *= alpha;
+    if (wide_v) {
+#pragma unroll
+      for (int j = 0; j < EV; ++j) acc16[j] *= alpha;
+      // the probabilities go to LDS (lane = key there) and come back to the lanes of their rows
+      sc[wave][lane] = pr;
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+      const int sub = lane & 15, rowg = lane >> 4;
+#pragma unroll 4
+      for (int pass = 0; pass < 16; ++pass) {
+        const int kidx = min(k0 + 4 * pass + rowg, p.TK - 1);   // keys past the end are clamped (their probability is 0)
+        const bf16_t* vrow = reinterpret_cast<const bf16_t*>(p.v) + (((size_t)b * p.TK + kidx) * p.HKV + hkv) * DV + EV * sub;
+        const float pk = sc[wave][4 * pass + rowg];
+        u32x4 w;
+        if (EV == 8) {
+          w = *reinterpret_cast<const u32x4*>(vrow);
+        } else {
+          const u32x2 w2 = *reinterpret_cast<const u32x2*>(vrow);
+          w = u32x4{w2[0], w2[1], 0u, 0u};
+        }
+#pragma unroll
+        for (int e = 0; e < EV / 2; ++e) {
+          acc16[2 * e] += pk * __uint_as_float(w[e] << 16);
+          acc16[2 * e + 1] += pk * __uint_as_float(w[e] & 0xffff0000u);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();   // sc[wave] is written again by the next chunk's scores
+      continue;
+    }
     // rows of V: keys past the end are clamped (their probability is 0)
     for (int kk = 0; kk < 64; kk += ATTN_VROWS) {
       float vv[ATTN_VROWS][CPL];
@@ -242,8 +279,20 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
   }
   // join the waves
   if (lane == 0) { part_m[wave] = m_run; part_l[wave] = l_run; }
+  if (wide_v) {
 #pragma unroll
-  for (int j = 0; j < CPL; ++j) part_acc[wave][CPL * lane + j] = acc[j];
+    for (int j = 0; j < EV; ++j) {
+      acc16[j] += __shfl_xor(acc16[j], 16);
+      acc16[j] += __shfl_xor(acc16[j], 32);
+    }
+    if (lane < 16) {
+#pragma unroll
+      for (int j = 0; j < EV; ++j) part_acc[wave][EV * lane + j] = acc16[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) part_acc[wave][CPL * lane + j] = acc[j];
+  }
   __syncthreads();
   if (wave == 0) {
     float m = -INFINITY;
