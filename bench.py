@@ -66,9 +66,52 @@ def make_inputs(w, torch, device):
     return host, dev
 
 
-# HBM bytes per launch of the dominant kernel (read + written), from FETCH_SIZE / WRITE_SIZE counter runs of this
-# script scaled by a 1 GiB copy in the same run; the counter summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"hybrid_gdn_B8_T8192_H16_d128_p25": 864.7e6 + 302.6e6}
+def csrc_sha():
+    """sha256 over the kernel sources the library is built from: names the code a counter measurement belongs to."""
+    import hashlib
+    d = os.path.join(ROOT, "neuralattentionsearchlinear_amd", "csrc")
+    h = hashlib.sha256()
+    for f in sorted(os.listdir(d)):
+        if f.endswith((".hip", ".h")):
+            h.update(f.encode())
+            h.update(open(os.path.join(d, f), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch (read + written) per kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this script
+    whose summary is kept in profiles/bench_<workload>.md on a line `traffic-json: {...}`.  The line names the kernel
+    sources it was measured on (csrc_sha); counters of other sources are stale and are not reported."""
+    path = os.path.join(ROOT, "profiles", f"bench_{workload}.md")
+    if not os.path.exists(path):
+        return None, "no counter summary under profiles/"
+    for line in open(path):
+        if line.startswith("traffic-json:"):
+            rec = json.loads(line[len("traffic-json:"):])
+            if rec.get("csrc_sha") != csrc_sha():
+                return None, f"profiles/{os.path.basename(path)} was measured on other kernel sources ({rec.get('csrc_sha')})"
+            return rec, f"profiles/{os.path.basename(path)} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, csrc_sha {rec['csrc_sha']})"
+    return None, "no traffic-json line in the counter summary"
+
+
+def clock_probe(torch, device):
+    """Shader clock and matrix rate of a pure v_mfma_f32_32x32x16_bf16 loop, right after the timed steps."""
+    from neuralattentionsearchlinear_amd import _capi
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    n_wg, iters = 2 * cus, 40000
+    out = torch.zeros(2 * n_wg, dtype=torch.int64, device=device)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    _capi.check(_capi.lib().natsl_mfma_clock_probe(_capi.ptr(out), n_wg, 2000, _capi.stream_ptr(device)), "natsl_mfma_clock_probe")
+    ev[0].record()
+    _capi.check(_capi.lib().natsl_mfma_clock_probe(_capi.ptr(out), n_wg, iters, _capi.stream_ptr(device)), "natsl_mfma_clock_probe")
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = ev[0].elapsed_time(ev[1])
+    o = out.cpu().view(n_wg, 2).double()
+    mhz = float((o[:, 0] / o[:, 1]).median()) * 100.0
+    tflops = n_wg * 4 * iters * 4 * 32768.0 / (ms * 1e-3) / 1e12
+    return dict(clock_mhz_under_load=mhz, mfma_loop_tflops=tflops,
+                note="pure 32x32x16 bf16 MFMA loop, 2 workgroups x 4 waves per CU, launched right after the timed steps")
 
 
 def softmax_flops(types, T, block, K, V):
@@ -247,6 +290,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS))
+    ap.add_argument("--prewarm-ms", type=float, default=300.0,
+                    help="milliseconds of untimed load before the warm-up steps, to let the GPU clocks settle (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the slice timed on the CPU")
     ap.add_argument("--cpu-batch", type=int, default=8, help="sequences of the slice timed on the CPU")
@@ -295,6 +340,16 @@ def main():
     with torch.no_grad():
         if args.serial_branches or args.concurrent_branches:
             _mixed_common.CONCURRENT_BRANCHES = bool(args.concurrent_branches)
+        # The GPU leaves idle at reduced clocks and needs about 40 ms of load to settle (the first 30 steps of a cold
+        # run take up to 15 % longer per kernel): load it for --prewarm-ms with the same step before the W warm-up
+        # steps, so that a short run measures the steady state it would also reach after more steps.
+        t_pre = time.perf_counter()
+        n_pre = 0
+        while (time.perf_counter() - t_pre) * 1e3 < args.prewarm_ms:
+            step()
+            n_pre += 1
+            if n_pre % 8 == 0:
+                torch.cuda.synchronize()
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
@@ -338,21 +393,26 @@ def main():
     types_host = ty.cpu()
     f_attn = softmax_flops(types_host, w["T"], w["block"], w["K"], w["V"])
     f_gdn = gdn_flops(types_host, w["K"], w["V"])
+    B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
+    traffic, traffic_source = measured_traffic(args.workload)
+    # the linear branch (prep + scan kernels): algorithmic bytes = q, k, v read once, o written once, g and beta, final state
+    lin_bytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * 6 + B * H * K * V * 4
+    roof_lin = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=lin_bytes / (lin_ms * 1e-3) / 1e9,
+                    peak=PEAK_HBM_GBS, unit="GB/s", frac=lin_bytes / (lin_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                    traffic=(traffic or {}).get("linear_bytes"), launch_ms=lin_ms, algorithmic_bytes=lin_bytes,
+                    algorithmic_flops=f_gdn, frac_of_mfma_peak=f_gdn / (lin_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                    launch_ms_alone=lin_alone_ms)
     if f_attn >= f_gdn:
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", kernel="softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
-                    unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=MEASURED_TRAFFIC.get(args.workload), launch_ms=sm_ms,
-                    algorithmic_flops=f_attn,
+                    unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=(traffic or {}).get("softmax_bytes"),
+                    traffic_source=traffic_source, launch_ms=sm_ms, algorithmic_flops=f_attn,
                     # the same kernel with the GPU to itself (branches launched one after the other, outside the timed region)
                     launch_ms_alone=sm_alone_ms, frac_alone=f_attn / (sm_alone_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS)
     else:
-        # GDN-only workload: HBM-bound; algorithmic bytes = q,k,v read + o written + g,beta + final state
-        B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
-        nbytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * 6 + B * H * K * V * 4
-        achieved = nbytes / (lin_ms * 1e-3) / 1e9
-        roof = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=achieved, peak=PEAK_HBM_GBS,
-                    unit="GB/s", frac=achieved / PEAK_HBM_GBS, traffic=None, launch_ms=lin_ms, algorithmic_bytes=nbytes,
-                    launch_ms_alone=lin_alone_ms, frac_alone=nbytes / (lin_alone_ms * 1e-3) / 1e9 / PEAK_HBM_GBS)
+        # GDN-only workload: HBM-bound
+        roof = dict(roof_lin, traffic_source=traffic_source)
+    probe = clock_probe(torch, device)
 
     rec = dict(
         metric="hybrid-layer fwd tokens/sec @T=8192,H=16,d=128 bf16; % of MFMA/HBM roofline",
@@ -362,6 +422,9 @@ def main():
                     softmax_ms=sm_ms, linear_ms=lin_ms, softmax_alone_ms=sm_alone_ms, linear_alone_ms=lin_alone_ms, step_flops=f_attn + f_gdn,
                     step_frac_of_mfma_peak=(f_attn + f_gdn) / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS),
         roofline=roof,
+        roofline_linear=roof_lin,
+        clock=probe,
+        prewarm=dict(ms=args.prewarm_ms, steps=n_pre),
     )
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(host, w, types_host, torch, max_heads=args.cpu_heads, max_batch=args.cpu_batch)

@@ -219,6 +219,12 @@ int natsl_kv_compact(const void* src_k, const void* src_v, long long src_tokens,
                      int HN, int K, int V, int dtype, int block, int NB, int n_complete, int tail_dst, int tail_tokens,
                      natsl_stream_t stream);
 
+/* Measurement aid (no counterpart in the reference; used by the benchmark only): n_workgroups workgroups of 4 waves each
+ * run `iters` rounds of four independent 32x32x16 bf16 matrix instructions per wave (iters * 4 * 32768 FLOPs per wave) and
+ * write, per workgroup, out[2i] = shader-clock cycles and out[2i+1] = ticks of the constant 100 MHz counter the loop took:
+ * cycles / ticks * 100 is the shader clock in MHz under a dense matrix load. */
+int natsl_mfma_clock_probe(unsigned long long* out, int n_workgroups, int iters, natsl_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

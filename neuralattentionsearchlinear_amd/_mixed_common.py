@@ -153,8 +153,11 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
     _mark("linear:end", cur)
     if side is not cur:
         cur.wait_stream(side)
-        for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks'], o_attn):
+        # tensors allocated on the caller's stream and read on the side stream, and the side stream's own output
+        # that the caller's stream goes on to use
+        for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks']):
             t.record_stream(side)
+        o_attn.record_stream(cur)
     if io_dtype != torch.bfloat16:
         o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
     if not inference:

@@ -195,7 +195,7 @@ class NAtSLayerCache:
             types = types.float()
         types = types.contiguous()
         B, NB, HN, _ = types.shape
-        new_blocks = (types[:, :n_complete, :, self.attn_offset] == 1).sum(1)                     # int64 [B, HN]
+        new_blocks = (torch.round(types[:, :n_complete, :, self.attn_offset].float()) == 1).sum(1)                     # int64 [B, HN]
         before = self.n_attn_blocks
         after = new_blocks if before is None else before + new_blocks
         new_max = int(after.max()) if after.numel() else 0                                        # one host sync per completed block

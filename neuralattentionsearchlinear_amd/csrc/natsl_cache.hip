@@ -39,7 +39,7 @@ NATSL_DEVICE bool kv_is_attn(const KvCompactParams& p, int b, int s, int hn) {
   size_t i = (((size_t)b * p.NB + s) * p.HN + hn) * 2;
   float t = p.types_dtype == NATSL_F32 ? reinterpret_cast<const float*>(p.types)[i]
                                        : bf16_to_f32(reinterpret_cast<const bf16_t*>(p.types)[i]);
-  return t == 1.0f;
+  return rintf(t) == 1.0f;   // the predicate of the router and of both branches (mixed_attn_gdn.py:88 rounds the types)
 }
 
 __global__ __launch_bounds__(256) void kv_compact_kernel(KvCompactParams p) {

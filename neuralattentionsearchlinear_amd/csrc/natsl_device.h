@@ -16,14 +16,6 @@
 
 namespace natsl {
 
-// Ablation switches for kernel development (skip loads / compute to time the remainder).  They exist
-// only in a build with -DNATSL_ABLATE; the shipped library compiles them to nothing.
-#ifdef NATSL_ABLATE
-#define NATSL_ABL(x) (x)
-#else
-#define NATSL_ABL(x) false
-#endif
-
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;

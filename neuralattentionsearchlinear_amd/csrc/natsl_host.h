@@ -8,7 +8,7 @@
 
 namespace natsl {
 
-char* error_buffer();  // thread-local, 512 bytes (natsl_capi.hip)
+char* error_buffer();  // thread-local, 512 bytes (defined in natsl_route.hip)
 
 inline int fail(int code, const char* fmt, ...) {
   va_list ap;

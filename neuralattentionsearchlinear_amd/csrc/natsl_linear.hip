@@ -29,9 +29,6 @@
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
 #include "natsl_device.h"
 #include "natsl_host.h"
-#ifdef NATSL_ABLATE
-#include <stdlib.h>  // development build only: getenv for the ablation switch
-#endif
 
 namespace natsl {
 
@@ -58,18 +55,10 @@ struct LinearParams {
   bf16_t* ws_tm;
   bf16_t* ws_p;
   float* ws_sc;
-  int dbg;
 };
 
 constexpr int C = 64;
 constexpr int BV = 32;
-
-// Development build only: per-phase cycle counters of the scan's step, written over the first floats of ht.
-#ifdef NATSL_PHASE_TIMING
-#define NATSL_TICK(i) { const long long now_ = __builtin_readcyclecounter(); tacc[i] += now_ - tlast; tlast = now_; }
-#else
-#define NATSL_TICK(i)
-#endif
 
 NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
   float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i]
@@ -150,7 +139,6 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
       rk[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
     }
   }
-  if (NATSL_ABL(p.dbg & 32)) return;  // loads only
   // ---- gamma = inclusive cumsum of g over the chunk (wave 0), beta -------------------------
   if (wave == 0) {
     const bool ok = t0 + lane < len;
@@ -258,7 +246,6 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     }
   }
   if (!DELTA) return;
-  if (NATSL_ABL(p.dbg & 64)) return;  // no solve, no Tm store
   __syncthreads();
 
   // ---- X = (I + A)^-1 in fp32, 4x4 blocks of 16x16 ------------------------------------------
@@ -316,7 +303,7 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     __syncthreads();
   }
   // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above)
-  if (!NATSL_ABL(p.dbg & 128)) {
+  {
     const int row = tid >> 2, cb = tid & 3;
     float x[16];
 #pragma unroll
@@ -491,27 +478,16 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
   };
 
   float gsum = 0.f;
-#ifdef NATSL_PHASE_TIMING
-  long long tacc[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_readcyclecounter();
-#endif
   // one chunk: CUR holds its operands, kbuf/vbuf[buf] its k and v tiles
   Staging G;
   auto step = [&](const int c, const int buf, Operands& CUR) {
-    NATSL_TICK(9)
     __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
-    NATSL_TICK(0)
     // Loads are issued unconditionally (chunk indices clamped to the last chunk): a load inside a
     // branch would force the waits below to assume it may not have been issued, i.e. to drain the queue.
     const int c1 = min(c + 1, NT - 1), c2 = min(c + 2, NT - 1);
     const float dec_c = CUR.dec, glast_c = CUR.glast, linf_c = CUR.linf;
     load_scalars(CUR, c2);  // first, so that nothing younger has to be waited for along with them
     gload_kv(G, c1);
-    if (NATSL_ABL(p.dbg & 4)) {
-      load_q(CUR, c2); load_se(CUR, c2); load_T(CUR, c2); load_sk(CUR, c2); load_P(CUR, c2); load_sq(CUR, c2);
-      __syncthreads(); __syncthreads();
-      lstore(G, buf ^ 1);
-      return;
-    }
 
     if (c % per_blk == 0) {
 #pragma unroll
@@ -537,7 +513,6 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
       O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
     }
-    NATSL_TICK(1)
     load_q(CUR, c2);
     // (2) v in accumulator layout via the transposing read; X = v - se * R
     f32x4 VN[2];
@@ -556,9 +531,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
         *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + perm0) = pack4(X);
       }
       load_se(CUR, c2);
-      NATSL_TICK(2)
       __syncthreads();
-      NATSL_TICK(3)
       // (3) v_new = TmB X
 #pragma unroll
       for (int nn = 0; nn < 2; ++nn) {
@@ -578,9 +551,7 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
     }
     load_sk(CUR, c2);
-    NATSL_TICK(4)
     __syncthreads();
-    NATSL_TICK(5)
     // (5) o = sq * O1 + P v_new
 #pragma unroll
     for (int nn = 0; nn < 2; ++nn) {
@@ -604,7 +575,6 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
       if (tok < len)
         *reinterpret_cast<u32x4*>(op + (size_t)tok * v_row + 8 * (lane & 3)) = *reinterpret_cast<const u32x4*>(Os + row * VP + 8 * (lane & 3));
     }
-    NATSL_TICK(6)
     // (6) state update / roll-back
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
     gsum += glast_c;
@@ -636,11 +606,9 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
 #pragma unroll
           for (int r = 0; r < 4; ++r) S[mi][nn][r] = Ssave[mi][nn][r] * f;
     }
-    NATSL_TICK(7)
     // (7) bf16 copy of the state and the staged k, v tiles for the next step
     write_ST();
     lstore(G, buf ^ 1);
-    NATSL_TICK(8)
   };
 
   Operands A0, A1;
@@ -680,12 +648,6 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
           p.ht[((size_t)chain * DK + kd) * p.V + vc] = S[mi][nn][r];
         }
   }
-#ifdef NATSL_PHASE_TIMING
-  if (p.ht && blockIdx.x == 17 && (tid & 63) == 0) {
-    __syncthreads();
-    for (int i = 0; i < 10; ++i) p.ht[10 * wave + i] = (float)tacc[i] / NT;
-  }
-#endif
 }
 
 constexpr size_t WS_UNIT_BYTES = (size_t)C * C * 2 * 2 + 4 * C * 4;
@@ -725,10 +687,6 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
   p.nt = cdiv(T, C);
   p.total_chunks = seqs ? total_units : B * p.nt;
   p.scale = scale; p.flags = flags;
-  p.dbg = 0;
-#ifdef NATSL_ABLATE
-  if (getenv("NATSL_DBG")) p.dbg = atoi(getenv("NATSL_DBG"));
-#endif
   const size_t units = (size_t)p.total_chunks * H;
   const size_t need = natsl_linear_workspace_bytes(p.total_chunks, H);
   if (!workspace || workspace_bytes < need) return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);

@@ -13,9 +13,6 @@
 #include "natsl_device.h"
 #include "natsl_host.h"
 #include <type_traits>
-#ifdef NATSL_ABLATE
-#include <stdlib.h>  // development build only: getenv for the ablation switches
-#endif
 
 namespace natsl {
 
@@ -38,7 +35,6 @@ struct SoftmaxParams {
   int same_block;
   int variant;  // 4: 128-query tile on 4 waves, 8: 256-query tile on 8 waves
   int g_kv, g_n;  // query heads per kv head / per selector head
-  int dbg;      // ablation bits, always 0 unless built with NATSL_ABLATE
 };
 
 NATSL_DEVICE bool type_is_one(const void* types, int dtype, size_t i) {
@@ -133,9 +129,6 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
   // operand j of the chunk: K rows of half j/KS at k-step j%KS, then V^T rows (half, 16-key group ss, value tile vt);
   // the 16-key groups of odd value tiles are stored swapped
   auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
-#ifdef NATSL_ABL_NOLDS
-    return QB[j % KS];
-#endif
     if (j < NK) return ld8(krow + 32 * (j / KS) * KP + 16 * (j % KS));
     const int i = j - NK, half = i / (2 * VT), ss = (i / VT) & 1, vt = i % VT;
     const bf16_t* vr = vrow + 32 * vt * TP + 16 * ((2 * half + ss) ^ (vt & 1));
@@ -164,9 +157,7 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
   }
   if (causal) mask_half(s0, 0, lane, qloc0);
   float mx = half_max(s0, c);
-#ifndef NATSL_ABL_NOCHECK
   if (__any(mx > m_ref + RESCALE_SLACK)) rescale<DV>(acc, m_ref, l_run, mx);
-#endif
   float neg = m_ref == -INFINITY ? 0.f : -m_ref;
   float rs = 0.f;
   bf16x8 PB0[2], PB1[2];
@@ -187,7 +178,6 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
   }
   if (causal) mask_half(s1, 1, lane, qloc0);
   mx = half_max(s1, c);
-#ifndef NATSL_ABL_NOCHECK
   if (__any(mx > m_ref + RESCALE_SLACK)) {
     // the second half outgrew the reference: move it, and form the first half's probabilities again
     rescale<DV>(acc, m_ref, l_run, mx);
@@ -195,7 +185,6 @@ NATSL_DEVICE void chunk_pipelined(const bf16_t* Kb, const bf16_t* VTb, const bf1
     rs = 0.f;
     probs_half(s0, c, neg, rs, PB0);
   }
-#endif
 
   // ---- PV(0) with exp(1)
 #pragma unroll
@@ -896,7 +885,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
           active = active && jc < my_chunk && kblk < my_blk && ((diag_attn >> (kblk - dblk)) & 1ull);
         }
       }
-      if (active && !NATSL_ABL(p.dbg & 2))
+      if (active)
         chunk_pipelined<DK, DV>(Ks + buf * 64 * KP, Vs + buf * DV * TP, QB, acc, m_ref, l_run, c, lane, causal, qloc0);
     };
 
@@ -1009,14 +998,9 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.same_block = same_block_visible ? 1 : 0;
   p.g_kv = HQ / HKV;
   p.g_n = HQ / HN;
-  p.dbg = 0;
   // 256-query tiles on 8 waves once there is at least one of them per CU (measured: from there on that shape is the
   // faster one; below, the 128-query tiles fill more CUs)
   p.variant = (long long)B * HQ * cdiv(T, 256) >= 256 ? 8 : 4;
-#ifdef NATSL_ABLATE
-  if (getenv("NATSL_DBG")) p.dbg = atoi(getenv("NATSL_DBG"));
-  if (getenv("NATSL_SOFTMAX_WAVES")) p.variant = atoi(getenv("NATSL_SOFTMAX_WAVES"));
-#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define NATSL_SM(KK, VV)                                              \
   if (K == KK && V == VV)                                             \

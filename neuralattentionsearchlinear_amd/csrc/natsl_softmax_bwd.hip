@@ -822,9 +822,6 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     size_t lds = (size_t)3 * (64 * (DK + DV) * sizeof(bf16_t) + 512);   // the ring of three query tiles
     const size_t red = (size_t)2 * (DV / 32 + DK / 32) * 16 * 64 * sizeof(float);
     if (red > lds) lds = red;
-    // the DMA requests address a sequence's rows with 32-bit byte offsets
-    if ((long long)p.T * p.HQ * (DK > DV ? DK : DV) * 2 >= (1ll << 32))
-      return fail(NATSL_ERR_UNSUPPORTED, "softmax bwd: T * HQ = %lld rows of one sequence exceed the 32-bit offsets of the dk/dv kernel", (long long)p.T * p.HQ);
     auto kern = dkdv_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
@@ -859,6 +856,11 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
   if (HQ % HKV || HQ % HN) return fail(NATSL_ERR_INVALID, "%s: HQ=%d must be a multiple of HKV=%d and HN=%d", what, HQ, HKV, HN);
   if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
   if (TN != cdiv(T, block)) return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d", what, TN, T, block);
+  // the dk/dv kernel's DMA requests address the rows of one sequence with 32-bit byte offsets: checked here, before
+  // anything is launched
+  if ((long long)T * HQ * (K > V ? K : V) * 2 >= (1ll << 32))
+    return fail(NATSL_ERR_UNSUPPORTED, "%s: T * HQ * max(K, V) * 2 = %lld bytes per sequence exceed the kernel's 32-bit row offsets",
+                what, (long long)T * HQ * (K > V ? K : V) * 2);
   if (!workspace || workspace_bytes < natsl_softmax_bwd_workspace_bytes(B, T, HQ))
     return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", what, natsl_softmax_bwd_workspace_bytes(B, T, HQ));
   SoftmaxBwdParams p;

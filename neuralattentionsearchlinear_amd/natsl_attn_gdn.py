@@ -147,6 +147,13 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
         if cache is not None and cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported together with a cache")
 
+        if cache is not None and mode != 'chunk' and q_len > 1:
+            # refuse BEFORE the cache is touched: a refused step must leave it as it was
+            if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
+                raise NotImplementedError("a decode step of several tokens that crosses a selector-block boundary is not built: "
+                                          "split it at the boundary")
+            if self.ops_for_incomplete_chunks == 'gated_delta_net':
+                raise NotImplementedError("several new tokens per decode step are not built for ops_for_incomplete_chunks=gated_delta_net")
         # selector: on a cache, over the tokens of the incomplete block + the new ones, once they complete a block
         if cache is not None:
             selector_input = cache.update_attn_types(input_hidden_states=hidden_states)

@@ -176,3 +176,11 @@ def test_layer_rejects_what_the_cache_cannot_do():
             layer(xd[:, 100:200], past_key_values=cache, use_cache=True)      # a second chunked forward
         with pytest.raises(NotImplementedError):
             layer(xd[:, 100:140], past_key_values=cache, use_cache=True)      # 36 + 40 tokens cross a block boundary
+        # a refused step leaves the cache as it was: the same tokens fed one at a time afterwards give what an
+        # untouched cache gives
+        fresh = NAtSCache()
+        layer(xd[:, :100], past_key_values=fresh, use_cache=True)
+        for t in range(100, 104):
+            a = layer(xd[:, t:t + 1], past_key_values=cache, use_cache=True)[0]
+            b = layer(xd[:, t:t + 1], past_key_values=fresh, use_cache=True)[0]
+            assert torch.equal(a, b), f"token {t} differs after a refused step"

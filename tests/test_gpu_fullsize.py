@@ -237,3 +237,75 @@ def test_c4_mamba_homogeneity_and_hand_off():
     sc = (q[1, :, 4].float() @ k[1, :, 4].float().T) * K ** -0.5
     ref = torch.softmax(sc.masked_fill(~mask, float('-inf')), -1) @ v[1, :, 4].float()
     assert_close(oa1[1, :, 4].float(), ref, "o_attn slice")
+
+
+# --------------------------------------------------------------------------------------------
+# full-depth checks of the Gated-DeltaNet chain against the fp64 token recurrence, one (sequence, head)
+# slice at a time (the recurrence runs on the host: a slice of 65 536 tokens takes a few seconds)
+# --------------------------------------------------------------------------------------------
+def _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o, s, b, h, block, scale, t0=0, t1=None, s_index=None, what=""):
+    """Slice (b, h), tokens [t0, t1) of the packed row, of the kernel's output `o` and final state `s` against the
+    oracle's token-by-token recurrence in fp64 under the drawn block types.  Returns the measured errors."""
+    from oracle import linear_branch as LB
+    t1 = q.shape[1] if t1 is None else t1
+    sl = lambda t: t[b:b + 1, t0:t1, h:h + 1].float().cpu()
+    lin = ty[b:b + 1, t0 // block:-(-t1 // block), h:h + 1, 1].float().cpu()
+    o_ref, s_ref = LB.gdn_token_recurrence(sl(q), sl(k), sl(v), sl(g), sl(beta), lin, scale, None, block=block)
+    e_o = assert_close(o[b:b + 1, t0:t1, h:h + 1].float(), o_ref, f"{what} o_gdn[{b},{t0}:{t1},{h}]")
+    si = b if s_index is None else s_index
+    e_s = assert_close(s[si:si + 1, h:h + 1], s_ref, f"{what} final_state[{si},{h}]")
+    # the tail of the chain on its own: an error that grows with depth shows here first
+    tail = slice(t1 - t0 - 1024, t1 - t0)
+    e_t = assert_close(o[b:b + 1, t0:t1, h:h + 1][:, tail].float(), o_ref[:, tail], f"{what} last 1024 tokens of o_gdn[{b},:,{h}]")
+    print(f"\n{what} slice ({b},{h}) tokens {t0}:{t1}: o max-abs {e_o[0]:.2e} rel-L2 {e_o[1]:.2e}; "
+          f"last 1024 tokens rel-L2 {e_t[1]:.2e}; final state max-abs {e_s[0]:.2e} rel-L2 {e_s[1]:.2e}", flush=True)
+    return e_o, e_s
+
+
+def test_c2_gdn_full_depth_slices_against_token_recurrence(c2):
+    """c2 with the drawn mask (25 % attention blocks, decay across them): 128 chunks deep."""
+    w = C2
+    scale = w['K'] ** -0.5
+    o, s = _linear('gdn', c2['q'], c2['k'], c2['v'], c2['g'], c2['beta'], None, c2['ty'], w['block'], scale)
+    for b, h in ((0, 0), (6, 13)):
+        _gdn_slice_against_token_recurrence(c2['q'], c2['k'], c2['v'], c2['g'], c2['beta'], c2['ty'], o, s, b, h, w['block'], scale, what="c2")
+
+
+def test_c3_unpacked_single_sequence_against_the_oracle():
+    """c3 as ONE sequence: B1 T65536 H32 K=V=128, 10 % attention blocks; 1024 chunks deep.
+    Gated DeltaNet: two head slices against the fp64 token recurrence.  Softmax branch: the last 512 queries and a
+    window in the middle of one head against the dense fp32 masked softmax over all 65 536 keys."""
+    T, H, K, V, block = 65536, 32, 128, 128, 64
+    q, k, v, g, beta = _inputs(1, T, H, K, V, 900)
+    ty = make_types(1, T // block, H, 0.10, 31, torch.bfloat16).to(DEV)
+    scale = K ** -0.5
+    o_lin, s = _linear('gdn', q, k, v, g, beta, None, ty, block, scale)
+    o_attn, lse = _softmax(q, k, v, ty, block, scale, True)
+    assert torch.isfinite(o_lin.float()).all() and torch.isfinite(s).all() and torch.isfinite(o_attn.float()).all()
+    for h in (0, 21):
+        _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o_lin, s, 0, h, block, scale, what="c3")
+    h = 17
+    mask_rows = SB.visibility_mask(ty[0, :, h, 0].float().cpu(), T, block, True)
+    kf, vf = k[0, :, h].float(), v[0, :, h].float()
+    for a, b_ in ((T - 512, T), (T // 2 - 256, T // 2 + 256)):
+        m = mask_rows[a:b_].to(DEV)
+        sc = ((q[0, a:b_, h].float() @ kf.T) * scale).masked_fill(~m, float('-inf'))
+        ref = torch.softmax(sc, -1) @ vf
+        assert_close(o_attn[0, a:b_, h].float(), ref, f"c3 o_attn[0,{a}:{b_},{h}]")
+        lse_ref = torch.logsumexp(sc, -1) * 1.4426950408889634
+        assert float((lse[0, a:b_, h] - lse_ref).abs().max()) <= 2e-2, "c3 lse (log2 units)"
+
+
+def test_c3_packed_sequence_against_token_recurrence():
+    """The packed c3 row (8192/16384/16384/24576 via cu_seqlens): the longest sequence's chain, cut out of the packed
+    call's output, against the token recurrence started from a zero state at that sequence's first token."""
+    from neuralattentionsearchlinear_amd.nats_util import pack_sequences
+    T, H, K, V, block = 65536, 32, 128, 128, 64
+    cu = [0, 8192, 24576, 40960, 65536]
+    q, k, v, g, beta = _inputs(1, T, H, K, V, 500)
+    ty = torch.cat([make_types(1, (b - a) // block, H, 0.10, 20 + i, torch.bfloat16) for i, (a, b) in enumerate(zip(cu[:-1], cu[1:]))], 1).to(DEV)
+    scale = K ** -0.5
+    seqs = pack_sequences(torch.tensor(cu, dtype=torch.int64, device=DEV), None, block, torch.device(DEV))
+    o_lin, s = _linear('gdn', q, k, v, g, beta, None, ty, block, scale, seqs=seqs)
+    _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o_lin, s, 0, 9, block, scale, t0=cu[3], t1=cu[4], s_index=3, what="c3 packed")
+    _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o_lin, s, 0, 30, block, scale, t0=cu[1], t1=cu[2], s_index=1, what="c3 packed")
