@@ -202,6 +202,18 @@ int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uin
                           int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
                           size_t workspace_bytes, natsl_stream_t stream);
 
+/* natsl_attn_masked_fwd for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): the same kernels with the split scratch in a device array of the library itself, so the caller
+ * passes inputs and outputs only and the call allocates nothing.  It has no counterpart in the reference.  The array
+ * holds natsl_attn_masked_static_scratch_bytes() = 256 KiB per GPU for the life of the process; a shape whose splits need
+ * more (natsl_attn_masked_workspace_bytes() above that limit) is refused with NATSL_ERR_WORKSPACE.  Results are
+ * identical to natsl_attn_masked_fwd with a workspace.  All calls on one GPU share the array: calls that overlap on
+ * one GPU (different streams or threads) race. */
+size_t natsl_attn_masked_static_scratch_bytes(void);
+int natsl_attn_masked_fwd_static(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
+                                 int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype,
+                                 natsl_stream_t stream);
+
 /* KV cache of the softmax branch: keep the attention-typed blocks of a region of new tokens, per (sequence, kv
  * head), back to back behind the blocks already kept, and put the tokens of the incomplete last block at block
  * index tail_dst (the same for every head; pass -1 when the region ends on a block boundary).

@@ -52,6 +52,9 @@ _SIGNATURES = {
     "natsl_attn_masked_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "natsl_attn_masked_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_int, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "natsl_attn_masked_static_scratch_bytes": (c_size_t, []),
+    "natsl_attn_masked_fwd_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                             c_int, c_int, c_float, c_int, c_void_p]),
     "natsl_mfma_clock_probe": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "natsl_kv_compact": (c_int, [c_void_p, c_void_p, c_longlong, c_int, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -411,10 +411,11 @@ extern "C" size_t natsl_attn_masked_workspace_bytes(int B, int TQ, int TK, int H
   return ns > 1 ? (size_t)B * TQ * HQ * ns * (2 + V) * sizeof(float) : 0;
 }
 
-extern "C" int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
-                                     int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
-                                     size_t workspace_bytes, natsl_stream_t stream) {
-  const char* what = "natsl_attn_masked_fwd";
+// The one implementation behind both entry points.  `strict`: a workspace smaller than the split needs is an error
+// instead of a silent fall-back to one workgroup per query.
+static int attn_masked_run(const char* what, const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
+                           int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
+                           size_t workspace_bytes, bool strict, natsl_stream_t stream) {
   if (!q || !k || !v || !mask || !o) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: tensors must be f32 or bf16", what);
   if (B <= 0 || TQ <= 0 || TK <= 0 || HQ <= 0 || HKV <= 0 || HM <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
@@ -425,7 +426,12 @@ extern "C" int natsl_attn_masked_fwd(const void* q, const void* k, const void* v
   p.scale_log2 = scale * 1.4426950408889634f;
   // without a workspace (or with one that is too small) every query is handled by one workgroup
   p.nsplit = attn_masked_splits(B, TQ, TK, HQ);
-  if (!workspace || workspace_bytes < natsl_attn_masked_workspace_bytes(B, TQ, TK, HQ, V)) p.nsplit = 1;
+  const size_t need = natsl_attn_masked_workspace_bytes(B, TQ, TK, HQ, V);
+  if (!workspace || workspace_bytes < need) {
+    if (strict && need > 0)
+      return fail(NATSL_ERR_WORKSPACE, "%s: this shape needs %zu bytes of split scratch, the built-in buffer holds %zu", what, need, workspace_bytes);
+    p.nsplit = 1;
+  }
   p.partials = reinterpret_cast<float*>(workspace);
   if (TQ > 65535 || HQ > 65535 || (long long)B * p.nsplit > 65535) return fail(NATSL_ERR_UNSUPPORTED, "%s: grid dimension above 65535", what);
   const dim3 grid(TQ, HQ, B * p.nsplit), jgrid(TQ, HQ, B);
@@ -442,4 +448,58 @@ extern "C" int natsl_attn_masked_fwd(const void* q, const void* k, const void* v
   NATSL_MA(128, 64)
 #undef NATSL_MA
   return fail(NATSL_ERR_UNSUPPORTED, "%s: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", what, K, V);
+}
+
+extern "C" int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
+                                     int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
+                                     size_t workspace_bytes, natsl_stream_t stream) {
+  return attn_masked_run("natsl_attn_masked_fwd", q, k, v, mask, o, B, TQ, TK, HQ, HKV, HM, K, V, scale, dtype, workspace,
+                         workspace_bytes, false, stream);
+}
+
+// ---- the variant that allocates nothing -----------------------------------------------------------------------------
+// The split scratch (per query and split: running maximum, sum and DV partial outputs, fp32) lives in a device array
+// of this library instead of a caller's workspace.  Every GPU holds its own copy at its own address until the process
+// ends; the array's name is a host-side handle, so its device address is looked up once per device and only that
+// pointer is ever handed to a kernel.  Nothing in it has to start at zero: every (query, split) slot that the join
+// kernel reads is written by the split kernel of the same call.  Calls that overlap on one GPU share the array and race.
+#define NATSL_ATTN_STATIC_SCRATCH_BYTES (256u << 10)
+static __device__ __align__(256) unsigned char scratch[NATSL_ATTN_STATIC_SCRATCH_BYTES];
+
+#include <mutex>
+static void* scratch_device_address(const char* what, int* rc) {
+  constexpr int MAX_DEVICES = 64;
+  static void* ptr[MAX_DEVICES];
+  static std::mutex mu;
+  *rc = NATSL_OK;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    *rc = fail(NATSL_ERR_LAUNCH, "%s: cannot name the current device (%s)", what, hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* a = nullptr;
+    e = hipGetSymbolAddress(&a, HIP_SYMBOL(scratch));   // with device `dev` current: that device's copy
+    if (e != hipSuccess || !a) {
+      *rc = fail(NATSL_ERR_LAUNCH, "%s: hipGetSymbolAddress failed on device %d (%s)", what, dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr[dev] = a;
+  }
+  return ptr[dev];
+}
+
+extern "C" size_t natsl_attn_masked_static_scratch_bytes(void) { return NATSL_ATTN_STATIC_SCRATCH_BYTES; }
+
+extern "C" int natsl_attn_masked_fwd_static(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B,
+                                            int TQ, int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype,
+                                            natsl_stream_t stream) {
+  const char* what = "natsl_attn_masked_fwd_static";
+  int rc;
+  void* ws = scratch_device_address(what, &rc);
+  if (!ws) return rc;
+  return attn_masked_run(what, q, k, v, mask, o, B, TQ, TK, HQ, HKV, HM, K, V, scale, dtype, ws, NATSL_ATTN_STATIC_SCRATCH_BYTES,
+                         true, stream);
 }
