@@ -14,16 +14,20 @@
 //                                               sk = rk e^{gamma_last-gamma}, {e^{gamma_last}, gamma_last, is_linear}
 //                        (rq, rk = reciprocal L2 norms, or 1).
 //
-//   linear_scan_kernel   one workgroup per (sequence, head, 32-wide slice of V) walks the chunks
-//                        in order with the state slice S[K][32] in fp32 registers:
+//   linear_scan_kernel   walks the chunks of one (sequence, head) in order.  A wave owns 16 columns of the state
+//                        for ALL K rows, as the fp32 accumulators of 16x16x32 matrix instructions:
 //                          R = k S;  X = v - se*R;  v_new = TmB X               (delta rule)
 //                          o = sq*(q S) + P v_new
-//                          S <- e^{gamma_last} S + (sk*k)^T v_new               (blocks typed linear)
-//                        q, k, TmB, P reach the matrix cores straight from global memory in
-//                        A-operand layout; only what changes layout goes through LDS (S, X, v_new
-//                        written transposed from the accumulator layout, k read back transposed
-//                        with the transposing LDS load).  Raw q, k are used: the 1/norm factors
-//                        are folded into the per-token scale vectors.
+//                          S <- e^{gamma_last} S + k^T (sk*v_new)               (blocks typed linear)
+//                        With the columns in the lanes, every product above takes the state, X and v_new as the
+//                        B operand STRAIGHT FROM THE ACCUMULATOR REGISTERS (rounded to bf16 in place): an accumulator
+//                        tile holds, per lane, four consecutive rows, and two tiles side by side are the eight
+//                        contraction slots of a lane -- under a fixed relabelling of the contraction index that the
+//                        A operand follows (which K row a state register holds; which token a column of TmB / P
+//                        stands for, chosen by the prep kernel).  Nothing state-dependent goes through LDS and the
+//                        waves never exchange data: the only barrier of a step hands over the next chunk's inputs.
+//                        Those (k, q, v tiles, TmB, P, sc) arrive by LDS-DMA, double buffered, one chunk ahead.
+//                        Raw q, k are used: the 1/norm factors are folded into the per-token scale vectors.
 //                        A block that is not typed linear leaves S rolled back at its end (times
 //                        e^{sum g} when decay is on), which is all the reference's carry logic
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
@@ -58,7 +62,6 @@ struct LinearParams {
 };
 
 constexpr int C = 64;
-constexpr int BV = 32;
 
 NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
   float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i]
@@ -160,11 +163,11 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
   float* Sout = p.ws_sc + unit * (4 * C);
 
   // ---- Gram products on the matrix cores: wave w owns the 32x32 tile (w/2, w%2) ------------
-  // P and TmB are stored in the order the scan kernel consumes them as MFMA A operands, so that its
-  // loads are contiguous: the 16 bytes of scan-lane (row i%16, group g4) of 16-row band i/16 and
-  // k-step s sit at ((2(i/16) + s) * 64 + 16 g4 + i%16) * 16 bytes.  Within a k-step the 32
-  // contraction tokens are permuted: slot (g4, e) holds token 8(2(g4&1) + e/4) + 4(g4/2) + e%4,
-  // which is how one lane of the transposed 32x32 Gram accumulator holds them.
+  // P and TmB are stored as the scan kernel's MFMA A operands (16x16x32: 16 rows x 32 contraction tokens), 1 KiB each,
+  // operand (t, s) = rows 16t.., tokens 32s.. at index 2t + s; in it, scan-lane (row i%16, group g) finds its 16 bytes
+  // at (16 g + i%16) * 16.  The scan feeds the other operand from accumulator registers, where lane group g holds
+  // tokens 4g..4g+3 of a 16-token tile, so slot j of group g stands for token 32s + 16(j/4) + 4g + j%4.
+  // Operands (0,1) and (1,1) lie above the diagonal: never written, never read.
   {
     const int ti = wave >> 1, tj = wave & 1, l32 = lane & 31, hf = lane >> 5;
     const int i = 32 * ti + l32;  // P row owned by this lane
@@ -187,6 +190,8 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
       {
         // this lane's 16 key tokens are four runs of four: 16-byte reads of their gamma and 1/|k|
         const float gi = gam[i], fi = p.scale * rq[i];
+        // this lane holds tokens 8 q4 + 4 hf + e of the tile: q4 = 0, 2 are the two halves of group hf's slots,
+        // q4 = 1, 3 those of group 2 + hf
         u32x4 w[2];
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
@@ -195,17 +200,12 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
           float pv[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) pv[e] = i >= j0 + e ? fi * rj[e] * gq[4 * q4 + e] * __expf(gi - gj[e]) : 0.f;
-          w[q4 >> 1][2 * (q4 & 1)] = pack_bf16x2(pv[0], pv[1]);
-          w[q4 >> 1][2 * (q4 & 1) + 1] = pack_bf16x2(pv[2], pv[3]);
+          w[q4 & 1][2 * (q4 >> 1)] = pack_bf16x2(pv[0], pv[1]);
+          w[q4 & 1][2 * (q4 >> 1) + 1] = pack_bf16x2(pv[2], pv[3]);
         }
-        *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = w[0];
-        *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = w[1];
+        *reinterpret_cast<u32x4*>(prow + hf * 128) = w[0];
+        *reinterpret_cast<u32x4*>(prow + (2 + hf) * 128) = w[1];
       }
-    } else {
-      // the strictly upper 32x32 tile is zero
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      *reinterpret_cast<u32x4*>(prow + (2 * hf) * 128) = z;
-      *reinterpret_cast<u32x4*>(prow + (2 * hf + 1) * 128) = z;
     }
     if (DELTA) {
       // all waves are done reading the q, k tiles before the A blocks overwrite them
@@ -302,57 +302,112 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
     }
     __syncthreads();
   }
-  // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above)
+  // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above): this thread's 16 columns are one
+  // half (cb % 2) of the 32 tokens of operand (row / 16, cb / 2); columns 4g..4g+3 of them are the lower (upper) 8 bytes
+  // of scan-lane group g.  Blocks above the diagonal are zero; operands (0,1), (1,1) are not stored at all.
   {
     const int row = tid >> 2, cb = tid & 3;
-    float x[16];
+    if (!((row >> 4) < 2 && cb >= 2)) {
+      float x[16];
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4) {
-      const f32x4 xv = cb <= (row >> 4) ? *reinterpret_cast<const f32x4*>(Xb + bidx(row >> 4, cb <= (row >> 4) ? cb : 0) * BLK + (row & 15) * BP + 4 * e4)
-                                        : (f32x4){0.f, 0.f, 0.f, 0.f};
-      const f32x4 bv = *reinterpret_cast<const f32x4*>(bet + 16 * cb + 4 * e4);
+      for (int e4 = 0; e4 < 4; ++e4) {
+        const f32x4 xv = cb <= (row >> 4) ? *reinterpret_cast<const f32x4*>(Xb + bidx(row >> 4, cb <= (row >> 4) ? cb : 0) * BLK + (row & 15) * BP + 4 * e4)
+                                          : (f32x4){0.f, 0.f, 0.f, 0.f};
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(bet + 16 * cb + 4 * e4);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[4 * e4 + e] = xv[e] * bv[e];
+        for (int e = 0; e < 4; ++e) x[4 * e4 + e] = xv[e] * bv[e];
+      }
+      bf16_t* trow = Tout + ((size_t)((2 * (row >> 4) + (cb >> 1)) * 64 + (row & 15))) * 8 + 4 * (cb & 1);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack_bf16x2(x[4 * g], x[4 * g + 1]);
+        w[1] = pack_bf16x2(x[4 * g + 2], x[4 * g + 3]);
+        *reinterpret_cast<u32x2*>(trow + g * 128) = w;
+      }
     }
-    u32x4 w0, w1;  // tokens {0..3, 8..11} and {4..7, 12..15} of this thread's 16
-    w0[0] = pack_bf16x2(x[0], x[1]);  w0[1] = pack_bf16x2(x[2], x[3]);   w0[2] = pack_bf16x2(x[8], x[9]);   w0[3] = pack_bf16x2(x[10], x[11]);
-    w1[0] = pack_bf16x2(x[4], x[5]);  w1[1] = pack_bf16x2(x[6], x[7]);   w1[2] = pack_bf16x2(x[12], x[13]); w1[3] = pack_bf16x2(x[14], x[15]);
-    bf16_t* trow = Tout + ((size_t)((2 * (row >> 4) + (cb >> 1)) * 64 + (row & 15))) * 8;
-    *reinterpret_cast<u32x4*>(trow + (cb & 1) * 128) = w0;
-    *reinterpret_cast<u32x4*>(trow + (2 + (cb & 1)) * 128) = w1;
   }
 }
 
 // =============================================================================================
 // scan
 // =============================================================================================
-NATSL_DEVICE u32x2 pack4(f32x4 v) {
-  u32x2 w;
-  w[0] = pack_bf16x2(v[0], v[1]);
-  w[1] = pack_bf16x2(v[2], v[3]);
-  return w;
+// 8 fp32 -> one bf16x8 operand: slots 0..3 from a, 4..7 from b
+NATSL_DEVICE bf16x8 pack8(const f32x4 a, const f32x4 b) {
+  u32x4 w;
+  w[0] = pack_bf16x2(a[0], a[1]);
+  w[1] = pack_bf16x2(a[2], a[3]);
+  w[2] = pack_bf16x2(b[0], b[1]);
+  w[3] = pack_bf16x2(b[2], b[3]);
+  return __builtin_bit_cast(bf16x8, w);
 }
 
-template <int DK, bool DELTA>
-__global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams p) {
-  constexpr int KS = DK / 32;   // MFMA k-steps over the key dimension
-  constexpr int MT = DK / 64;   // 16-row state tiles per wave
-  constexpr int KP = DK + 8;    // kbuf / ST row pitch (elements)
-  constexpr int VP = BV + 8;    // vbuf row pitch
-  constexpr int XP = C + 8;     // XT / VNT / VTT row pitch
-  __shared__ __align__(16) bf16_t kbuf[2][C * KP];
-  __shared__ __align__(16) bf16_t vbuf[2][C * VP];
-  __shared__ __align__(16) bf16_t ST[BV * KP];
-  __shared__ __align__(16) bf16_t XT[BV * XP];
-  __shared__ __align__(16) bf16_t VNT[BV * XP];
-  __shared__ __align__(16) bf16_t VTT[BV * XP];
-  __shared__ __align__(16) bf16_t Os[C * VP];  // output tile, row-major, for 16-byte stores
+// one DMA instruction: lane l copies 16 bytes from base + voff to LDS byte address lds + 16 l
+NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+}
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+// Swizzle of the k / q tiles in LDS (row-major, unpadded, rows of DK bf16): 16-byte segment s of row r sits at
+// s ^ kq_swizzle(r).  The A-operand read of a 16x16x32 instruction (16 lanes = 16 consecutive rows at one segment) and
+// the transposing read of k^T (16 lanes = 4 consecutive rows x 4 segments 0..3 of an aligned group) must both fall on
+// 16 different 16-byte slots of the 256-byte bank period.
+template <int DK>
+NATSL_DEVICE int kq_swizzle(const int r) {
+  if constexpr (DK == 128) return ((r & 3) << 2) | ((r >> 2) & 3);   // 16 segments per row, a row = one bank period
+  return (r >> 1) & 7;                                               // 8 or 24 segments per row: low three bits only
+}
+
+typedef __attribute__((address_space(3))) const bf16x8* lds_b128_t;
+typedef __attribute__((address_space(3))) const f32x4* lds_f4_t;
+typedef __attribute__((address_space(3))) const float* lds_f1_t;
+typedef __attribute__((address_space(3))) s16x4* lds_tr_t;
+typedef __attribute__((address_space(3))) bf16_t* lds_h_t;
+typedef __attribute__((address_space(3))) const u32x4* lds_u4_t;
+
+NATSL_DEVICE s16x4 lds_tr4_at(const unsigned addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr_t>(addr));
+}
+
+// LDS layout of the scan kernel: two stages (chunk c in stage c % 2) and two output tiles.
+template <int DK, int NW>
+struct ScanLds {
+  static constexpr int BVW = 16 * NW;                 // state columns of the workgroup
+  static constexpr int KROW = DK * 2;                 // bytes per k / q row
+  static constexpr int VROW = BVW * 2;                // bytes per v row
+  static constexpr int KB = 64 * KROW, VB = 64 * VROW, TB = 6 * 1024, PB = 6 * 1024, SCB = 1024;
+  static constexpr int OFF_K = 0, OFF_Q = OFF_K + KB, OFF_V = OFF_Q + KB, OFF_T = OFF_V + VB, OFF_P = OFF_T + TB, OFF_SC = OFF_P + PB;
+  static constexpr int STAGE = OFF_SC + SCB;
+  static constexpr int OROW = VROW + 16;              // output tile row pitch (bytes)
+  static constexpr int OB = 64 * OROW;
+  static constexpr int TOTAL = 2 * STAGE + 2 * OB;
+};
+
+// index of A operand (t, s) of TmB / P among the six that are stored (the two above the diagonal are skipped)
+NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t : 2 * t - 2 + s; }
+
+// Registers per wave: with DK <= 128 the kernel fits 256, so it asks for the two-waves-per-SIMD register budget even though
+// LDS admits one workgroup per CU: within that budget the matrix instructions take their accumulators in ordinary vector
+// registers and the state can be scaled and rounded in place (with the larger budget the compiler moves accumulators to the
+// second register file and every vector operation on the state costs two extra copies).
+#define NATSL_SCAN_FITS_256(DK) ((DK) <= 128)
+#define NATSL_SCAN_ATTR(DK, NW) \
+  __launch_bounds__(64 * (NW + 1)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
+
+// NW compute waves (16 state columns each) + one data-movement wave.
+template <int DK, bool DELTA, int NW>
+__global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p) {
+  using L = ScanLds<DK, NW>;
+  constexpr int KS = DK / 32;   // matrix k-steps over the key dimension
+  constexpr int KT = DK / 16;   // 16-row state tiles
+  extern __shared__ __align__(1024) unsigned char smem[];
+  const unsigned lds0 = (unsigned)(size_t)smem;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g4 = lane >> 4;
 
-  // ---- which (sequence, head, V slice): the slices of one chain sit on one XCD --------------
-  const int nsplit = p.V / BV;
+  // ---- which (sequence, head, column slice): the slices of one chain sit on one XCD --------------
+  const int nsplit = p.V / L::BVW;
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int split = slot % nsplit;
@@ -366,291 +421,369 @@ __global__ __launch_bounds__(256, 2) void linear_scan_kernel(const LinearParams 
     bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; chunk_off = p.seqs[n].chunk_off;
   }
   const int NT = (len + C - 1) / C;
+  const int vcol0 = split * L::BVW;           // first column of the workgroup
+  constexpr int VSEG = L::VROW / 16;          // 16-byte segments per v row (2, 4 or 8)
+  auto v_swz = [](const int r) { return VSEG == 8 ? 2 * ((r >> 1) & 1) : 0; };   // rows 2 apart share banks when a row is 128 bytes
+  // Output tile, TRANSPOSED in LDS: [column][64 tokens], rows of OT_ROW bytes: a compute lane writes the four tokens
+  // 16 t + 4 g4 .. of its column with one 8-byte store; the data-movement wave reads it back with the transposing read.
+  constexpr int OT_ROW = 2 * C + 16;
+  static_assert(L::BVW * OT_ROW <= L::OB, "the transposed output tile fits the space of the row-major one");
+
+  if (wave == NW) {
+    // ======================= the data-movement wave =============================================================
+    // Per step c: request chunk c + 1 into stage (c + 1) % 2 by LDS-DMA, store the output tile of chunk c - 1, wait for
+    // the requests, meet the barrier.  The compute waves never touch global memory inside the loop.
+    const size_t qk_pitch = (size_t)p.H * DK * 2, v_pitch = (size_t)p.H * p.V * 2;   // bytes per token
+    const char* kb = reinterpret_cast<const char*>(p.k + ((size_t)bos * p.H + h) * DK);
+    const ptrdiff_t q_minus_k = reinterpret_cast<const char*>(p.q) - reinterpret_cast<const char*>(p.k);
+    const char* vb = reinterpret_cast<const char*>(p.v + ((size_t)bos * p.H + h) * p.V + vcol0);
+    char* ob_g = reinterpret_cast<char*>(p.o + ((size_t)bos * p.H + h) * p.V + vcol0);
+    const size_t unit0 = (size_t)chunk_off * p.H + h;
+    const char* tb = reinterpret_cast<const char*>(p.ws_tm + unit0 * (C * C));
+    const ptrdiff_t p_minus_t = reinterpret_cast<const char*>(p.ws_p) - reinterpret_cast<const char*>(p.ws_tm);
+    const char* sb = reinterpret_cast<const char*>(p.ws_sc + unit0 * (4 * C));
+    const size_t ws_step = (size_t)p.H * (C * C) * 2, sc_step = (size_t)p.H * (4 * C) * 4;
+    const size_t qk_step = (size_t)C * qk_pitch, v_step = (size_t)C * v_pitch;
+
+    // k, q tiles: piece u covers LDS bytes [1024 u, 1024 u + 1024) of the tile; lane l fills byte 1024 u + 16 l, i.e. row
+    // (1024 u + 16 l) / KROW, position pos, with the source segment pos ^ swizzle(row).  v the same with its own geometry.
+    constexpr int KQ_PIECES = L::KB / 1024, V_PIECES = L::VB / 1024;
+    auto kq_src = [&](const int u, const int nvalid) -> unsigned {
+      const int byte = 1024 * u + 16 * lane, row = byte / L::KROW, pos = (byte % L::KROW) / 16;
+      return (unsigned)((size_t)min(row, nvalid - 1) * qk_pitch) + 16u * (unsigned)(pos ^ kq_swizzle<DK>(row));
+    };
+    auto v_src = [&](const int u, const int nvalid) -> unsigned {
+      const int byte = 1024 * u + 16 * lane, row = byte / L::VROW, pos = (byte % L::VROW) / 16;
+      return (unsigned)((size_t)min(row, nvalid - 1) * v_pitch) + 16u * (unsigned)(pos ^ v_swz(row));
+    };
+    unsigned kq_off[KQ_PIECES], v_off[V_PIECES];
+#pragma unroll
+    for (int u = 0; u < KQ_PIECES; ++u) kq_off[u] = kq_src(u, C);
+#pragma unroll
+    for (int u = 0; u < V_PIECES; ++u) v_off[u] = v_src(u, C);
+    // workspace pieces are plain copies: lane l moves bytes [16 l, 16 l + 16) of each; TmB / P keep operands 0, 2, 4..7 of 8
+    unsigned ws_off[6];
+#pragma unroll
+    for (int v = 0; v < 6; ++v) ws_off[v] = 16u * lane + 1024u * (v < 2 ? 2 * v : v + 2);
+
+    auto request = [&](const int cc) __attribute__((always_inline)) {
+      const unsigned st = lds0 + (cc & 1) * L::STAGE;
+      const int nvalid = min(C, len - cc * C);
+      if (nvalid < C) {
+        // the sequence's ragged last chunk (at most once per chain): rows past the end are clamped
+#pragma unroll
+        for (int u = 0; u < KQ_PIECES; ++u) kq_off[u] = kq_src(u, nvalid);
+#pragma unroll
+        for (int u = 0; u < V_PIECES; ++u) v_off[u] = v_src(u, nvalid);
+      }
+      const char* qb = kb + q_minus_k;
+      const char* pb = tb + p_minus_t;
+      // in the order the compute waves need them: sc, k (R = k S comes first), q, v, TmB, P
+      dma16(sb, 16u * lane, st + L::OFF_SC);
+#pragma unroll
+      for (int u = 0; u < KQ_PIECES; ++u) dma16(kb, kq_off[u], st + L::OFF_K + 1024 * u);
+#pragma unroll
+      for (int u = 0; u < KQ_PIECES; ++u) dma16(qb, kq_off[u], st + L::OFF_Q + 1024 * u);
+#pragma unroll
+      for (int u = 0; u < V_PIECES; ++u) dma16(vb, v_off[u], st + L::OFF_V + 1024 * u);
+      if (DELTA) {
+#pragma unroll
+        for (int v = 0; v < 6; ++v) dma16(tb, ws_off[v], st + L::OFF_T + 1024 * v);
+      }
+#pragma unroll
+      for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
+      kb += qk_step; vb += v_step; tb += ws_step; sb += sc_step;
+    };
+
+    // read-back of the output tile.  A 16-lane group covers 4 tokens x 16 or 32 columns: within it lane i'' names the four
+    // tokens of one column and lane i receives four adjacent columns of token tok0 + i % 4 -- with 32 columns per group,
+    // columns 8 (i / 4) .. + 3 from the first read and the next four from the second (one 16-byte store); with 16
+    // columns per group (one-wave workgroups) columns 4 (i / 4) .. + 3 (one 8-byte store).
+    constexpr bool WIDE = L::BVW >= 32;
+    constexpr int GCOLS = WIDE ? 32 : 16, O_GROUPS = 16 * (L::BVW / GCOLS), O_PASSES = O_GROUPS / 4;
+    unsigned o_lds[O_PASSES];
+    unsigned o_glb[O_PASSES];
+    int o_tok[O_PASSES];
+#pragma unroll
+    for (int j = 0; j < O_PASSES; ++j) {
+      const int grp = 4 * j + g4;
+      const int tok0 = 4 * (grp / (L::BVW / GCOLS)), cbase = GCOLS * (grp % (L::BVW / GCOLS));
+      const int c_first = WIDE ? cbase + 8 * (i16 & 3) + (i16 >> 2) : cbase + 4 * (i16 & 3) + (i16 >> 2);
+      o_lds[j] = (unsigned)(c_first * OT_ROW + 2 * tok0);
+      o_tok[j] = tok0 + (i16 & 3);
+      o_glb[j] = (unsigned)((size_t)o_tok[j] * v_pitch) + 2u * (unsigned)(cbase + (WIDE ? 8 : 4) * (i16 >> 2));
+    }
+    auto store_out = [&](const int cc) __attribute__((always_inline)) {
+      const unsigned ob = lds0 + 2 * L::STAGE + (cc & 1) * L::OB;
+      const int nvalid = len - cc * C;
+#pragma unroll
+      for (int j = 0; j < O_PASSES; ++j) {
+        if constexpr (WIDE) {
+          const s16x4 lo = lds_tr4_at(ob + o_lds[j]), hi = lds_tr4_at(ob + o_lds[j] + 4 * OT_ROW);
+          if (o_tok[j] < nvalid) *reinterpret_cast<bf16x8*>(ob_g + o_glb[j]) = join4(lo, hi);
+        } else {
+          const s16x4 w = lds_tr4_at(ob + o_lds[j]);
+          if (o_tok[j] < nvalid) *reinterpret_cast<s16x4*>(ob_g + o_glb[j]) = w;
+        }
+      }
+      ob_g += v_step;
+    };
+
+    if (NT > 0) request(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    for (int c = 0; c < NT; ++c) {
+      if (c + 1 < NT) request(c + 1);   // into the stage that step c - 1 read: every wave is past the barrier that ended it
+      if (c > 0) store_out(c - 1);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+    }
+    if (NT > 0) store_out(NT - 1);
+    return;
+  }
+
+  // ======================= compute waves ===========================================================================
   const int per_blk = p.block / C;
   const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0;
   const bool intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
-  const int vcol0 = split * BV;
+  const int col = vcol0 + 16 * wave + i16;    // this lane's state column
 
-  const size_t qk_row = (size_t)p.H * DK, v_row = (size_t)p.H * p.V;
-  const bf16_t* qp = p.q + ((size_t)bos * p.H + h) * DK;
-  const bf16_t* kp = p.k + ((size_t)bos * p.H + h) * DK;
-  const bf16_t* vp = p.v + ((size_t)bos * p.H + h) * p.V + vcol0;
-  bf16_t* op = p.o + ((size_t)bos * p.H + h) * p.V + vcol0;
-
-  // ---- state slice in accumulator layout: tile (mi, nn) = rows 16(wave*MT+mi).., cols 16nn.. ---
-  f32x4 S[MT][2], Ssave[MT][2];
+  // ---- state: tile m, lane group g4, register r holds K row krow_of(m, r), column `col` -----------------
+  // (two tiles 2s, 2s+1 side by side are the eight contraction slots of k-step s: rows 32s + 8 g4 + 0..7, which is what a
+  // 16-byte read of a k or q row delivers)
+  auto krow_of = [&](const int m, const int r) { return 32 * (m >> 1) + 8 * g4 + 4 * (m & 1) + r; };
+  f32x4 S[KT], Ssave[KT];
 #pragma unroll
-  for (int mi = 0; mi < MT; ++mi)
+  for (int m = 0; m < KT; ++m)
 #pragma unroll
-    for (int nn = 0; nn < 2; ++nn)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
-        S[mi][nn][r] = p.h0 ? p.h0[((size_t)chain * DK + kd) * p.V + vc] : 0.f;
-        Ssave[mi][nn][r] = 0.f;
-      }
-  auto write_ST = [&]() {
-#pragma unroll
-    for (int mi = 0; mi < MT; ++mi)
-#pragma unroll
-      for (int nn = 0; nn < 2; ++nn)
-        *reinterpret_cast<u32x2*>(ST + (16 * nn + i16) * KP + 16 * (wave * MT + mi) + 4 * g4) = pack4(S[mi][nn]);
-  };
-
-  // ---- operand staging ------------------------------------------------------------------------
-  // Two register sets hold the MFMA A operands (q, TmB, P) and the per-token scales of chunks c and
-  // c+1.  Each piece of the set in use is reloaded with chunk c+2's data right after its last use,
-  // so every one of these loads has two steps to arrive.  k and v go through LDS (double-buffered):
-  // they are loaded at the start of step c for chunk c+1 and stored at its end.
-  struct Operands {
-    bf16x8 qA[KS], TA[2], PA[2];
-    f32x4 se, sq, sk;
-    float dec, glast, linf;
-  };
-  struct Staging {
-    u32x4 kld[KS], vld;  // row-contiguous k and v pieces on their way to LDS
-  };
-  const int a_row = 16 * wave + i16;          // this lane's A-operand row (token within the chunk)
-  const int v_ld_row = tid >> 2, v_ld_seg = tid & 3;
-  const int r0 = 16 * wave + 4 * g4;          // first of this lane's four accumulator rows
-  // where those four tokens sit in the contraction order P and TmB were stored in
-  const int perm0 = 32 * (wave >> 1) + 8 * (2 * (g4 & 1) + (wave & 1)) + 4 * (g4 >> 1);
-  // k staging: one pass of the 256 threads covers KROWS token rows of DK*2 bytes
-  constexpr int KSEGS = DK / 8, KROWS = 256 / KSEGS;
-  const int k_ld_row = tid / KSEGS, k_ld_seg = tid % KSEGS;
-  // rows past the end of the sequence are clamped (beta = 0 there makes their v_new exactly 0, and
-  // their outputs are never stored)
-  const bf16_t* k_ptr = kp + 8 * k_ld_seg;
-  const bf16_t* q_ptr = qp + 8 * g4;
-  const bf16_t* v_ptr = vp + 8 * v_ld_seg;
-  const size_t unit0 = (size_t)chunk_off * p.H + h;
-  const size_t unit_step = (size_t)p.H * (C * C), sc_step = (size_t)p.H * (4 * C);
-  // P and TmB come in A-operand order: 16 contiguous bytes per lane, 1 KiB per wave and k-step
-  const bf16_t* P_base = p.ws_p + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
-  const bf16_t* T_base = p.ws_tm + unit0 * (C * C) + (2 * wave * 64 + lane) * 8;
-  const float* sc_base = p.ws_sc + unit0 * (4 * C);
-  // the pieces of an operand set, each loadable on its own (cc = chunk index, must be < NT)
-  auto load_q = [&](Operands& A, int cc) {
-    const bf16_t* qr = q_ptr + (size_t)min(cc * C + a_row, len - 1) * qk_row;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) A.qA[s] = ld8(qr + 32 * s);
-  };
-  auto load_T = [&](Operands& A, int cc) {
-    A.TA[0] = ld8(T_base + cc * unit_step);
-    A.TA[1] = ld8(T_base + cc * unit_step + 512);
-  };
-  auto load_P = [&](Operands& A, int cc) {
-    A.PA[0] = ld8(P_base + cc * unit_step);
-    A.PA[1] = ld8(P_base + cc * unit_step + 512);
-  };
-  auto load_se = [&](Operands& A, int cc) { A.se = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + r0); };
-  auto load_sq = [&](Operands& A, int cc) { A.sq = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + C + r0); };
-  auto load_sk = [&](Operands& A, int cc) { A.sk = *reinterpret_cast<const f32x4*>(sc_base + cc * sc_step + 2 * C + r0); };
-  auto load_scalars = [&](Operands& A, int cc) {
-    const float* sp = sc_base + cc * sc_step + 3 * C;
-    A.dec = sp[0];
-    A.glast = sp[1];
-    A.linf = sp[2];
-  };
-  auto load_all = [&](Operands& A, int cc) {
-    load_q(A, cc);
-    if (DELTA) load_se(A, cc);
-    if (DELTA) load_T(A, cc);
-    load_sk(A, cc);
-    load_P(A, cc);
-    load_sq(A, cc);
-    load_scalars(A, cc);
-  };
-  auto gload_kv = [&](Staging& G, int cc) {
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int kt = min(cc * C + k_ld_row + KROWS * s, len - 1);
-      G.kld[s] = *reinterpret_cast<const u32x4*>(k_ptr + (size_t)kt * qk_row);
+    for (int r = 0; r < 4; ++r) {
+      S[m][r] = p.h0 ? p.h0[((size_t)chain * DK + krow_of(m, r)) * p.V + col] : 0.f;
+      Ssave[m][r] = 0.f;
     }
-    const int vt = cc * C + v_ld_row;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    G.vld = vt < len ? *reinterpret_cast<const u32x4*>(v_ptr + (size_t)vt * v_row) : z;  // v must be 0 past the end
-  };
-  auto lstore = [&](const Staging& G, int buf) {
+
+  // ---- per-lane operand addresses inside a stage ------------------------------------------------------------------
+  // k / q as A operand (token tile t, k-step s): row 16 t + i16, segment 4 s + g4 (swizzled); t goes into the offset field
+  unsigned a_kq[KS];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) *reinterpret_cast<u32x4*>(&kbuf[buf][(k_ld_row + KROWS * s) * KP + 8 * k_ld_seg]) = G.kld[s];
-    *reinterpret_cast<u32x4*>(&vbuf[buf][v_ld_row * VP + 8 * v_ld_seg]) = G.vld;
-  };
+  for (int s = 0; s < KS; ++s) a_kq[s] = (unsigned)(i16 * L::KROW) + 16u * (unsigned)((4 * s + g4) ^ kq_swizzle<DK>(i16));
+  // k^T as A operand (state tile m, token k-step s2, read rd): lane i16 addresses token 32 s2 + 16 rd + 4 g4 + i16 / 4,
+  // the four K rows 32 (m / 2) + 8 (i16 % 4) + 4 (m % 2) ..: segment 4 (m / 2) + i16 % 4, half m % 2
+  unsigned a_kt[KT / 2];
+  {
+    const int tok = 4 * g4 + (i16 >> 2);
+#pragma unroll
+    for (int mh = 0; mh < KT / 2; ++mh)
+      a_kt[mh] = (unsigned)(tok * L::KROW) + 16u * (unsigned)((4 * mh + (i16 & 3)) ^ kq_swizzle<DK>(tok));
+  }
+  // v through the transposing read (token tile t): lane i16 addresses token 16 t + 4 g4 + i16 / 4, columns 16 wave + 4 (i16 % 4)..
+  unsigned a_v;
+  {
+    const int tok = 4 * g4 + (i16 >> 2), seg = 2 * wave + ((i16 & 3) >> 1);
+    a_v = (unsigned)(tok * L::VROW) + 16u * (unsigned)(seg ^ v_swz(tok)) + 8u * (i16 & 1);
+  }
+  const unsigned a_o = (unsigned)((16 * wave + i16) * OT_ROW + 8 * g4);
+  const unsigned a_sc = 16u * g4;    // this lane group's four tokens in a row of sc
 
   float gsum = 0.f;
-  // one chunk: CUR holds its operands, kbuf/vbuf[buf] its k and v tiles
-  Staging G;
-  auto step = [&](const int c, const int buf, Operands& CUR) {
-    __syncthreads();  // ST, kbuf[buf], vbuf[buf] are in place
-    // Loads are issued unconditionally (chunk indices clamped to the last chunk): a load inside a
-    // branch would force the waits below to assume it may not have been issued, i.e. to drain the queue.
-    const int c1 = min(c + 1, NT - 1), c2 = min(c + 2, NT - 1);
-    const float dec_c = CUR.dec, glast_c = CUR.glast, linf_c = CUR.linf;
-    load_scalars(CUR, c2);  // first, so that nothing younger has to be waited for along with them
-    gload_kv(G, c1);
+  __syncthreads();   // chunk 0 has landed
 
+  for (int c = 0; c < NT; ++c) {
+    const unsigned st = lds0 + (c & 1) * L::STAGE;
+    // the chunk's scalars (three separate 4-byte reads on purpose: read as one 16-byte vector whose lanes all name the
+    // same address, the compiler folded the three elements into the first)
+    const float dec_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C));
+    const float glast_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C + 1));
+    const float linf_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C + 2));
     if (c % per_blk == 0) {
 #pragma unroll
-      for (int mi = 0; mi < MT; ++mi)
-#pragma unroll
-        for (int nn = 0; nn < 2; ++nn) Ssave[mi][nn] = S[mi][nn];
+      for (int m = 0; m < KT; ++m) Ssave[m] = S[m];
       gsum = 0.f;
     }
-
-    // (1) R = k S, O1 = q S
-    f32x4 R[2], O1[2];
+    // (1) the state as B operands
+    bf16x8 SB[KS];
 #pragma unroll
-    for (int nn = 0; nn < 2; ++nn) { R[nn] = (f32x4){0.f, 0.f, 0.f, 0.f}; O1[nn] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const bf16x8 sb0 = ld8(ST + i16 * KP + 32 * s + 8 * g4);
-      const bf16x8 sb1 = ld8(ST + (16 + i16) * KP + 32 * s + 8 * g4);
-      if (DELTA) {
-        const bf16x8 ka = ld8(&kbuf[buf][a_row * KP + 32 * s + 8 * g4]);
-        R[0] = mfma16(ka, sb0, R[0]);
-        R[1] = mfma16(ka, sb1, R[1]);
-      }
-      O1[0] = mfma16(CUR.qA[s], sb0, O1[0]);
-      O1[1] = mfma16(CUR.qA[s], sb1, O1[1]);
-    }
-    load_q(CUR, c2);
-    // (2) v in accumulator layout via the transposing read; X = v - se * R
-    f32x4 VN[2];
-#pragma unroll
-    for (int nn = 0; nn < 2; ++nn) {
-      const s16x4 vv = lds_tr4(&vbuf[buf][(16 * wave + 4 * g4 + (i16 >> 2)) * VP + 16 * nn + 4 * (i16 & 3)]);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) VN[nn][r] = bf16_to_f32((bf16_t)vv[r]);
-    }
-    if (DELTA) {
-#pragma unroll
-      for (int nn = 0; nn < 2; ++nn) {
-        f32x4 X;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) X[r] = VN[nn][r] - CUR.se[r] * R[nn][r];
-        *reinterpret_cast<u32x2*>(XT + (16 * nn + i16) * XP + perm0) = pack4(X);
-      }
-      load_se(CUR, c2);
-      __syncthreads();
-      // (3) v_new = TmB X
-#pragma unroll
-      for (int nn = 0; nn < 2; ++nn) {
-        VN[nn] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 2; ++s) VN[nn] = mfma16(CUR.TA[s], ld8(XT + (16 * nn + i16) * XP + 32 * s + 8 * g4), VN[nn]);
-      }
-      load_T(CUR, c2);
-    }
-    // (4) v_new and sk * v_new, transposed, for the two products that reduce over tokens
-#pragma unroll
-    for (int nn = 0; nn < 2; ++nn) {
-      f32x4 vt;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) vt[r] = VN[nn][r] * CUR.sk[r];
-      *reinterpret_cast<u32x2*>(VNT + (16 * nn + i16) * XP + perm0) = pack4(VN[nn]);
-      *reinterpret_cast<u32x2*>(VTT + (16 * nn + i16) * XP + 16 * wave + 4 * g4) = pack4(vt);
-    }
-    load_sk(CUR, c2);
-    __syncthreads();
-    // (5) o = sq * O1 + P v_new
-#pragma unroll
-    for (int nn = 0; nn < 2; ++nn) {
-      f32x4 O;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) O[r] = O1[nn][r] * CUR.sq[r];
-      if (intra) {
-#pragma unroll
-        for (int s = 0; s < 2; ++s) O = mfma16(CUR.PA[s], ld8(VNT + (16 * nn + i16) * XP + 32 * s + 8 * g4), O);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) Os[(r0 + r) * VP + 16 * nn + i16] = f32_to_bf16(O[r]);
-    }
-    load_P(CUR, c2);
-    load_sq(CUR, c2);
-    {
-      // each wave stores the 16 rows it owns: 4 lanes x 16 bytes per row
-      __builtin_amdgcn_s_waitcnt(0xc07f);
-      __builtin_amdgcn_wave_barrier();
-      const int row = 16 * wave + (lane >> 2), tok = c * C + row;
-      if (tok < len)
-        *reinterpret_cast<u32x4*>(op + (size_t)tok * v_row + 8 * (lane & 3)) = *reinterpret_cast<const u32x4*>(Os + row * VP + 8 * (lane & 3));
-    }
-    // (6) state update / roll-back
+    for (int s = 0; s < KS; ++s) SB[s] = pack8(S[2 * s], S[2 * s + 1]);
+    const float dec_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, dec_v)));
+    const float glast_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, glast_v)));
+    const float linf_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, linf_v)));
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
-    gsum += glast_c;
     const bool keep = linf_c != 0.f || !last_of_block;
+    gsum += glast_c;
+
+    // R = k S, then O1 = q S (X below only needs R); operands are read AHEAD instructions before their use
+    f32x4 R[4], O1[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) { R[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; O1[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+    {
+      constexpr int NOP = (DELTA ? 2 : 1) * 4 * KS, AHEAD = 4;
+      auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+        const int which = DELTA ? j / (4 * KS) : 1, jj = j % (4 * KS), s = jj / 4, t = jj % 4;
+        return *reinterpret_cast<lds_b128_t>(st + (which ? L::OFF_Q : L::OFF_K) + a_kq[s] + t * 16 * L::KROW);
+      };
+      bf16x8 opnd[NOP + AHEAD];
+#pragma unroll
+      for (int j = 0; j < AHEAD; ++j) opnd[j] = ld_op(j);
+#pragma unroll
+      for (int j = 0; j < NOP; ++j) {
+        if (j + AHEAD < NOP) opnd[j + AHEAD] = ld_op(j + AHEAD);
+        const int which = DELTA ? j / (4 * KS) : 1, jj = j % (4 * KS), s = jj / 4, t = jj % 4;
+        if (which) O1[t] = mfma16(opnd[j], SB[s], O1[t]);
+        else R[t] = mfma16(opnd[j], SB[s], R[t]);
+      }
+    }
+    // the state's decay for the update at the end of the step (in the shadow of the matrix instructions above)
     if (keep) {
 #pragma unroll
-      for (int mi = 0; mi < MT; ++mi) {
-        const int m = wave * MT + mi;
-        bf16x8 kt[2];
+      for (int m = 0; m < KT; ++m)
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const bf16_t* kb = &kbuf[buf][(32 * s + 8 * g4 + (i16 >> 2)) * KP + 16 * m + 4 * (i16 & 3)];
-          kt[s] = join4(lds_tr4(kb), lds_tr4(kb + 4 * KP));
-        }
+        for (int r = 0; r < 4; ++r) S[m][r] *= dec_c;
+    }
+    // (2) v in accumulator layout (lane = column, registers = tokens 16 t + 4 g4 + r); zero past the end of the sequence
+    f32x4 VN[4];
+    const int nvalid = len - c * C;
 #pragma unroll
-        for (int nn = 0; nn < 2; ++nn) {
+    for (int t = 0; t < 4; ++t) {
+      const s16x4 vv = lds_tr4_at(st + L::OFF_V + a_v + t * 16 * L::VROW);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) S[mi][nn][r] *= dec_c;
+      for (int r = 0; r < 4; ++r) VN[t][r] = bf16_to_f32((bf16_t)vv[r]);
+    }
+    if (__builtin_expect(nvalid < C, 0)) {
+      asm volatile("" ::: "memory");   // (keeps this a branch: it runs once per chain)
 #pragma unroll
-          for (int s = 0; s < 2; ++s) S[mi][nn] = mfma16(kt[s], ld8(VTT + (16 * nn + i16) * XP + 32 * s + 8 * g4), S[mi][nn]);
-        }
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (16 * t + 4 * g4 + r >= nvalid) VN[t][r] = 0.f;
+    }
+    if (DELTA) {
+      // X = v - se * R;  v_new = TmB X
+      f32x4 se[4];
+      bf16x8 TA[6];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) se[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + a_sc + 64 * t);
+#pragma unroll
+      for (int v = 0; v < 6; ++v) TA[v] = *reinterpret_cast<lds_b128_t>(st + L::OFF_T + 1024 * v + 16 * lane);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) VN[t][r] -= se[t][r] * R[t][r];
+      const bf16x8 XB[2] = {pack8(VN[0], VN[1]), pack8(VN[2], VN[3])};
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+      VN[0] = mfma16(TA[tri_slot(0, 0)], XB[0], zero);
+      VN[1] = mfma16(TA[tri_slot(1, 0)], XB[0], zero);
+      VN[2] = mfma16(TA[tri_slot(2, 0)], XB[0], zero);
+      VN[3] = mfma16(TA[tri_slot(3, 0)], XB[0], zero);
+      VN[2] = mfma16(TA[tri_slot(2, 1)], XB[1], VN[2]);
+      VN[3] = mfma16(TA[tri_slot(3, 1)], XB[1], VN[3]);
+    }
+    // (3) state update / roll-back (the next step waits for it: before the output)
+    const bf16x8 VB[2] = {pack8(VN[0], VN[1]), pack8(VN[2], VN[3])};
+    if (keep) {
+      f32x4 W[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const f32x4 sk = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * (2 * C) + a_sc + 64 * t);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) W[t][r] = VN[t][r] * sk[r];
+      }
+      const bf16x8 WB[2] = {pack8(W[0], W[1]), pack8(W[2], W[3])};
+      constexpr int NOP = 2 * KT, AHEAD = 4;
+      auto ld_kt = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
+        const int s = j / KT, m = j % KT;
+        const unsigned a = st + L::OFF_K + a_kt[m >> 1] + 8u * (m & 1) + (32 * s) * L::KROW;
+        return join4(lds_tr4_at(a), lds_tr4_at(a + 16 * L::KROW));
+      };
+      bf16x8 opnd[NOP + AHEAD];
+#pragma unroll
+      for (int j = 0; j < AHEAD; ++j) opnd[j] = ld_kt(j);
+#pragma unroll
+      for (int j = 0; j < NOP; ++j) {
+        if (j + AHEAD < NOP) opnd[j + AHEAD] = ld_kt(j + AHEAD);
+        S[j % KT] = mfma16(opnd[j], WB[j / KT], S[j % KT]);
       }
     } else {
       const float f = decay ? __expf(gsum) : 1.f;
 #pragma unroll
-      for (int mi = 0; mi < MT; ++mi)
+      for (int m = 0; m < KT; ++m)
 #pragma unroll
-        for (int nn = 0; nn < 2; ++nn)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) S[mi][nn][r] = Ssave[mi][nn][r] * f;
+        for (int r = 0; r < 4; ++r) S[m][r] = Ssave[m][r] * f;
     }
-    // (7) bf16 copy of the state and the staged k, v tiles for the next step
-    write_ST();
-    lstore(G, buf ^ 1);
-  };
-
-  Operands A0, A1;
-  if (NT > 0) {
-    gload_kv(G, 0);
-    load_all(A0, 0);
-    if (NT > 1) load_all(A1, 1);
-    lstore(G, 0);
-  }
-  write_ST();
-  for (int c = 0; c < NT; c += 2) {
-    step(c, 0, A0);
-    if (c + 1 < NT) step(c + 1, 1, A1);
+    // (4) o = sq * O1 + P v_new, into the (transposed) output tile: the four token tiles side by side
+    {
+      const unsigned ob = lds0 + 2 * L::STAGE + (c & 1) * L::OB;
+      f32x4 O[4];
+      bf16x8 PA[6];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) O[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * C + a_sc + 64 * t);
+      if (intra) {
+#pragma unroll
+        for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>(st + L::OFF_P + 1024 * v + 16 * lane);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) O[t][r] *= O1[t][r];
+      if (intra) {
+        O[0] = mfma16(PA[tri_slot(0, 0)], VB[0], O[0]);
+        O[1] = mfma16(PA[tri_slot(1, 0)], VB[0], O[1]);
+        O[2] = mfma16(PA[tri_slot(2, 0)], VB[0], O[2]);
+        O[3] = mfma16(PA[tri_slot(3, 0)], VB[0], O[3]);
+        O[2] = mfma16(PA[tri_slot(2, 1)], VB[1], O[2]);
+        O[3] = mfma16(PA[tri_slot(3, 1)], VB[1], O[3]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        u32x2 w;
+        w[0] = pack_bf16x2(O[t][0], O[t][1]);
+        w[1] = pack_bf16x2(O[t][2], O[t][3]);
+        *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(ob + a_o + 32 * t) = w;
+      }
+    }
+    // every wave is done with this stage and has written its part of the output tile; the data-movement wave has
+    // waited for the next chunk's inputs
+    __syncthreads();
   }
 
   if (p.hs) {
     // Ssave / gsum still belong to the last block: the state that entered it and its total log-decay
 #pragma unroll
-    for (int mi = 0; mi < MT; ++mi)
+    for (int m = 0; m < KT; ++m)
 #pragma unroll
-      for (int nn = 0; nn < 2; ++nn)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
-          p.hs[((size_t)chain * DK + kd) * p.V + vc] = Ssave[mi][nn][r];
-        }
+      for (int r = 0; r < 4; ++r) p.hs[((size_t)chain * DK + krow_of(m, r)) * p.V + col] = Ssave[m][r];
     if (p.gs && split == 0 && tid == 0) p.gs[chain] = gsum;
   }
   if (p.ht) {
 #pragma unroll
-    for (int mi = 0; mi < MT; ++mi)
+    for (int m = 0; m < KT; ++m)
 #pragma unroll
-      for (int nn = 0; nn < 2; ++nn)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int kd = 16 * (wave * MT + mi) + 4 * g4 + r, vc = vcol0 + 16 * nn + i16;
-          p.ht[((size_t)chain * DK + kd) * p.V + vc] = S[mi][nn][r];
-        }
+      for (int r = 0; r < 4; ++r) p.ht[((size_t)chain * DK + krow_of(m, r)) * p.V + col] = S[m][r];
   }
 }
 
 constexpr size_t WS_UNIT_BYTES = (size_t)C * C * 2 * 2 + 4 * C * 4;
+
+inline int cu_count_linear() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
+template <int DK, bool DELTA, int NW>
+static int launch_scan(const LinearParams& p, hipStream_t stream, const char* what) {
+  using L = ScanLds<DK, NW>;
+  auto kern = linear_scan_kernel<DK, DELTA, NW>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
+  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
+  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+  const int grid = 8 * cdiv(n_chains, 8) * (p.V / L::BVW);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (NW + 1)), L::TOTAL, stream, p);
+  return check_launch(what);
+}
 
 template <int DK, bool DELTA>
 static int launch_linear(const LinearParams& p, hipStream_t stream, const char* what) {
@@ -659,10 +792,14 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
   hipLaunchKernelGGL((linear_prep_kernel<DK, DELTA>), dim3((unsigned)units), dim3(256), 0, stream, p);
   int rc = check_launch(what);
   if (rc != NATSL_OK) return rc;
-  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
-  const int grid = 8 * cdiv(n_chains, 8) * (p.V / BV);
-  hipLaunchKernelGGL((linear_scan_kernel<DK, DELTA>), dim3(grid), dim3(256), 0, stream, p);
-  return check_launch(what);
+  // Waves per workgroup (16 state columns each): the widest workgroup that still gives every CU one, so that the
+  // chunk's inputs are staged once for as many columns as possible without leaving CUs idle.
+  const long long n_chains = (long long)(p.seqs ? p.n_seqs : p.B) * p.H;
+  const int cus = cu_count_linear();
+  // (K = 192: five waves of that size do not fit the registers of a CU without spilling; three do)
+  if (DK <= 128 && p.V % 64 == 0 && n_chains * (p.V / 64) >= cus) return launch_scan<DK <= 128 ? DK : 128, DELTA, 4>(p, stream, what);
+  if (p.V % 32 == 0 && n_chains * (p.V / 32) >= cus) return launch_scan<DK, DELTA, 2>(p, stream, what);
+  return launch_scan<DK, DELTA, 1>(p, stream, what);
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
@@ -676,7 +813,7 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
   if (B <= 0 || T <= 0 || H <= 0 || HN <= 0 || TN <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
   if (H % HN) return fail(NATSL_ERR_INVALID, "%s: H=%d must be a multiple of HN=%d", what, H, HN);
   if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
-  if (V % BV || V <= 0) return fail(NATSL_ERR_UNSUPPORTED, "%s: V=%d must be a multiple of %d", what, V, BV);
+  if (V % 16 || V <= 0) return fail(NATSL_ERR_UNSUPPORTED, "%s: V=%d must be a multiple of 16", what, V);
   if (seqs ? (B != 1 || n_seqs <= 0 || total_units <= 0) : (TN != cdiv(T, block)))
     return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   LinearParams p;
@@ -698,11 +835,13 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
   if (delta) {
     if (K == 128) return launch_linear<128, true>(p, s, what);
     if (K == 64) return launch_linear<64, true>(p, s, what);
+    if (K == 192) return launch_linear<192, true>(p, s, what);
   } else {
     if (K == 128) return launch_linear<128, false>(p, s, what);
     if (K == 64) return launch_linear<64, false>(p, s, what);
+    if (K == 192) return launch_linear<192, false>(p, s, what);
   }
-  return fail(NATSL_ERR_UNSUPPORTED, "%s: key dim K=%d not built (supported: 64, 128)", what, K);
+  return fail(NATSL_ERR_UNSUPPORTED, "%s: key dim K=%d not built (supported: 64, 128, 192)", what, K);
 }
 
 }  // namespace natsl
