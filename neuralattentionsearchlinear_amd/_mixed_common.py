@@ -19,18 +19,18 @@ TIMING_HOOK = None
 # Where the softmax branch is launched.  True: on a side stream next to the linear branch (as the
 # reference's Mamba operator does); False: on the caller's stream, one branch after the other (as the
 # reference's GDN operator does); None: decide per call - side by side only when the linear branch's scan
-# has too few workgroups to fill the GPU on its own.  Both kernels are sized to occupy whole CUs, so when
-# each fills the machine alone, running them side by side gains nothing (measured) and only blurs timings.
+# cannot give every CU a workgroup even at its narrowest (one compute wave = 16 state columns per workgroup).
+# Both kernels take most of a CU's LDS (127 KiB / 159 KiB), so they never share a CU: when each fills the
+# machine alone, running them side by side gains nothing (measured) and only blurs timings.
 CONCURRENT_BRANCHES = None
-_SCAN_V_SLICE = 32          # value columns per scan workgroup (BV in csrc/natsl_linear.hip)
-_SCAN_WGS_PER_CU = 2        # scan workgroups resident per CU
+_SCAN_COLUMNS_PER_WG = 16   # state columns of the scan's narrowest workgroup (csrc/natsl_linear.hip)
 
 
 def _run_side_by_side(dev, n_chains: int, V: int) -> bool:
     if CONCURRENT_BRANCHES is not None:
         return bool(CONCURRENT_BRANCHES)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    return n_chains * (V // _SCAN_V_SLICE) < _SCAN_WGS_PER_CU * cus
+    return n_chains * (V // _SCAN_COLUMNS_PER_WG) < cus
 
 
 def _mark(name, stream):

@@ -368,7 +368,7 @@ NATSL_DEVICE s16x4 lds_tr4_at(const unsigned addr) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr_t>(addr));
 }
 
-// LDS layout of the scan kernel: two stages (chunk c in stage c % 2) and two output tiles.
+// LDS layout of the scan kernel: two or three stages and two output tiles.
 template <int DK, int NW>
 struct ScanLds {
   static constexpr int BVW = 16 * NW;                 // state columns of the workgroup
@@ -379,7 +379,10 @@ struct ScanLds {
   static constexpr int STAGE = OFF_SC + SCB;
   static constexpr int OROW = VROW + 16;              // output tile row pitch (bytes)
   static constexpr int OB = 64 * OROW;
-  static constexpr int TOTAL = 2 * STAGE + 2 * OB;
+  // Stages: chunk c lives in stage c % NSTAGE.  Three when they fit (narrow workgroups): the requests of chunk c + 2
+  // are issued in step c and have a whole step more to land; two otherwise (requests of chunk c + 1 in step c).
+  static constexpr int NSTAGE = 3 * STAGE + 2 * OB <= 160 * 1024 ? 3 : 2;
+  static constexpr int TOTAL = NSTAGE * STAGE + 2 * OB;
 };
 
 // index of A operand (t, s) of TmB / P among the six that are stored (the two above the diagonal are skipped)
@@ -391,9 +394,9 @@ NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t
 // second register file and every vector operation on the state costs two extra copies).
 #define NATSL_SCAN_FITS_256(DK) ((DK) <= 128)
 #define NATSL_SCAN_ATTR(DK, NW) \
-  __launch_bounds__(64 * (NW + 1)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
+  __launch_bounds__(64 * (NW + 2)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
 
-// NW compute waves (16 state columns each) + one data-movement wave.
+// NW compute waves (16 state columns each) + two data-movement waves.
 template <int DK, bool DELTA, int NW>
 __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p) {
   using L = ScanLds<DK, NW>;
@@ -429,10 +432,12 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
   constexpr int OT_ROW = 2 * C + 16;
   static_assert(L::BVW * OT_ROW <= L::OB, "the transposed output tile fits the space of the row-major one");
 
-  if (wave == NW) {
-    // ======================= the data-movement wave =============================================================
-    // Per step c: request chunk c + 1 into stage (c + 1) % 2 by LDS-DMA, store the output tile of chunk c - 1, wait for
-    // the requests, meet the barrier.  The compute waves never touch global memory inside the loop.
+  if (wave >= NW) {
+    // ======================= the two data-movement waves ========================================================
+    // Per step c: request chunk c + 1 into stage (c + 1) % 2 by LDS-DMA (wave NW: sc, k, q; wave NW + 1: v, TmB, P),
+    // store the output tile of chunk c - 1 (wave NW + 1), wait for the requests, meet the barrier.  The compute waves
+    // never touch global memory inside the loop.  (One wave issues about 1 KiB per 36 cycles; two share the 53 KiB.)
+    const bool first = wave == NW;
     const size_t qk_pitch = (size_t)p.H * DK * 2, v_pitch = (size_t)p.H * p.V * 2;   // bytes per token
     const char* kb = reinterpret_cast<const char*>(p.k + ((size_t)bos * p.H + h) * DK);
     const ptrdiff_t q_minus_k = reinterpret_cast<const char*>(p.q) - reinterpret_cast<const char*>(p.k);
@@ -467,7 +472,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     for (int v = 0; v < 6; ++v) ws_off[v] = 16u * lane + 1024u * (v < 2 ? 2 * v : v + 2);
 
     auto request = [&](const int cc) __attribute__((always_inline)) {
-      const unsigned st = lds0 + (cc & 1) * L::STAGE;
+      const unsigned st = lds0 + (cc % L::NSTAGE) * L::STAGE;
       const int nvalid = min(C, len - cc * C);
       if (nvalid < C) {
         // the sequence's ragged last chunk (at most once per chain): rows past the end are clamped
@@ -478,20 +483,23 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       }
       const char* qb = kb + q_minus_k;
       const char* pb = tb + p_minus_t;
-      // in the order the compute waves need them: sc, k (R = k S comes first), q, v, TmB, P
-      dma16(sb, 16u * lane, st + L::OFF_SC);
+      if (first) {
+        // in the order the compute waves need them: sc, k (R = k S comes first), q
+        dma16(sb, 16u * lane, st + L::OFF_SC);
 #pragma unroll
-      for (int u = 0; u < KQ_PIECES; ++u) dma16(kb, kq_off[u], st + L::OFF_K + 1024 * u);
+        for (int u = 0; u < KQ_PIECES; ++u) dma16(kb, kq_off[u], st + L::OFF_K + 1024 * u);
 #pragma unroll
-      for (int u = 0; u < KQ_PIECES; ++u) dma16(qb, kq_off[u], st + L::OFF_Q + 1024 * u);
+        for (int u = 0; u < KQ_PIECES; ++u) dma16(qb, kq_off[u], st + L::OFF_Q + 1024 * u);
+      } else {
 #pragma unroll
-      for (int u = 0; u < V_PIECES; ++u) dma16(vb, v_off[u], st + L::OFF_V + 1024 * u);
-      if (DELTA) {
+        for (int u = 0; u < V_PIECES; ++u) dma16(vb, v_off[u], st + L::OFF_V + 1024 * u);
+        if (DELTA) {
 #pragma unroll
-        for (int v = 0; v < 6; ++v) dma16(tb, ws_off[v], st + L::OFF_T + 1024 * v);
+          for (int v = 0; v < 6; ++v) dma16(tb, ws_off[v], st + L::OFF_T + 1024 * v);
+        }
+#pragma unroll
+        for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
       }
-#pragma unroll
-      for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
       kb += qk_step; vb += v_step; tb += ws_step; sb += sc_step;
     };
 
@@ -514,7 +522,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       o_glb[j] = (unsigned)((size_t)o_tok[j] * v_pitch) + 2u * (unsigned)(cbase + (WIDE ? 8 : 4) * (i16 >> 2));
     }
     auto store_out = [&](const int cc) __attribute__((always_inline)) {
-      const unsigned ob = lds0 + 2 * L::STAGE + (cc & 1) * L::OB;
+      const unsigned ob = lds0 + L::NSTAGE * L::STAGE + (cc & 1) * L::OB;
       const int nvalid = len - cc * C;
 #pragma unroll
       for (int j = 0; j < O_PASSES; ++j) {
@@ -529,16 +537,33 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       ob_g += v_step;
     };
 
-    if (NT > 0) request(0);
+    // AHEAD = how many chunks the requests run ahead of the compute waves.  With AHEAD = 2 the newest requests (and the
+    // stores issued after them) may still be in flight at the barrier: vector memory operations complete in the order
+    // they were issued, so allowing as many outstanding as one step issues leaves exactly the older step's complete.
+    constexpr int AHEAD = L::NSTAGE - 1;
+    constexpr int PER_STEP_FIRST = 1 + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? 6 : 0) + 6 + O_PASSES;
+    static_assert(PER_STEP_FIRST <= 63 && PER_STEP_SECOND <= 63, "the wait counter has six bits");
+    constexpr int VM_FIRST = (PER_STEP_FIRST & 15) | ((PER_STEP_FIRST >> 4) << 14) | 0x0f70;
+    constexpr int VM_SECOND = (PER_STEP_SECOND & 15) | ((PER_STEP_SECOND >> 4) << 14) | 0x0f70;
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a)
+      if (a < NT) request(a);
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     for (int c = 0; c < NT; ++c) {
-      if (c + 1 < NT) request(c + 1);   // into the stage that step c - 1 read: every wave is past the barrier that ended it
-      if (c > 0) store_out(c - 1);
-      __builtin_amdgcn_s_waitcnt(0x0f70);
+      // into the stage that step c - 1 read: every wave is past the barrier that ended it
+      const bool more = c + AHEAD < NT;
+      if (more) request(c + AHEAD);
+      if (c > 0 && !first) store_out(c - 1);
+      if (AHEAD == 2 && more) {
+        if (first) __builtin_amdgcn_s_waitcnt(VM_FIRST);
+        else __builtin_amdgcn_s_waitcnt(VM_SECOND);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+      }
       __syncthreads();
     }
-    if (NT > 0) store_out(NT - 1);
+    if (NT > 0 && !first) store_out(NT - 1);
     return;
   }
 
@@ -588,17 +613,12 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
   __syncthreads();   // chunk 0 has landed
 
   for (int c = 0; c < NT; ++c) {
-    const unsigned st = lds0 + (c & 1) * L::STAGE;
+    const unsigned st = lds0 + (c % L::NSTAGE) * L::STAGE;
     // the chunk's scalars (three separate 4-byte reads on purpose: read as one 16-byte vector whose lanes all name the
     // same address, the compiler folded the three elements into the first)
     const float dec_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C));
     const float glast_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C + 1));
     const float linf_v = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * C + 2));
-    if (c % per_blk == 0) {
-#pragma unroll
-      for (int m = 0; m < KT; ++m) Ssave[m] = S[m];
-      gsum = 0.f;
-    }
     // (1) the state as B operands
     bf16x8 SB[KS];
 #pragma unroll
@@ -608,14 +628,25 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     const float linf_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, linf_v)));
     const bool last_of_block = ((c + 1) % per_blk == 0) || (c == NT - 1);
     const bool keep = linf_c != 0.f || !last_of_block;
+    if (c % per_blk == 0) {
+      // The state that enters a block is needed again when the block is rolled back at its end (not typed linear) and
+      // for the hand-off output (the sequence's last block).  The type is the same for every chunk of a block.
+      if (linf_c == 0.f || c + per_blk >= NT) {
+#pragma unroll
+        for (int m = 0; m < KT; ++m) Ssave[m] = S[m];
+      }
+      gsum = 0.f;
+    }
     gsum += glast_c;
 
-    // R = k S, then O1 = q S (X below only needs R); operands are read AHEAD instructions before their use
+    // R = k S, then O1 = q S (X below only needs R); operands are read AHEAD instructions before their use.  The state's
+    // decay for the update at the end of the step rides along, one multiply under each matrix instruction (a step that
+    // ends in a roll-back overwrites the state anyway).
     f32x4 R[4], O1[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) { R[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; O1[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
     {
-      constexpr int NOP = (DELTA ? 2 : 1) * 4 * KS, AHEAD = 4;
+      constexpr int NOP = (DELTA ? 2 : 1) * 4 * KS, AHEAD = 4, NS = 4 * KT, PER = (NS + NOP - 1) / NOP;
       auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
         const int which = DELTA ? j / (4 * KS) : 1, jj = j % (4 * KS), s = jj / 4, t = jj % 4;
         return *reinterpret_cast<lds_b128_t>(st + (which ? L::OFF_Q : L::OFF_K) + a_kq[s] + t * 16 * L::KROW);
@@ -629,14 +660,9 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         const int which = DELTA ? j / (4 * KS) : 1, jj = j % (4 * KS), s = jj / 4, t = jj % 4;
         if (which) O1[t] = mfma16(opnd[j], SB[s], O1[t]);
         else R[t] = mfma16(opnd[j], SB[s], R[t]);
+#pragma unroll
+        for (int e = PER * j; e < PER * j + PER && e < NS; ++e) S[e >> 2][e & 3] *= dec_c;
       }
-    }
-    // the state's decay for the update at the end of the step (in the shadow of the matrix instructions above)
-    if (keep) {
-#pragma unroll
-      for (int m = 0; m < KT; ++m)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) S[m][r] *= dec_c;
     }
     // (2) v in accumulator layout (lane = column, registers = tokens 16 t + 4 g4 + r); zero past the end of the sequence
     f32x4 VN[4];
@@ -710,7 +736,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     }
     // (4) o = sq * O1 + P v_new, into the (transposed) output tile: the four token tiles side by side
     {
-      const unsigned ob = lds0 + 2 * L::STAGE + (c & 1) * L::OB;
+      const unsigned ob = lds0 + L::NSTAGE * L::STAGE + (c & 1) * L::OB;
       f32x4 O[4];
       bf16x8 PA[6];
 #pragma unroll
@@ -781,7 +807,7 @@ static int launch_scan(const LinearParams& p, hipStream_t stream, const char* wh
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
   const int grid = 8 * cdiv(n_chains, 8) * (p.V / L::BVW);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (NW + 1)), L::TOTAL, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (NW + 2)), L::TOTAL, stream, p);
   return check_launch(what);
 }
 
