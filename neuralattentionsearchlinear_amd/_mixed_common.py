@@ -47,11 +47,8 @@ def _get_attn_stream(device: torch.device) -> torch.cuda.Stream:
     return _attn_streams[idx]
 
 
-def _no_backward(*tensors):
-    if torch.is_grad_enabled() and any(t is not None and torch.is_tensor(t) and t.requires_grad for t in tensors):
-        raise NotImplementedError(
-            "only the forward of the mixed operator is built for gfx950; call it under torch.no_grad() "
-            "or with tensors that do not require grad")
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and torch.is_tensor(t) and t.requires_grad for t in tensors)
 
 
 def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block: int, flags: int,
@@ -89,11 +86,11 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
     return o, ht
 
 
-def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
+def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
                   scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size, attn_sw_size,
                   attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
                   incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
-                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0):
+                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0, return_aux: bool = False):
     """Shared forward of the mixed operators.  With inference=True it also returns the state at the
     start of the current selector block (4-tuple), as the reference's *_chunk_inference operators do."""
     if nats_block_size < CHUNK_SIZE:
@@ -112,8 +109,6 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
         raise NotImplementedError("packed sequences are not supported by the prefill hand-off")
     if not q_lattn.is_cuda:
         raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
-    _no_backward(q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types)
-
     io_dtype = q_lattn.dtype
     if io_dtype not in (torch.bfloat16, torch.float32):
         raise NotImplementedError(f"dtype {io_dtype} is not supported (bf16, or fp32 which is computed in bf16)")
@@ -158,8 +153,13 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
         for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks']):
             t.record_stream(side)
         o_attn.record_stream(cur)
+        _lse.record_stream(cur)
     if io_dtype != torch.bfloat16:
         o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
+    if return_aux:
+        aux = dict(q_attn=q_attn, k_attn=k_attn, v_attn=v_attn, q_lattn=q_lattn, k_lattn=k_lattn, v_lattn=v_lattn, beta=beta, g=g,
+                   types=types, lse=_lse, nats_block_indices=r['nats_block_indices'], n_nats_blocks=r['n_nats_blocks'])
+        return o_lin, o_attn, ht, aux
     if not inference:
         return o_lin, o_attn, ht
     h_start = None
@@ -180,3 +180,83 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
             rolled = hs * torch.exp(gs).view(ht.shape[0], H, 1, 1) if decay_non_linear else hs
             h_start = torch.where(lin, ht, rolled)
     return o_lin, o_attn, ht, h_start
+
+
+class _MixedFunction(torch.autograd.Function):
+    """The mixed operator with its backward (src/nats/ops/mixed_ops/mixed_attn_gdn.py:193-283,
+    src/nats/ops/mixed_ops/mixed_attn_mamba.py:194-292): the softmax branch's gradients come from the HIP backward
+    (natsl_softmax_sparse_bwd), the linear branch's from the differentiable chunked forward in _linear_bwd.py; the
+    selector's straight-through gradient is returned for nats_block_types, column 0 = softmax op, column 1 = linear op."""
+
+    @staticmethod
+    def forward(ctx, cfg, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types):
+        with torch.no_grad():
+            o_lin, o_attn, ht, aux = _mixed_forward_impl(
+                cfg['kind'], q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
+                cfg['scale_attn'], cfg['scale_lattn'], None, None, cfg['block'], None, cfg['attn_same_block'], cfg['lin_intra'],
+                cfg['output_final_state'], cfg['decay_non_linear'], True, False, cfg['qk_l2norm'], return_aux=True)
+        ctx.cfg = cfg
+        ctx.in_dtypes = tuple(None if t is None else t.dtype for t in (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
+                                                                       initial_state, g, beta, nats_block_types))
+        ctx.has_h0 = initial_state is not None
+        saved = [aux[n] for n in ('q_attn', 'k_attn', 'v_attn', 'q_lattn', 'k_lattn', 'v_lattn', 'g', 'types', 'lse',
+                                  'nats_block_indices', 'n_nats_blocks')]
+        saved += [o_attn.to(torch.bfloat16), aux['beta'] if aux['beta'] is not None else g.new_zeros(0),
+                  initial_state if initial_state is not None else g.new_zeros(0)]
+        ctx.save_for_backward(*saved)
+        if ht is None:
+            return o_lin, o_attn, None
+        return o_lin, o_attn, ht
+
+    @staticmethod
+    def backward(ctx, do_lin, do_attn, dht):
+        from ._linear_bwd import linear_chunk_backward
+        from .attns import parallel_attn_nats_bwd
+        cfg = ctx.cfg
+        (q_a, k_a, v_a, q_l, k_l, v_l, g, types, lse, idx, nblk, o_attn, beta, h0) = ctx.saved_tensors
+        beta = beta if beta.numel() else None
+        h0 = h0 if ctx.has_h0 else None
+        B, NB, HN, _ = types.shape
+        if do_attn is not None:
+            dq_a, dk_a, dv_a, _, dn_attn = parallel_attn_nats_bwd(
+                q_a, k_a, v_a, o_attn, types, idx, nblk, None, lse, do_attn.to(torch.bfloat16).contiguous(), scale=cfg['scale_attn'],
+                NAtS_block_size=cfg['block'], compute_incomplete_chunk_scores=cfg['attn_same_block'],
+                compute_dnats_for_invalid_blocks_attn=cfg['dnats_invalid_attn'])
+        else:
+            dq_a, dk_a, dv_a = torch.zeros_like(q_a), torch.zeros_like(k_a), torch.zeros_like(v_a)
+            dn_attn = torch.zeros(B, NB, HN, dtype=torch.float32, device=types.device)
+        if do_lin is None:
+            do_lin = torch.zeros(*q_l.shape[:3], v_l.shape[-1], dtype=torch.float32, device=q_l.device)
+        dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
+            cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, cfg['scale_lattn'], cfg['block'], cfg['decay_non_linear'],
+            cfg['qk_l2norm'], cfg['lin_intra'], do_lin, dht, cfg['dnats_invalid_linear'])
+        d_types = torch.stack([dn_attn.float(), dn_lin.float()], -1)
+        grads = [dq_a, dk_a, dv_a, dq_l, dk_l, dv_l, dh0, dg, dbeta, d_types]
+        grads = [None if (t is None or dt is None) else t.to(dt) for t, dt in zip(grads, ctx.in_dtypes)]
+        return (None, *grads)
+
+
+def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
+                  scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size, attn_sw_size,
+                  attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
+                  incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
+                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0,
+                  dnats_invalid_attn: bool = False, dnats_invalid_linear: bool = False):
+    """Entry of the mixed operators: the plain forward, or, when a tensor requires grad, the differentiable operator."""
+    tensors = (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types)
+    # (the prefill operators are plain functions in the reference too: their outputs carry no gradient)
+    if inference or not _wants_grad(*tensors):
+        return _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta,
+                                   nats_block_types, scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size,
+                                   attn_sw_size, attn_same_block, lin_intra, output_final_state, decay_non_linear,
+                                   incomplete_block_start_with_ht, use_g_for_attn, qk_l2norm, inference, op_type_last_chunk,
+                                   n_tokens_in_current_block)
+    if cu_seqlens is not None or cu_seqlens_nats is not None:
+        raise NotImplementedError("packed sequences are not supported by the backward yet")
+    if attn_sw_size is not None or use_g_for_attn or not incomplete_block_start_with_ht:
+        raise NotImplementedError("attn_sw_size / use_g_for_attn / incomplete_block_start_with_ht=False are not built")
+    cfg = dict(kind=kind, scale_attn=float(scale_attn), scale_lattn=float(scale_lattn), block=int(nats_block_size),
+               attn_same_block=bool(attn_same_block), lin_intra=bool(lin_intra), output_final_state=bool(output_final_state),
+               decay_non_linear=bool(decay_non_linear), qk_l2norm=bool(qk_l2norm), dnats_invalid_attn=bool(dnats_invalid_attn),
+               dnats_invalid_linear=bool(dnats_invalid_linear))
+    return _MixedFunction.apply(cfg, *tensors)

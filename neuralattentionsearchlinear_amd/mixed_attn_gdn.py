@@ -1,5 +1,5 @@
 """nats_mixed_attn_gdn: softmax branch + Gated DeltaNet branch behind the reference's operator API
-(src/nats/ops/mixed_ops/mixed_attn_gdn.py:286-325), forward only."""
+(src/nats/ops/mixed_ops/mixed_attn_gdn.py:286-325)."""
 from __future__ import annotations
 
 from dataclasses import dataclass
@@ -48,8 +48,8 @@ def nats_mixed_attn_gdn(
 ):
     """-> (o_gated_delta_net [B,T,H,V], o_attn [B,T,HQ,Va], final_state fp32 [N,H,K,V] or None).
 
-    n_nats_blocks and the two compute_dnats_* flags (backward-only) are accepted for signature
-    compatibility; the block counts are recomputed on the device from nats_block_types.
+    n_nats_blocks is accepted for signature compatibility (the block counts are recomputed on the device from
+    nats_block_types); the two compute_dnats_* flags select the selector gradient of the backward.
     """
     strategy = all_incomplete_ops[ops_for_incomplete_chunks]
     if scale_attn is None:
@@ -62,7 +62,9 @@ def nats_mixed_attn_gdn(
         attn_same_block=strategy.attn, lin_intra=strategy.gated_delta_net,
         output_final_state=output_final_state_gated_delta, decay_non_linear=decay_for_non_gdn_blocks,
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
-        qk_l2norm=lattn_use_qk_l2norm_in_kernel)
+        qk_l2norm=lattn_use_qk_l2norm_in_kernel,
+        dnats_invalid_attn=compute_dnats_for_invalid_blocks_attn,
+        dnats_invalid_linear=compute_dnats_for_invalid_blocks_linear_att)
 
 
 def nats_mixed_attn_gdn_chunk_inference(

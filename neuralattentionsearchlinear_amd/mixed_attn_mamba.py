@@ -1,5 +1,5 @@
 """nats_mixed_attn_mamba: softmax branch + Mamba2-style SSD branch behind the reference's operator
-API (src/nats/ops/mixed_ops/mixed_attn_mamba.py:295-332), forward only."""
+API (src/nats/ops/mixed_ops/mixed_attn_mamba.py:295-332)."""
 from __future__ import annotations
 
 from dataclasses import dataclass
@@ -56,7 +56,9 @@ def nats_mixed_attn_mamba(
         attn_same_block=strategy.attn, lin_intra=strategy.mamba,
         output_final_state=output_final_state_mamba, decay_non_linear=decay_for_non_mamba_blocks,
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
-        qk_l2norm=False)
+        qk_l2norm=False,
+        dnats_invalid_attn=compute_dnats_for_invalid_blocks_attn,
+        dnats_invalid_linear=compute_dnats_for_invalid_blocks_linear_att)
 
 
 def nats_mixed_attn_mamba_chunk_inference(

@@ -88,11 +88,7 @@ class FusedMultiInputRMSNormGated(nn.Module):
         return two_inputs_rms_norm_gated(x1, x2, g, x_weights_after_norm, self.weight1, self.weight2, self.eps)
 
 
-def two_inputs_rms_norm_gated(x1, x2, g, x_weights, weight1, weight2, eps: float = 1e-5):
-    if not x1.is_cuda:
-        raise _capi.NatslError("the norm-gate runs on the GPU only (no CPU fallback)")
-    if torch.is_grad_enabled() and any(t.requires_grad for t in (x1, x2, g, x_weights, weight1, weight2)):
-        raise NotImplementedError("only the forward of the two-input norm-gate is built; call it under torch.no_grad()")
+def _norm_gate_fwd(x1, x2, g, x_weights, weight1, weight2, eps):
     io_dtype = x1.dtype
     D = x1.shape[-1]
     to = lambda t: t.detach().to(torch.bfloat16).contiguous()
@@ -107,3 +103,35 @@ def two_inputs_rms_norm_gated(x1, x2, g, x_weights, weight1, weight2, eps: float
                                          _capi.stream_ptr(a.device))
     _capi.check(rc, "natsl_norm_gate_fwd")
     return y.to(io_dtype)
+
+
+class _NormGate(torch.autograd.Function):
+    """The HIP forward with a backward for training: the gradients are those of the same formula evaluated as fp32 torch
+    operations (elementwise work plus two row reductions; replaces the backward of
+    src/nats/modules/fused_norm_gate.py:185-420 in function)."""
+
+    @staticmethod
+    def forward(ctx, x1, x2, g, x_weights, weight1, weight2, eps):
+        ctx.save_for_backward(x1, x2, g, x_weights, weight1, weight2)
+        ctx.eps = eps
+        return _norm_gate_fwd(x1, x2, g, x_weights, weight1, weight2, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        saved = ctx.saved_tensors
+        with torch.enable_grad():
+            x1, x2, g, xw, w1, w2 = (t.detach().float().requires_grad_(True) for t in saved)
+            r1 = x1 * torch.rsqrt((x1 * x1).mean(-1, keepdim=True) + ctx.eps) * w1
+            r2 = x2.reshape(x1.shape) * torch.rsqrt((x2.reshape(x1.shape) ** 2).mean(-1, keepdim=True) + ctx.eps) * w2
+            gate = g.reshape(x1.shape)
+            y = (r1 * xw[..., 0:1] + r2 * xw[..., 1:2]) * gate * torch.sigmoid(gate)
+            grads = torch.autograd.grad(y, (x1, x2, g, xw, w1, w2), dy.float())
+        return tuple(gr.to(t.dtype) for gr, t in zip(grads, saved)) + (None,)
+
+
+def two_inputs_rms_norm_gated(x1, x2, g, x_weights, weight1, weight2, eps: float = 1e-5):
+    if not x1.is_cuda:
+        raise _capi.NatslError("the norm-gate runs on the GPU only (no CPU fallback)")
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (x1, x2, g, x_weights, weight1, weight2)):
+        return _NormGate.apply(x1, x2, g, x_weights, weight1, weight2, eps)
+    return _norm_gate_fwd(x1, x2, g, x_weights, weight1, weight2, eps)

@@ -61,22 +61,51 @@ def _seq_args(seqs: Optional[PackedSeqs], total: int = 0):
     return _capi.ptr(seqs.table), seqs.n_seqs, total
 
 
-def mean_pooling(x: torch.Tensor, chunk_size: int, cu_seqlens=None, seqs: Optional[PackedSeqs] = None) -> torch.Tensor:
-    """x [B,T,H,D] (or [B,T,D]) -> block means [B,ceil(T/chunk),H,D]; replaces fla's mean_pooling
-    as used at src/nats/layers/natsl_attn_gdn.py:412-417 (kernel src/nats/ops/utils/pooling.py:26-57)."""
-    squeeze = x.dim() == 3
-    if squeeze:
-        x = x.unsqueeze(-2)
+def _mean_pooling_fwd(x: torch.Tensor, chunk_size: int, seqs: Optional[PackedSeqs]) -> torch.Tensor:
     B, T, H, D = x.shape
     x = x.contiguous()
-    if cu_seqlens is not None and seqs is None:
-        seqs = pack_sequences(cu_seqlens, None, chunk_size, x.device)
     nb = seqs.total_blocks if seqs is not None else -(-T // chunk_size)
     out = torch.empty(B, nb, H, D, dtype=x.dtype, device=x.device)
     sp, ns, tot = _seq_args(seqs, nb)
     rc = _capi.lib().natsl_mean_pool(_capi.ptr(x), _capi.ptr(out), B, T, H * D, chunk_size, _capi.dtype_code(x.dtype), sp, ns,
                                      tot, _capi.stream_ptr(x.device))
     _capi.check(rc, "natsl_mean_pool")
+    return out
+
+
+class _MeanPooling(torch.autograd.Function):
+    """Block means with their backward: every token of a block receives the block's gradient over the block's length
+    (the reference's pooling backward, src/nats/ops/utils/pooling.py:60-100)."""
+
+    @staticmethod
+    def forward(ctx, x, chunk_size):
+        ctx.chunk, ctx.T = chunk_size, x.shape[1]
+        return _mean_pooling_fwd(x, chunk_size, None)
+
+    @staticmethod
+    def backward(ctx, dy):
+        T, n = ctx.T, ctx.chunk
+        nb = dy.shape[1]
+        lens = torch.full((nb,), float(n), device=dy.device, dtype=torch.float32)
+        lens[-1] = float(T - (nb - 1) * n)
+        dx = (dy.float() / lens.view(1, nb, 1, 1)).to(dy.dtype).repeat_interleave(n, dim=1)[:, :T]
+        return dx, None
+
+
+def mean_pooling(x: torch.Tensor, chunk_size: int, cu_seqlens=None, seqs: Optional[PackedSeqs] = None) -> torch.Tensor:
+    """x [B,T,H,D] (or [B,T,D]) -> block means [B,ceil(T/chunk),H,D]; replaces fla's mean_pooling
+    as used at src/nats/layers/natsl_attn_gdn.py:412-417 (kernel src/nats/ops/utils/pooling.py:26-57)."""
+    squeeze = x.dim() == 3
+    if squeeze:
+        x = x.unsqueeze(-2)
+    if cu_seqlens is not None and seqs is None:
+        seqs = pack_sequences(cu_seqlens, None, chunk_size, x.device)
+    if torch.is_grad_enabled() and x.requires_grad:
+        if seqs is not None:
+            raise NotImplementedError("the pooling backward is not built for packed sequences")
+        out = _MeanPooling.apply(x, chunk_size)
+    else:
+        out = _mean_pooling_fwd(x, chunk_size, seqs)
     return out.squeeze(-2) if squeeze else out
 
 
@@ -97,6 +126,11 @@ def hard_select(logits: torch.Tensor, force_last_block: bool = False, seqs: Opti
                                        _capi.dtype_code(logits.dtype), int(force_last_block), sp, ns, tot,
                                        _capi.stream_ptr(logits.device))
     _capi.check(rc, "natsl_hard_select")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        # straight-through estimator of the reference (hard value, gradient of the softmax:
+        # `y_hard - y_soft.detach() + y_soft`, src/nats/layers/natsl_attn_gdn.py:47-61); the added term is exactly zero
+        y_soft = logits.softmax(-1)
+        types = types + (y_soft - y_soft.detach())
     return types, nblk
 
 

@@ -2,7 +2,8 @@
 names of the reference layer (src/nats/layers/natsl_attn_gdn.py:64-666).
 
 Projections, short convolutions and norms are torch; block pooling, the selector, the mixed operator
-and the output norm-gate are the HIP kernels of this package.  Forward only (no backward).  With a NAtSCache
+and the output norm-gate are the HIP kernels of this package.  Training works: the softmax branch's backward is a HIP
+kernel, the linear branch, the pooling and the norm-gate differentiate through torch operations.  With a NAtSCache
 the layer prefills once in chunk mode on the empty cache and then decodes in steps of fewer than 64 tokens;
 continuing a chunked prefill on a cache that already holds tokens raises NotImplementedError (the reference's
 attention operator cannot do it either: it sizes its output by the keys, src/nats/ops/attns/attns.py:1439,1491).

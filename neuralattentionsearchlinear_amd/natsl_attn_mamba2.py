@@ -1,7 +1,8 @@
 """Mamba2-SSD / softmax hybrid token mixer with the forward signature, returns and parameter names of
 the reference layer (src/nats/layers/natsl_attn_mamba2.py:100-599).  Same scope as the Gated-DeltaNet
-layer: forward only; with a cache, one chunked prefill on the empty cache and then decode steps of fewer
-than 64 tokens."""
+layer: trainable (the linear branch, the pooling and the norm-gate differentiate through torch operations, the
+softmax branch through its HIP backward); with a cache, one chunked prefill on the empty cache and then decode steps of
+fewer than 64 tokens."""
 from __future__ import annotations
 
 import math

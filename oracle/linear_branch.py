@@ -130,7 +130,11 @@ def _intra_chunk_terms(qh, kh, g_c, C):
 
 
 def _scan(qe, w, u, kd, P, glast, lin, scale, h0, block, C, T, decay_non_linear, delta_rule, B, H, K, V, NT, dtype,
-          intra=True):
+          intra=True, gate_on=None, gate_off=None):
+    """gate_on / gate_off [B,NT,H] (default: ones / absent) multiply a chunk's additive state update where it is kept /
+    add it, scaled, to the rolled-back state where it is not: d loss / d gate is the selector's straight-through gradient
+    for the linear operator, <state gradient behind the chunk, k~^T v_new> (src/nats/ops/common/chunk_o.py:438-443 for
+    blocks typed linear, :487-492 for the others when their gradient is asked for)."""
     S = torch.zeros(B, H, K, V, dtype=dtype) if h0 is None else h0.to(dtype).clone()
     o = torch.zeros(B, H, NT, C, V, dtype=dtype)
     S_start, gsum = S, torch.zeros(B, H, dtype=dtype)
@@ -142,18 +146,25 @@ def _scan(qe, w, u, kd, P, glast, lin, scale, h0, block, C, T, decay_non_linear,
         o[:, :, c] = scale * (qe[:, :, c] @ S)
         if intra:
             o[:, :, c] += scale * (P[:, :, c] @ v_new)
-        S = torch.exp(glast[:, :, c])[..., None, None] * S + kd[:, :, c].transpose(-1, -2) @ v_new
+        upd = kd[:, :, c].transpose(-1, -2) @ v_new
+        if gate_on is not None:
+            upd_on = gate_on[:, c, :, None, None] * upd
+        else:
+            upd_on = upd
+        S = torch.exp(glast[:, :, c])[..., None, None] * S + upd_on
         gsum = gsum + glast[:, :, c]
         if (c + 1) % per == 0 or c == NT - 1:
             keep = lin[:, (c * C) // block][..., None, None]
             back = S_start * torch.exp(gsum)[..., None, None] if decay_non_linear else S_start
+            if gate_off is not None:
+                back = back + gate_off[:, c, :, None, None] * upd
             S = torch.where(keep, S, back)
     o = o.permute(0, 2, 3, 1, 4).reshape(B, NT * C, H, V)[:, :T]
     return o, S
 
 
 def gdn_chunked(q, k, v, g, beta, lin_types, scale, h0=None, block=64, decay_non_linear=True, l2norm_qk=True,
-                dtype=torch.float32, intra=True):
+                dtype=torch.float32, intra=True, gate_on=None, gate_off=None):
     """Chunk-parallel Gated DeltaNet forward (same result as gdn_token_recurrence).
 
     Per 64-token chunk: A = strict_lower(beta_i k_i.k_j e^{gamma_i-gamma_j}), Tm = (I+A)^-1,
@@ -186,11 +197,11 @@ def gdn_chunked(q, k, v, g, beta, lin_types, scale, h0=None, block=64, decay_non
     kd = kc * torch.exp(glast.unsqueeze(-1) - gamma).unsqueeze(-1)
     lin = _expand_types(lin_types, H)
     return _scan(qe, w, u, kd, P, glast, lin, scale, h0, block, C, T, decay_non_linear, True, B, H, K, V, NT, dtype,
-                 intra)
+                 intra, gate_on, gate_off)
 
 
 def mamba_chunked(q, k, v, g, lin_types, scale, h0=None, block=64, decay_non_linear=True, dtype=torch.float32,
-                  intra=True):
+                  intra=True, gate_on=None, gate_off=None):
     """Chunk-parallel SSD forward: o = scale[(q e^{gamma}) S + tril(q k^T e^{gamma_i-gamma_j}) v],
     S' = e^{gamma_last} S + (k e^{min(gamma_last-gamma,0)})^T v
     (src/nats/ops/mamba/chunk_h.py:139-204, src/nats/ops/mamba/chunk_o.py:146-198)."""
@@ -208,7 +219,7 @@ def mamba_chunked(q, k, v, g, lin_types, scale, h0=None, block=64, decay_non_lin
     kd = kc * torch.exp(torch.clamp(glast.unsqueeze(-1) - gamma, max=0.0)).unsqueeze(-1)
     lin = _expand_types(lin_types, H)
     return _scan(qe, None, vc, kd, P, glast, lin, scale, h0, block, C, T, decay_non_linear, False, B, H, K, V, NT,
-                 dtype, intra)
+                 dtype, intra, gate_on, gate_off)
 
 
 # --------------------------------------------------------------------------------------
@@ -286,3 +297,37 @@ def gdn_flops(n_chunks_total: float, n_linear_chunks: float, K: int, V: int, C: 
 def mamba_flops(n_chunks_total: float, n_linear_chunks: float, K: int, V: int, C: int = CHUNK) -> float:
     per = 2 * C * C * (K + V) + 4 * C * K * V
     return per * n_chunks_total - 2 * C * K * V * (n_chunks_total - n_linear_chunks)
+
+
+def linear_branch_bwd(kind, q, k, v, g, beta, lin_types, scale, do, dht=None, h0=None, block=64, decay_non_linear=True,
+                      l2norm_qk=True, intra=True, dnats_for_invalid_blocks=False, dtype=torch.float64):
+    """Gradients of the chunked linear branch by autograd through gdn_chunked / mamba_chunked in fp64:
+    -> dict(dq, dk, dv, dg, dbeta, dh0, dnats [B,NB,HN]).  dnats: per selector block and head, the gate gradients of its
+    chunks and heads summed (src/nats/ops/common/chunk_o.py:1571-1575); blocks not typed linear contribute their
+    zero-gate gradient only when dnats_for_invalid_blocks."""
+    B, T, H, K = q.shape
+    NT = -(-T // CHUNK)
+    per = block // CHUNK
+    HN = lin_types.shape[2]
+    leaf = lambda t: None if t is None else t.detach().to(dtype).requires_grad_(True)
+    qf, kf, vf, gf, bf, hf = leaf(q), leaf(k), leaf(v), leaf(g), leaf(beta), leaf(h0)
+    gate_on = torch.ones(B, NT, H, dtype=dtype, requires_grad=True)
+    gate_off = torch.zeros(B, NT, H, dtype=dtype, requires_grad=True)
+    if kind == 'gdn':
+        o, S = gdn_chunked(qf, kf, vf, gf, bf, lin_types, scale, hf, block, decay_non_linear, l2norm_qk, dtype, intra, gate_on, gate_off)
+    else:
+        o, S = mamba_chunked(qf, kf, vf, gf, lin_types, scale, hf, block, decay_non_linear, dtype, intra, gate_on, gate_off)
+    loss = (o * do.to(dtype)).sum()
+    if dht is not None:
+        loss = loss + (S * dht.to(dtype)).sum()
+    loss.backward()
+    lin_c = _expand_types(lin_types, H).repeat_interleave(per, dim=1)[:, :NT]
+    dn = torch.where(lin_c, gate_on.grad, torch.zeros_like(gate_on.grad))
+    if dnats_for_invalid_blocks:
+        dn = dn + torch.where(lin_c, torch.zeros_like(dn), gate_off.grad)
+    NB = lin_types.shape[1]
+    if NB * per != NT:
+        dn = torch.cat([dn, dn.new_zeros(B, NB * per - NT, H)], 1)
+    dn = dn.view(B, NB, per, HN, H // HN).sum((2, 4))
+    g_ = lambda t: None if t is None else t.grad
+    return dict(dq=g_(qf), dk=g_(kf), dv=g_(vf), dg=g_(gf), dbeta=g_(bf), dh0=g_(hf), dnats=dn)

@@ -1,0 +1,111 @@
+"""GPU parity: backward of the mixed operators and a training step of the two layers.
+
+Oracle: oracle.linear_branch.linear_branch_bwd (autograd through the chunked form in fp64, pinned on the CPU by the
+token recurrence and by finite differences of the gates) and oracle.softmax_branch.softmax_branch_bwd.  Gradient tolerance
+as for the softmax backward: rel-L2 5e-3, max-abs 2e-2 of the reference's largest magnitude."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import linear_branch as LB
+from oracle import softmax_branch as SB
+from tests._util import make_gates, make_qkv, make_types, max_abs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+def _close(a, b, what, rl_tol=5e-3):
+    rl, ma, top = rel_l2(a, b), max_abs(a, b), float(b.abs().max())
+    assert rl <= rl_tol and ma <= 2e-2 * max(top, 1.0), f"{what}: rel-L2 {rl:.3e}, max-abs {ma:.3e} (largest reference value {top:.3e})"
+
+
+@pytest.mark.parametrize("kind,K,V,block,h0,invalid", [('gdn', 128, 128, 64, False, False), ('gdn', 64, 64, 64, True, True),
+                                                        ('gdn', 128, 64, 128, True, False), ('mamba', 128, 64, 64, True, False),
+                                                        ('mamba', 64, 64, 256, False, True)])
+def test_mixed_operator_backward(kind, K, V, block, h0, invalid):
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
+    B, T, H, HN = 2, 512, 4, 2
+    gen = torch.Generator().manual_seed(K + V)
+    q, k, v = make_qkv(B, T, H, K, V, 11)
+    if kind == 'mamba':
+        q, k = F.normalize(q.float(), dim=-1).bfloat16(), F.normalize(k.float(), dim=-1).bfloat16()
+    g, beta = make_gates(B, T, H, 12)
+    ty = make_types(B, T // block, HN, 0.4, 13, torch.bfloat16)
+    init = (torch.randn(B, H, K, V, generator=gen) * 0.3) if h0 else None
+    do_l, do_a = (torch.randn(B, T, H, V, generator=gen).bfloat16() for _ in range(2))
+    dht = torch.randn(B, H, K, V, generator=gen)
+    scale_l = K ** -0.5 if kind == 'gdn' else 1.0
+    # oracle
+    rl = LB.linear_branch_bwd(kind, q, k, v, g, beta if kind == 'gdn' else None, ty[..., 1], scale_l, do_l, dht, init, block, True,
+                              True, True, invalid)
+    dq_a, dk_a, dv_a, dn_a, dn_mag = SB.softmax_branch_bwd(q, k, v, ty, do_a, K ** -0.5, block, True, with_magnitude=True)
+    # the operator
+    leaf = lambda t: None if t is None else t.to(DEV).requires_grad_(True)
+    qa, ka, va, ql, kl, vl, gd, bd, hd, tyd = (leaf(t) for t in (q, k, v, q, k, v, g, beta, init, ty))
+    nb = ty.to(torch.int32).sum(1).to(DEV)
+    if kind == 'gdn':
+        o_l, o_a, ht = nats_mixed_attn_gdn(qa, ka, va, ql, kl, vl, hd, gd, bd, tyd, nb, nats_block_size=block,
+                                           ops_for_incomplete_chunks='all', output_final_state_gated_delta=True,
+                                           decay_for_non_gdn_blocks=True, compute_dnats_for_invalid_blocks_linear_att=invalid)
+    else:
+        o_l, o_a, ht = nats_mixed_attn_mamba(qa, ka, va, ql, kl, vl, hd, gd, tyd, nb, scale_lattn=1.0, nats_block_size=block,
+                                             ops_for_incomplete_chunks='all', output_final_state_mamba=True,
+                                             decay_for_non_mamba_blocks=True, compute_dnats_for_invalid_blocks_linear_att=invalid)
+    ((o_l.float() * do_l.to(DEV).float()).sum() + (o_a.float() * do_a.to(DEV).float()).sum() + (ht * dht.to(DEV)).sum()).backward()
+    torch.cuda.synchronize()
+    _close(ql.grad.float(), rl['dq'], "dq_lattn")
+    _close(kl.grad.float(), rl['dk'], "dk_lattn")
+    _close(vl.grad.float(), rl['dv'], "dv_lattn")
+    _close(gd.grad.float(), rl['dg'], "dg")
+    if kind == 'gdn':
+        _close(bd.grad.float(), rl['dbeta'], "dbeta")
+    if h0:
+        _close(hd.grad.float(), rl['dh0'], "dh0")
+    _close(qa.grad.float(), dq_a, "dq_attn")
+    _close(ka.grad.float(), dk_a, "dk_attn")
+    _close(va.grad.float(), dv_a, "dv_attn")
+    dt = tyd.grad.float().cpu().double()
+    err = (dt[..., 0] - dn_a).abs()
+    assert bool((err <= 2e-3 * dn_mag + 1e-6).all()), f"dnats (softmax op): error {float(err.max()):.3e}"
+    ref = rl['dnats']
+    assert float((dt[..., 1] - ref).abs().max()) <= 2e-2 * max(float(ref.abs().max()), 1.0) and rel_l2(dt[..., 1], ref) <= 1e-2, \
+        f"dnats (linear op): rel-L2 {rel_l2(dt[..., 1], ref):.3e}"
+    if not invalid:
+        nonlin = torch.round(ty[..., 1].float()) == 0
+        assert float(dt[..., 1][nonlin].abs().max() if nonlin.any() else 0.0) == 0.0
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+def test_layer_training_step(kind):
+    """One forward + backward of the layer in training mode: every parameter receives a finite gradient, and the gradients
+    of everything outside the selector agree with autograd through the layer oracle on the same (injected) block types.
+    The selector's own path (nats_layer) is the straight-through estimator of the operators, checked at operator level."""
+    from oracle import layer as olayer
+    from tests.test_gpu_layers import _layer_case
+    layer, cfg, w, x = _layer_case(kind)
+    layer = layer.to(DEV).float().train()
+    xd = x.to(DEV).requires_grad_(True)
+    out = layer(xd)
+    o = out[0] if isinstance(out, tuple) else out
+    gy = torch.randn(o.shape, generator=torch.Generator().manual_seed(5))
+    (o * gy.to(DEV)).sum().backward()
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        types, _, _ = layer.select_ops(xd.detach())
+    ocfg = dict(cfg, num_nats_head=cfg['num_heads'], attn_qk_norm=(kind == 'gdn'), attn_with_short_conv=(kind == 'gdn'))
+    wl = {k_: v_.detach().clone().float().requires_grad_(True) for k_, v_ in w.items()}
+    fn = olayer.gdn_layer if kind == 'gdn' else olayer.mamba_layer
+    # (the oracle rounds to bf16 where the operators do: their inputs and outputs; the cast passes gradients through)
+    ref, _ = fn(wl, ocfg, x, types=types.cpu(), act_dtype=torch.bfloat16, round_at='ops')
+    (ref * gy).sum().backward()
+    for name, p_ in layer.named_parameters():
+        assert p_.grad is not None and bool(torch.isfinite(p_.grad).all()), f"{name}: no finite gradient"
+        if name.startswith('nats_layer'):
+            assert float(p_.grad.abs().max()) > 0, "the selector receives no gradient"
+            continue
+        r_ = wl[name].grad
+        rl_, top = rel_l2(p_.grad.float(), r_), float(r_.abs().max())
+        assert rl_ <= 2e-2 and max_abs(p_.grad.float(), r_) <= 5e-2 * max(top, 1e-3), f"{name}: grad rel-L2 {rl_:.3e}"
+    assert xd.grad is not None and bool(torch.isfinite(xd.grad).all())

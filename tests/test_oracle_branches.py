@@ -245,3 +245,56 @@ def test_softmax_backward_closed_form_equals_autograd(same_block):
     want_dnats = (gb.view(B, NB, HN, HQ // HN).sum(-1)) * a                     # attention-typed blocks only
     for got, want, name in ((dq, gq, 'dq'), (dk, gk, 'dk'), (dv, gv, 'dv'), (dnats, want_dnats, 'dnats')):
         assert float((got - want).abs().max()) < 1e-9, name
+
+
+# --------------------------------------------------------------------------------------------
+# gradients of the linear branches (the oracle of the mixed operators' backward)
+# --------------------------------------------------------------------------------------------
+def test_linear_branch_gradients_match_finite_differences_and_the_token_recurrence():
+    """linear_branch_bwd is autograd through the chunked form; pinned by (i) autograd through the token-by-token
+    recurrence (a different computation of the same function) and (ii) central differences of the gates: the selector
+    gradient of a block typed linear is d loss / d (gate on its update), that of a block not typed linear
+    d loss / d (zero gate on the update it would have made)."""
+    import torch.nn.functional as F
+    from oracle import linear_branch as LB
+    g_ = torch.Generator().manual_seed(3)
+    B, T, H, K, V, block = 1, 256, 2, 16, 8, 64
+    q, k, v = (torch.randn(B, T, H, d, generator=g_, dtype=torch.float64) for d in (K, K, V))
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g_, dtype=torch.float64))
+    g = -F.softplus(torch.randn(B, T, H, generator=g_, dtype=torch.float64))
+    lin = torch.tensor([1., 0., 0., 1.]).view(1, 4, 1).expand(1, 4, 2).contiguous()
+    do = torch.randn(B, T, H, V, generator=g_, dtype=torch.float64)
+    dht = torch.randn(B, H, K, V, generator=g_, dtype=torch.float64)
+    r = LB.linear_branch_bwd('gdn', q, k, v, g, beta, lin, 0.3, do, dht, None, block, True, True, True, True)
+    # (i) the same gradients through the token recurrence
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, g, beta)]
+    o, S = LB.gdn_token_recurrence(*leaves, lin, 0.3, None, block, True, True, torch.float64)
+    ((o * do).sum() + (S * dht).sum()).backward()
+    for name, t in zip(('dq', 'dk', 'dv', 'dg', 'dbeta'), leaves):
+        assert torch.allclose(r[name], t.grad, rtol=1e-7, atol=1e-9), name
+    # (ii) gates by central differences
+    NT = T // 64
+
+    def loss(gate_on, gate_off):
+        o, S = LB.gdn_chunked(q, k, v, g, beta, lin, 0.3, None, block, True, True, torch.float64, True, gate_on, gate_off)
+        return float((o * do).sum() + (S * dht).sum())
+    eps = 1e-5
+    for c in range(NT):
+        for h in range(H):
+            on, off = torch.ones(B, NT, H, dtype=torch.float64), torch.zeros(B, NT, H, dtype=torch.float64)
+            which = on if lin[0, c, h] == 1 else off
+            which[0, c, h] += eps
+            up = loss(on, off)
+            which[0, c, h] -= 2 * eps
+            fd = (up - loss(on, off)) / (2 * eps)
+            assert abs(fd - float(r['dnats'][0, c, h])) <= 1e-6 * max(1.0, abs(fd)), (c, h, fd, float(r['dnats'][0, c, h]))
+    # without the gradient of the other blocks they get exactly zero
+    r0 = LB.linear_branch_bwd('gdn', q, k, v, g, beta, lin, 0.3, do, dht, None, block, True, True, True, False)
+    assert float(r0['dnats'][0, 1:3].abs().max()) == 0.0 and torch.equal(r0['dnats'][0, [0, 3]], r['dnats'][0, [0, 3]])
+    # Mamba: against its token recurrence
+    rm = LB.linear_branch_bwd('mamba', q, k, v, g, None, lin, 1.0, do, dht, None, block, True)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, g)]
+    o, S = LB.mamba_token_recurrence(*leaves, lin, 1.0, None, block, True, torch.float64)
+    ((o * do).sum() + (S * dht).sum()).backward()
+    for name, t in zip(('dq', 'dk', 'dv', 'dg'), leaves):
+        assert torch.allclose(rm[name], t.grad, rtol=1e-7, atol=1e-9), name
