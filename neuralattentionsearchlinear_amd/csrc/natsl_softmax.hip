@@ -12,6 +12,9 @@
 // apart).
 #include "natsl_device.h"
 #include "natsl_host.h"
+#include <atomic>
+#include <mutex>
+#include <stdlib.h>
 #include <type_traits>
 
 namespace natsl {
@@ -62,7 +65,9 @@ constexpr int OPERANDS_AHEAD = 3;
 
 // hide the keys behind the query (the wave's own chunk): key 32kt + 8(r/4) + 4hf + r%4 against query qloc0 + lane%32
 NATSL_DEVICE void mask_half(f32x16& s, const int kt, const int lane, const int qloc0) {
-  const int d = qloc0 + (lane & 31) - 32 * kt - 4 * (lane >> 5);  // visible iff 8(r/4) + r%4 <= d
+  int d = qloc0 + (lane & 31) - 32 * kt - 4 * (lane >> 5);  // visible iff 8(r/4) + r%4 <= d
+  // (kept where it is: hoisted out of the chunk loop, the sixteen comparisons below occupy 32 scalar registers for good)
+  asm volatile("" : "+v"(d));
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     if (8 * (r >> 2) + (r & 3) > d) s[r] = -INFINITY;
@@ -949,6 +954,506 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
   }
 }
 
+// =====================================================================================================================
+// The 8-wave schedule as a persistent kernel: one workgroup per CU works through 256-query tiles that it takes from
+// work queues, and the K/V rings never drain between two tiles.
+//
+// What a workgroup of the kernel above pays per tile besides its chunk loop (cycle counters, 19 chunks per tile on
+// average): ~5 500 cycles until the CU has been given its next workgroup, ~14 000 of prologue (kernel arguments, index
+// arithmetic, the queries, the block types and the block list, the first keys and values: four dependent round trips
+// to memory, two barriers, the first transposition) and ~3 800 of epilogue, against ~58 000 in the loop.  Here
+//  * the memory side is ONE stream of chunks across tiles.  Chunk c of a tile with n chunks has stream position sp0 + c,
+//    the next tile's chunk j has sp0 + n + j, and every ring slot is chosen by stream position.  The rules of the loop
+//    (after barrier k: request raw V(k+3), then K(k+4); the late waves transpose V(k+2)) simply run on into the next
+//    tile, whose first chunks need no block list: when a tile's loop ends, K(0..3) and V(0..2) of the next tile are on
+//    their way or already there, and V(0), V(1) are transposed;
+//  * the compute side makes a clean cut between tiles: output straight from the accumulators (no LDS), then one barrier
+//    that hands over what the late waves prepared for the new tile while the old one was running (its block types, its
+//    list of prior attention blocks in LDS, how many there are, and which tile comes after it), then QK(0);
+//  * the queries of the next tile are requested before the output code and used after it;
+//  * the kernel starts with a "virtual" tile of four chunks in which no wave has anything to compute: its loop is what
+//    fills the rings for the first real tile, so there is no separate prologue.
+// Tiles come from eight queues, one per XCD (a workgroup reads which XCD it runs on): queue x lists the tiles of
+// (batch, head) pairs x, x+8, ... pair after pair, heaviest tile first, so the tiles that share a pair's K/V run
+// together on one L2; a workgroup whose queue is used up takes from the others.  A queue is a ticket counter in device
+// memory; the last workgroup to finish sets the counters back to zero.
+constexpr int STREAM_ROWS = 1088;  // chunk table of a tile: up to 1024 + 32 chunks of its own and four of the next tile (two tiles' tables are resident)
+constexpr int STREAM_QUEUES = 8;
+constexpr int STREAM_SLOT_WORDS = 16;  // per launch slot: 8 ticket counters, 1 count of finished workgroups
+
+struct StreamTile {
+  int valid, n, hq, tile, hkv, hn, dstart, dblk;  // the tile AFTER the one this record belongs to
+  unsigned diag_lo, diag_hi;                      // this tile: which of the blocks from dstart on are typed attention
+  int count[4];                                   // this tile: prior attention blocks found by each late wave
+  int pad[2];
+};
+
+NATSL_DEVICE unsigned xcc_id() {
+  unsigned x;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+  return x & (STREAM_QUEUES - 1);
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(512, 1) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void softmax_stream_kernel(const SoftmaxParams p, unsigned* queue) {
+  constexpr int QW = 32, QTILE = 256, KSTEPS = DK / 16, VT = DV / 32;
+  constexpr int KTILE = 64 * DK * 2, VRING = 3, VTILE = DV * VTP * 2, RTILE = 64 * DV * 2;  // bytes
+  constexpr int KI = DK / 32, RI = DV / 32, KROWS_I = 512 / DK, RROWS_I = 512 / DV;
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int rows[2][STREAM_ROWS];
+  __shared__ __align__(16) StreamTile info[2];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hf = lane >> 5;
+  const bool late = wave >= 4;
+  const int gw = wave & 3;
+  const int Bs = p.block, per_blk = Bs >> 6;
+  const unsigned NT = (unsigned)p.T / QTILE;
+  const unsigned n_pairs = (unsigned)(p.B * p.HQ);
+  const size_t krow = (size_t)p.HKV * DK, vrow = (size_t)p.HKV * DV;
+  const size_t list_stride = (size_t)p.HN * 2;
+  constexpr int K_SHIFT = DK == 128 ? 8 : 7, V_SHIFT = DV == 128 ? 8 : 7;  // log2 of a K / V row in bytes
+  const unsigned lds_k = ((unsigned)(size_t)smem + 1023u) & ~1023u, lds_r = lds_k + 4 * KTILE, lds_v = lds_r + 2 * RTILE;
+
+  // ---- lane constants of the data movement (as in the kernel above) ----------------------------------------------
+  // Source offsets of the DMA instructions: lane l of instruction j fills LDS row rows_per_instr * j + l / segs, position
+  // l % segs, with the segment that the swizzle puts there.  A chunk is named by the row index of its first key in the
+  // [B*T*HKV] row space of K and V, (token * HKV + kv head): its address is the tensor base plus that index shifted.
+  unsigned k_src[KI], r_src[RI];
+#pragma unroll
+  for (int j = 0; j < KI; ++j) {
+    const int r = KROWS_I * (KI * gw + j) + lane / (DK / 8), pos = lane % (DK / 8);
+    k_src[j] = (unsigned)((size_t)r * krow * sizeof(bf16_t)) + 16u * (pos ^ (DK == 128 ? (r & 15) : ((r >> 1) & 7)));
+  }
+#pragma unroll
+  for (int j = 0; j < RI; ++j) {
+    const int r = RROWS_I * (RI * gw + j) + lane / (DV / 8), pos = lane % (DV / 8);
+    r_src[j] = (unsigned)((size_t)r * vrow * sizeof(bf16_t)) + 16u * (pos ^ ((r >> 2) & (DV / 8 - 1)));
+  }
+  auto dma_r = [&](const int row, const unsigned sp) __attribute__((always_inline)) {
+    const char* g = reinterpret_cast<const char*>(p.v) + ((size_t)(unsigned)row << V_SHIFT);
+    const unsigned l0 = lds_r + (sp & 1) * RTILE + RI * gw * 1024;
+#pragma unroll
+    for (int j = 0; j < RI; ++j) dma16(g, r_src[j], l0 + j * 1024);
+  };
+  auto dma_k = [&](const int row, const unsigned sp) __attribute__((always_inline)) {
+    const char* g = reinterpret_cast<const char*>(p.k) + ((size_t)(unsigned)row << K_SHIFT);
+    const unsigned l0 = lds_k + (sp & 3) * KTILE + KI * gw * 1024;
+#pragma unroll
+    for (int j = 0; j < KI; ++j) dma16(g, k_src[j], l0 + j * 1024);
+  };
+  const int lt = tid & 255;
+  const int v_kg = lt & 15, v_sg = lt >> 4;
+  const bool v_on = v_sg < DV / 8;
+  const unsigned v_raw = (unsigned)(4 * v_kg * DV * 2) + 16u * ((v_on ? v_sg : 0) ^ (v_kg & (DV / 8 - 1)));
+  const unsigned v_dst = (unsigned)(8 * v_sg * VTP * 2) + 32u * (v_kg >> 2) + 8u * (2 * (v_kg & 1) + ((v_kg >> 1) & 1));
+  auto transpose_v = [&](const unsigned sp) __attribute__((always_inline)) {
+    if (v_on) {
+      typedef __attribute__((address_space(3))) const u32x4* lds_r4;
+      typedef __attribute__((address_space(3))) u32x2* lds_w;
+      unsigned src = lds_r + (sp & 1) * RTILE + v_raw;
+      asm("" : "+v"(src));
+      u32x4 rv[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rv[j] = *reinterpret_cast<lds_r4>(src + j * DV * 2);
+      const unsigned a = lds_v + (sp % VRING) * VTILE + v_dst;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        u32x2 lo, hi;
+        lo[0] = __builtin_amdgcn_perm(rv[1][d], rv[0][d], 0x05040100u);
+        lo[1] = __builtin_amdgcn_perm(rv[3][d], rv[2][d], 0x05040100u);
+        hi[0] = __builtin_amdgcn_perm(rv[1][d], rv[0][d], 0x07060302u);
+        hi[1] = __builtin_amdgcn_perm(rv[3][d], rv[2][d], 0x07060302u);
+        *reinterpret_cast<lds_w>(a + (2 * d) * VTP * 2) = lo;
+        *reinterpret_cast<lds_w>(a + (2 * d + 1) * VTP * 2) = hi;
+      }
+    }
+  };
+  const unsigned k_lane = (unsigned)(l32 * DK * 2) + 16u * (hf ^ (DK == 128 ? (l32 & 15) : ((l32 >> 1) & 7)));
+  const unsigned v_lane = (unsigned)(l32 * VTP * 2) + 16u * hf;
+
+  // ---- work queues (wave 4 only) -----------------------------------------------------------------------------------
+  const unsigned xcc = xcc_id();
+  int cq = 0;  // queues used up so far; the queue in use is (xcc + cq) & 7
+  unsigned t_ahead = 0;
+  auto queue_units = [&](const unsigned qx) -> unsigned { return qx < n_pairs ? ((n_pairs - qx + 7u) / 8u) * NT : 0u; };
+  auto take_ticket = [&]() -> unsigned {
+    unsigned t = 0;
+    if (lane == 0) t = atomicAdd(&queue[(xcc + (unsigned)cq) & 7u], 1u);
+    return __builtin_amdgcn_readfirstlane(t);
+  };
+  // ticket t of the queue in use -> the tile it stands for, written as the "next tile" part of a record; moves on to the
+  // other queues (one synchronous ticket each) when the queue in use has no tiles left.  Returns the row index of the
+  // tile's first chunk (-1: no tile left).
+  auto resolve_ticket = [&](unsigned t, StreamTile* out) -> int {
+    bool ok = false;
+    unsigned qx = 0;
+    while (cq < STREAM_QUEUES) {
+      qx = (xcc + (unsigned)cq) & 7u;
+      if (t < queue_units(qx)) {
+        ok = true;
+        break;
+      }
+      if (++cq < STREAM_QUEUES) t = take_ticket();
+    }
+    if (!ok) {
+      if (lane == 0) out->valid = 0;
+      return -1;
+    }
+    // Order of a queue: first every pair's NT - NL late (long) tiles, pair after pair, latest tile first; then every
+    // pair's NL early (short) tiles the same way.  With the pairs' tiles simply one after the other, the last pair's
+    // longest tile would start when only that pair's tiles are left, and the other CUs of the XCD idle while it runs.
+    const unsigned NL = NT / 3u, NH = NT - NL, heavy = (queue_units(qx) / NT) * NH;
+    unsigned pidx, tile;
+    if (t < heavy) {
+      pidx = t / NH;
+      tile = NT - 1u - t % NH;
+    } else {
+      pidx = (t - heavy) / NL;   // (NL > 0 here: with NL = 0 every ticket is below `heavy`)
+      tile = NL - 1u - (t - heavy) % NL;
+    }
+    const unsigned pair = pidx * 8u + qx;
+    const unsigned n = pair / (unsigned)p.HQ, hq = pair - n * (unsigned)p.HQ;
+    const unsigned dstart = (tile * QTILE / (unsigned)Bs) * (unsigned)Bs;
+    const unsigned hkv = hq / (unsigned)p.g_kv;
+    if (lane == 0) {
+      out->valid = 1;
+      out->n = (int)n;
+      out->hq = (int)hq;
+      out->tile = (int)tile;
+      out->hkv = (int)hkv;
+      out->hn = (int)(hq / (unsigned)p.g_n);
+      out->dstart = (int)dstart;
+      out->dblk = (int)(dstart / (unsigned)Bs);
+    }
+    return (int)((n * (unsigned)p.T + dstart) * (unsigned)p.HKV + hkv);
+  };
+
+  // ---- state of the tile in work; the kernel starts in a virtual tile (four chunks, nothing to compute) ------------
+  int a = 0;          // which record / list buffer belongs to the tile in work
+  unsigned sp0 = 0;   // stream position of its chunk 0
+  bool cur_real = false;
+  int c_n = 0, c_hq = 0, c_tile = 0, c_hkv = 0, c_hn = 0, dstart = 0, dblk = 0;
+  bool k_req = false;  // the early waves' newest request is a K request that may still be in flight at the next barrier
+  int row_v = 0;       // early waves: row index of the chunk whose K was requested last (its V is requested next)
+  if (wave == 4) {
+    const int r0 = resolve_ticket(take_ticket(), &info[0]);
+    if (lane == 0) {
+      info[0].diag_lo = info[0].diag_hi = 0u;
+      info[0].count[0] = info[0].count[1] = info[0].count[2] = info[0].count[3] = 0;
+    }
+    if (r0 >= 0 && lane < 4) rows[0][4 + lane] = r0 + 64 * lane * p.HKV;   // the virtual tile has four chunks of its own
+  }
+
+  bf16x8 QB[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) QB[s] = bf16x8{};
+  f32x16 acc[VT];
+  float m_ref, l_run, thr;
+
+  // ---- a tile's output.  A lane holds, of its query, value columns 8 rg + 4 hf .. + 3 of every 32-column tile: stored
+  // from there, an instruction would touch 64 separate 16-byte pieces.  The rows go through LDS instead, half of the
+  // columns at a time (a wave's 32 rows x DV/2 columns; 16-byte segments XOR-swizzled by the row), and leave as whole
+  // lines.  The space is a raw V buffer, a quarter of it per wave.  The early waves use, right after their last chunk,
+  // the buffer whose next request (the next tile's chunk 2) they hold back until they are done: a wave's requests go
+  // to the same quarter as its rows, so no barrier is needed.  The late waves use the other buffer, whose contents (the
+  // next tile's chunk 1) all of them have transposed once the hand-over barrier of the next tile is behind them: they
+  // store there, before anything of the new tile touches the accumulators.  row0: flat (token, head) index of the
+  // wave's first query.
+  auto store_tile = [&](const unsigned stage, const size_t row0) __attribute__((always_inline)) {
+    constexpr int PW = DV / 2, RB = PW * 2, NSEG = RB / 16, RPI = 64 / NSEG;   // columns per pass, row bytes, segments, rows per instruction
+    typedef __attribute__((address_space(3))) u32x2* lds_w8;
+    typedef __attribute__((address_space(3))) const u32x4* lds_r16;
+    const float l_tot = xhalf_sum(l_run);
+    const bool has = l_tot > 0.f;
+    const float inv = has ? 1.f / l_tot : 0.f;
+    int ol = lane;
+    asm volatile("" : "+v"(ol));   // (the lane's share of the addresses below is not to be kept through the chunk loops)
+    const int ol32 = ol & 31, ohf = ol >> 5;
+    if (ohf == 0) p.lse[row0 + (size_t)ol32 * p.HQ] = has ? m_ref + __builtin_amdgcn_logf(l_tot) : 0.f;
+    const unsigned wbase = stage + (unsigned)(ol32 * RB + 8 * ohf);
+    const int rrow = ol / NSEG, rseg = ol % NSEG;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+#pragma unroll
+      for (int vl = 0; vl < VT / 2; ++vl) {
+        const int vt = ps * (VT / 2) + vl;
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          u32x2 w;
+          w[0] = pack_bf16x2(acc[vt][4 * rg] * inv, acc[vt][4 * rg + 1] * inv);
+          w[1] = pack_bf16x2(acc[vt][4 * rg + 2] * inv, acc[vt][4 * rg + 3] * inv);
+          *reinterpret_cast<lds_w8>(wbase + 16u * ((unsigned)(4 * vl + rg) ^ (unsigned)(ol32 & (NSEG - 1)))) = w;
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's rows are in LDS
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < 32 / RPI; ++i) {
+        const int row = i * RPI + rrow;
+        const u32x4 w = *reinterpret_cast<lds_r16>(stage + (unsigned)(row * RB) + 16u * ((unsigned)rseg ^ (unsigned)(row & (NSEG - 1))));
+        *reinterpret_cast<u32x4*>(p.o + (row0 + (size_t)row * p.HQ) * DV + ps * PW + rseg * 8) = w;
+      }
+      if (ps == 0) {
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // the rows have been read before the second half overwrites them
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+  };
+  auto scale_next_q = [&]() __attribute__((always_inline)) {
+    const float qscale = p.scale_log2;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const u32x4 w = __builtin_bit_cast(u32x4, QB[s]);
+      u32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = pack_bf16x2(__uint_as_float(w[j] << 16) * qscale, __uint_as_float(w[j] & 0xffff0000u) * qscale);
+      QB[s] = __builtin_bit_cast(bf16x8, r);
+    }
+  };
+  bool pend_store = false;   // late waves: the previous tile's output is still in the accumulators
+  unsigned pend_stage = 0;
+  size_t pend_row0 = 0;
+
+  for (;;) {
+    // ---- hand-over barrier: the record and the list of the tile in work are complete ------------------------------
+    __syncthreads();
+    typedef __attribute__((address_space(3))) const int* lds_i;
+    const unsigned rec = (unsigned)(size_t)&info[a];
+    auto rd = [&](const int i) -> int { return __builtin_amdgcn_readfirstlane(*reinterpret_cast<lds_i>(rec + 4u * i)); };
+    // (one 4-byte read per field: a wider uniform read followed by readfirstlane of its elements was folded into
+    // element 0 by the compiler)
+    const bool n_valid = rd(0) != 0;
+    const int n_n = rd(1), n_hq = rd(2), n_tile = rd(3), n_hkv = rd(4), n_hn = rd(5), n_dstart = rd(6), n_dblk = rd(7);
+    const unsigned long long diag_attn = (unsigned long long)(unsigned)rd(8) | ((unsigned long long)(unsigned)rd(9) << 32);
+    const int n_prior = rd(10) + rd(11) + rd(12) + rd(13);
+    const int tile_start = c_tile * QTILE;
+    const int n_diag = cur_real ? (tile_start + QTILE - dstart) >> 6 : 4;
+    const int n_iters = n_diag + n_prior * per_blk;
+    const int bos = c_n * p.T;
+    const int q0 = tile_start + wave * QW;
+    const int my_chunk = q0 >> 6, qloc0 = q0 & 63;
+    const int my_blk = (int)((unsigned)q0 / (unsigned)Bs);
+    // the tile after this one
+    const int n_bos = n_n * p.T;
+    const int n_tile_start = n_tile * QTILE;
+
+    // queries of the next tile: raw into the query registers (issued during this tile's last chunk), scaled in place
+    auto load_next_q = [&]() __attribute__((always_inline)) {
+      // (lane ids made opaque here and in the output code below: otherwise the lane's share of every such address is
+      // computed once per kernel and kept in registers through the chunk loops)
+      int ql = lane;
+      asm volatile("" : "+v"(ql));
+      // (no next tile: this tile's rows are read again, so that the loads and the waits of the scaling below are on
+      // every path -- with the loads under a condition the compiler assumes them pending wherever the queries are used)
+      const size_t qrow = n_valid ? (size_t)(n_bos + n_tile_start) : (size_t)(bos + tile_start);
+      const bf16_t* qr = p.q + ((qrow + wave * QW + (ql & 31)) * p.HQ + (n_valid ? n_hq : c_hq)) * DK + 8 * (ql >> 5);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) QB[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(qr + 16 * s));
+    };
+
+    if (pend_store) store_tile(pend_stage, pend_row0);
+    scale_next_q();   // the queries requested at the end of the previous tile
+
+    // which of the chunks from dstart on this wave takes part in, and which one is its own, causal chunk
+    unsigned long long act_mask = 0;
+    int causal_it = -1;
+    if (cur_real) {
+      int al = lane;
+      asm volatile("" : "+v"(al));
+      const int jc = (dstart >> 6) + al;
+      const int kblk = (int)((unsigned)(jc * 64) / (unsigned)Bs);
+      const bool typed = (diag_attn >> ((kblk - dblk) & 63)) & 1ull;
+      bool act, cz = false;
+      if (p.same_block) {
+        cz = jc == my_chunk;
+        act = cz || (jc < my_chunk && (kblk == my_blk || typed));
+      } else {
+        act = jc < my_chunk && kblk < my_blk && typed;
+      }
+      act_mask = __ballot(act && al < n_diag);
+      const unsigned long long cm = __ballot(cz && al < n_diag);
+      causal_it = cm ? __builtin_ctzll(cm) : -1;
+    }
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[vt][r] = 0.f;
+    m_ref = 0.f;  // an arbitrary finite reference until the row's first visible key sets the real one
+    l_run = 0.f;
+    thr = -INFINITY;
+    f32x16 s0, s1;
+    auto is_active = [&](const int it) -> bool { return it < n_diag ? (act_mask >> it) & 1ull : it < n_iters; };
+    bool cur_active = act_mask & 1ull;
+    if (cur_active) qk_phase<DK>(lds_k + (sp0 & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
+
+    if (!late) {
+      // Stream chunks requested during this tile: its own from chunk 4 on (chunks 0..3 were requested while the previous
+      // tile ran) and the next tile's first four, all by their entry in this tile's chunk table.
+      // (the V request of the last iteration, the next tile's chunk 2, waits until the output code below is done with
+      // the buffer it goes to)
+      const int rq_lo = cur_real ? 0 : n_iters;
+      const unsigned rq_span = (unsigned)((n_valid ? n_iters + 4 : n_iters) - rq_lo);
+      const unsigned rv_span = (unsigned)((n_valid ? n_iters + 2 : n_iters) - rq_lo);
+      typedef __attribute__((address_space(3))) const int* lds_row;
+      const unsigned row_tab = (unsigned)(size_t)&rows[a][4];
+      for (int it = 0; it < n_iters; ++it) {
+        const bool nxt_active = is_active(it + 1);
+        const int row_ahead = *reinterpret_cast<lds_row>(row_tab + 4u * it);   // chunk it + 4, used after the barrier
+        bf16x8 PB[4];
+        if (cur_active) {
+          softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
+          __builtin_amdgcn_s_setprio(3);
+          pv_phase<DV>(lds_v + ((sp0 + it) % VRING) * VTILE + v_lane, PB, acc, l_run);
+        }
+        __builtin_amdgcn_s_setprio(3);
+        if (nxt_active) qk_phase<DK>(lds_k + ((sp0 + it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
+        __builtin_amdgcn_s_setprio(0);
+        // K(it+2) and raw V(it+2) must have landed; the newest K request, if the last request step made one, may stay
+        // in flight
+        if (k_req) __builtin_amdgcn_s_waitcnt(0x0f70 | KI);
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();                                  // sync(it)
+        // Requests: V(it+3), whose row index was found when its K was requested, then K(it+4).  (As few instructions
+        // as possible: the other wave of the SIMD runs its matrix phases at raised priority meanwhile, and every
+        // instruction of this one waits for an issue slot.)
+        if ((unsigned)(it + 3 - rq_lo) < rv_span) dma_r(row_v, sp0 + it + 3);
+        k_req = (unsigned)(it + 4 - rq_lo) < rq_span;
+        if (k_req) {
+          row_v = __builtin_amdgcn_readfirstlane(row_ahead);
+          dma_k(row_v, sp0 + it + 4);
+        }
+        cur_active = nxt_active;
+      }
+    } else {
+      // What the late waves prepare for the next tile while this one runs: its chunk table (the rows of its own chunks,
+      // then of the prior attention blocks from the sorted list: a thread takes up to four list entries, which covers
+      // the 1024 blocks the launcher admits), how many prior blocks there are, and the types of its own blocks.  Loads
+      // are issued in the first chunk and used in the second, so that no wave waits for memory.
+      const int32_t* n_list = p.idx + ((size_t)(n_n * p.TN) * p.HN + n_hn) * 2;
+      const int jmax = min(n_dblk, p.TN);
+      const int n_ndiag = (n_tile_start + QTILE - n_dstart) >> 6;
+      int pe[4] = {0, 0, 0, 0}, p_nattn = 0;
+      float p_type = 0.f;
+      int ev_it = n_valid ? 0 : -1;
+      // transpositions cover stream chunks tr_lo <= it + 2 < tr_lo + tr_span (this tile's, then the next tile's first two)
+      const int tr_lo = cur_real ? 0 : n_iters;
+      const unsigned tr_span = (unsigned)((n_valid ? n_iters + 2 : n_iters) - tr_lo);
+      for (int it = 0; it < n_iters; ++it) {
+        const bool nxt_active = is_active(it + 1);
+        const bool last = it == n_iters - 1;
+        // Preparation work for the next tile happens in iterations 0, 1, n-2 and n-1 only: `ev_it` is the next of
+        // those, so that an ordinary iteration pays one scalar comparison.
+        if (it == ev_it) {
+          if (it == 0) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              const int j = lt + 256 * m;
+              pe[m] = j < jmax ? n_list[(size_t)j * list_stride] : 0;
+            }
+            p_nattn = p.nblk[((size_t)n_n * p.HN + n_hn) * 2];
+            if (wave == 4) {
+              const int blk = n_dblk + lane;
+              const bool in_range = lane < n_ndiag && (size_t)blk * Bs < (size_t)(n_tile_start + QTILE);
+              const size_t ti = ((size_t)(n_n * p.TN + (in_range ? blk : n_dblk)) * p.HN + n_hn) * 2;
+              p_type = p.types_dtype == NATSL_F32 ? reinterpret_cast<const float*>(p.types)[ti]
+                                                  : bf16_to_f32(reinterpret_cast<const bf16_t*>(p.types)[ti]);
+            }
+          }
+          if (it == 1) {
+            int cnt = 0;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              const int j = lt + 256 * m;
+              const bool ok = j < jmax && j < p_nattn && (pe[m] + 1) * Bs <= n_dstart;
+              cnt += __popcll(__ballot(ok));
+              // (the qualifying entries form a prefix of the list: entry j's chunks follow those of the entries before it)
+              if (ok)
+                for (int sub = 0; sub < per_blk; ++sub)
+                  rows[a ^ 1][n_ndiag + j * per_blk + sub] = (n_bos + pe[m] * Bs + 64 * sub) * p.HKV + n_hkv;
+            }
+            if (lt < n_ndiag) rows[a ^ 1][lt] = (n_bos + n_dstart + 64 * lt) * p.HKV + n_hkv;
+            if (lane == 0) info[a ^ 1].count[gw] = cnt;
+            if (wave == 4) {
+              const int blk = n_dblk + lane;
+              const bool in_range = lane < n_ndiag && (size_t)blk * Bs < (size_t)(n_tile_start + QTILE);
+              const unsigned long long d = __ballot(in_range && rintf(p_type) == 1.0f);
+              if (lane == 0) {
+                info[a ^ 1].diag_lo = (unsigned)d;
+                info[a ^ 1].diag_hi = (unsigned)(d >> 32);
+              }
+            }
+          }
+          if (wave == 4) {
+            // the tile after the next: ticket asked for in the last chunk but one, turned into a tile in the last
+            if (it == n_iters - 2 && cq < STREAM_QUEUES && lane == 0) t_ahead = atomicAdd(&queue[(xcc + (unsigned)cq) & 7u], 1u);
+            if (last) {
+              const int r0 = resolve_ticket(__builtin_amdgcn_readfirstlane(t_ahead), &info[a ^ 1]);
+              // the next tile's table ends with the first four chunks of the tile after it
+              const int nn_iters = n_ndiag + (info[a ^ 1].count[0] + info[a ^ 1].count[1] + info[a ^ 1].count[2] + info[a ^ 1].count[3]) * per_blk;
+              if (r0 >= 0 && lane < 4) rows[a ^ 1][nn_iters + lane] = r0 + 64 * lane * p.HKV;
+            }
+          }
+          ev_it = it == 0 ? 1 : (it < n_iters - 2 ? n_iters - 2 : it + 1);
+        }
+        bf16x8 PB[4];
+        if (cur_active) softmax_phase<DV>(s0, s1, acc, m_ref, l_run, thr, lane, it == causal_it, qloc0, PB);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(PB[i]));   // the probabilities exist before the barrier
+        __syncthreads();                                  // sync(it)
+        __builtin_amdgcn_s_setprio(3);
+        if (cur_active) pv_phase<DV>(lds_v + ((sp0 + it) % VRING) * VTILE + v_lane, PB, acc, l_run);
+        if (nxt_active) qk_phase<DK>(lds_k + ((sp0 + it + 1) & 3) * KTILE + k_lane, QB, m_ref, s0, s1);
+        __builtin_amdgcn_s_setprio(0);
+        if ((unsigned)(it + 2 - tr_lo) < tr_span) transpose_v(sp0 + it + 2);
+        cur_active = nxt_active;
+      }
+    }
+
+    // ---- end of the tile: output (early waves now, late waves after the next hand-over barrier), the request held back,
+    // the next tile's queries
+    {
+      const size_t row0 = (size_t)(bos + q0) * p.HQ + c_hq;
+      const unsigned stage_e = lds_r + ((sp0 + n_iters) & 1) * RTILE + gw * (32 * DV);
+      const unsigned stage_l = lds_r + ((sp0 + n_iters + 1) & 1) * RTILE + gw * (32 * DV);
+      if (!late) {
+        load_next_q();   // (ahead of the stores: what waits for the queries later does not wait for the stores then)
+        if (cur_real) store_tile(stage_e, row0);
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // the staged rows have been read
+        if (!n_valid) break;
+        dma_r(__builtin_amdgcn_readfirstlane(rows[a][n_iters + 2]), sp0 + n_iters + 2);
+        k_req = false;   // the newest request is now a V request: everything has to land before the next barrier but one
+      } else {
+        load_next_q();
+        if (!n_valid) {
+          if (cur_real) store_tile(stage_l, row0);   // (no next tile: nothing was transposed after this tile's own chunks)
+          break;
+        }
+        pend_store = cur_real;
+        pend_stage = stage_l;
+        pend_row0 = row0;
+      }
+    }
+    c_n = n_n; c_hq = n_hq; c_tile = n_tile; c_hkv = n_hkv; c_hn = n_hn; dstart = n_dstart; dblk = n_dblk;
+    cur_real = true;
+    sp0 += (unsigned)n_iters;
+    a ^= 1;
+  }
+
+  // ---- the last workgroup to finish sets the queues back to zero for the next launch --------------------------------
+  if (tid == 0) {
+    __threadfence();
+    const unsigned done = atomicAdd(&queue[STREAM_QUEUES], 1u);
+    if (done == gridDim.x - 1) {
+#pragma unroll
+      for (int i = 0; i <= STREAM_QUEUES; ++i) atomicExch(&queue[i], 0u);
+    }
+  }
+}
+
 template <int DK, int DV, int NWAVES>
 static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   constexpr int KP = DK + 8, VP = DV + 8, QTILE = 32 * NWAVES;
@@ -964,6 +1469,56 @@ static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
                                 : (long long)8 * ((p.B * p.HQ + 7) / 8) * ((p.T + QTILE - 1) / QTILE);
   if (grid <= 0) return NATSL_OK;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NWAVES), lds, stream, p);
+  return check_launch("natsl_softmax_sparse_fwd");
+}
+
+// Ticket counters of the persistent kernel: zero when the library is loaded, and set back to zero by every launch's last
+// workgroup.  Consecutive launches rotate through the slots, so launches that overlap on one GPU (two streams) do not
+// share counters unless STREAM_SLOTS launches lie between them.
+constexpr int STREAM_SLOTS = 64;
+static __device__ __align__(256) unsigned stream_queues[STREAM_SLOTS * STREAM_SLOT_WORDS];
+
+struct StreamDevice {
+  unsigned* queues = nullptr;
+  int cus = 0;
+};
+
+static const StreamDevice* stream_device(int* rc) {
+  constexpr int MAX_DEVICES = 64;
+  static StreamDevice devs[MAX_DEVICES];
+  static std::mutex mu;
+  *rc = NATSL_OK;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    *rc = fail(NATSL_ERR_LAUNCH, "softmax: cannot name the current device (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!devs[dev].queues) {
+    void* a = nullptr;
+    e = hipGetSymbolAddress(&a, HIP_SYMBOL(stream_queues));  // with device `dev` current: that device's copy
+    int cus = 0;
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || !a || cus <= 0) {
+      *rc = fail(NATSL_ERR_LAUNCH, "softmax: cannot set up the work queues on device %d (%s)", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    devs[dev].cus = cus;
+    devs[dev].queues = static_cast<unsigned*>(a);
+  }
+  return &devs[dev];
+}
+
+template <int DK, int DV>
+static int launch_softmax_stream(const SoftmaxParams& p, const StreamDevice* d, hipStream_t stream) {
+  static std::atomic<unsigned> launches{0};
+  const size_t lds = ((size_t)4 * 64 * DK + (size_t)2 * 64 * DV + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;
+  auto kern = softmax_stream_kernel<DK, DV>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+  unsigned* queue = d->queues + (size_t)(launches.fetch_add(1) % STREAM_SLOTS) * STREAM_SLOT_WORDS;
+  hipLaunchKernelGGL(kern, dim3((unsigned)d->cus), dim3(512), lds, stream, p, queue);
   return check_launch("natsl_softmax_sparse_fwd");
 }
 
@@ -1002,9 +1557,20 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   // faster one; below, the 128-query tiles fill more CUs)
   p.variant = (long long)B * HQ * cdiv(T, 256) >= 256 ? 8 : 4;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // Whole 256-query tiles, at least two per CU: the persistent kernel (its per-tile saving needs a tile to follow)
+  const StreamDevice* sd = nullptr;
+  if (!seqs && T % 256 == 0 && T <= 65536 && block <= 2048 && (long long)B * T * HKV < (1ll << 31) &&
+      getenv("NATSL_SOFTMAX_NO_STREAM") == nullptr) {
+    int rc;
+    sd = stream_device(&rc);
+    if (!sd) return rc;
+    if ((long long)B * HQ * (T / 256) < 2ll * sd->cus) sd = nullptr;
+  }
 #define NATSL_SM(KK, VV)                                              \
-  if (K == KK && V == VV)                                             \
-    return p.variant == 8 ? launch_softmax<KK, VV, 8>(p, s) : launch_softmax<KK, VV, 4>(p, s);
+  if (K == KK && V == VV) {                                           \
+    if (sd) return launch_softmax_stream<KK, VV>(p, sd, s);           \
+    return p.variant == 8 ? launch_softmax<KK, VV, 8>(p, s) : launch_softmax<KK, VV, 4>(p, s); \
+  }
   NATSL_SM(128, 128)
   NATSL_SM(64, 64)
   NATSL_SM(64, 128)
