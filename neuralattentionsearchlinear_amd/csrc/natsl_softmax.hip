@@ -1557,6 +1557,8 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   // faster one; below, the 128-query tiles fill more CUs)
   p.variant = (long long)B * HQ * cdiv(T, 256) >= 256 ? 8 : 4;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (!((K == 64 || K == 128) && (V == 64 || V == 128)))
+    return fail(NATSL_ERR_UNSUPPORTED, "softmax: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", K, V);
   // Whole 256-query tiles, at least two per CU: the persistent kernel (its per-tile saving needs a tile to follow)
   const StreamDevice* sd = nullptr;
   if (!seqs && T % 256 == 0 && T <= 65536 && block <= 2048 && (long long)B * T * HKV < (1ll << 31) &&
