@@ -404,7 +404,7 @@ def main():
                     launch_ms_alone=lin_alone_ms)
     if f_attn >= f_gdn:
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", kernel="softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
+        roof = dict(bound="mfma", kernel="softmax_stream_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
                     unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=(traffic or {}).get("softmax_bytes"),
                     traffic_source=traffic_source, launch_ms=sm_ms, algorithmic_flops=f_attn,
                     # the same kernel with the GPU to itself (branches launched one after the other, outside the timed region)
