@@ -96,7 +96,12 @@ int natsl_route(const void* types, int types_dtype, int B, int TN, int HN, int T
  * q [B,T,HQ,K], k [B,T,HKV,K], v [B,T,HKV,V] -> o [B,T,HQ,V] (same dtype), lse [B,T,HQ] fp32 in
  * log2 units; rows that see no key give o = 0, lse = 0.
  * Replaces parallel_attn_nats_fwd (src/nats/ops/attns/attns.py:1421-1531, kernel :62-353) as
- * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:111-117. */
+ * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:111-117.
+ * K, V in {64, 128}.  Unpacked input of whole 256-query tiles, at least two per compute unit (T % 256 == 0,
+ * T <= 65536, block <= 2048), runs as a persistent kernel whose work queues are ticket counters in device
+ * memory owned by the library (64 slots in rotation, each launch sets its slot back to zero): launches may
+ * overlap across streams; NATSL_SOFTMAX_NO_STREAM=1 in the environment selects the per-tile kernel, whose
+ * results are the same bit for bit. */
 int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                              const void* types, int types_dtype, const int32_t* nats_block_indices,
                              const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
