@@ -98,3 +98,39 @@ def test_mamba(K, V, block, decay):
 
 def test_mamba_ragged():
     _mamba(1, 333, 2, 2, 128, 64, 64, 0.3, True, seed=11)
+
+
+# ---- the 760M configuration's head geometry: key dim 192, value dim 384 (reference experiments/configs/natsl_760M.json) ----
+@pytest.mark.parametrize("decay", [True, False])
+def test_gdn_key_dim_192(decay):
+    _gdn(2, 512, 4, 2, 192, 384, 64, 0.4, decay, seed=20, h0=True)
+
+
+def test_gdn_key_dim_192_other_shapes():
+    _gdn(1, 300, 2, 2, 192, 192, 128, 0.5, True, seed=21)            # ragged, block of two chunks
+    _gdn(1, 512, 2, 2, 192, 48, 64, 0.3, True, seed=22, l2=False)    # narrow value dim
+
+
+def test_mamba_key_dim_192():
+    _mamba(2, 512, 4, 2, 192, 384, 64, 0.3, True, seed=23, h0=True)
+
+
+# ---- the scan's three workgroup widths: 64 columns when that still gives one workgroup per CU, else 32, else 16; the small
+# shapes above all take 16 ----
+def _cus():
+    return torch.cuda.get_device_properties(0).multi_processor_count
+
+
+def test_gdn_scan_with_32_columns_per_workgroup():
+    B, H, V = 4, 16, 128
+    assert B * H * (V // 32) >= _cus() > B * H * (V // 64)
+    _gdn(B, 320, H, 8, 128, V, 64, 0.4, True, seed=24, h0=True)
+    _gdn(4, 256, 6, 3, 192, 384, 64, 0.4, True, seed=25)             # key dim 192 never takes 64 columns
+
+
+def test_gdn_and_mamba_scan_with_64_columns_per_workgroup():
+    B, H, V = 8, 16, 128
+    assert B * H * (V // 64) >= _cus()
+    _gdn(B, 320, H, 16, 128, V, 64, 0.3, True, seed=26, h0=True)
+    _gdn(B, 256, H, 4, 64, V, 128, 0.5, False, seed=27)
+    _mamba(B, 256, H, 8, 128, V, 64, 0.3, True, seed=28, h0=True)
