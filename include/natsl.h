@@ -112,9 +112,11 @@ int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* 
 /* Backward of the softmax branch: dq [B,T,HQ,K], dk [B,T,HKV,K], dv [B,T,HKV,V] (bf16, summed over the query heads of
  * a kv head) and dnats fp32 [B,TN,HQ], which must be ZERO on entry: per block typed "attention" and query head, the sum
  * of the score gradients dS = P (dP - delta) over (keys of the block) x (queries of later blocks), i.e. the gradient
- * with respect to a bias on that block's scores as later blocks see them; blocks not typed attention keep 0 (the
- * reference's default compute_dnats_for_invalid_blocks_attn = False).  The caller sums dnats over the query heads of a
- * selector head.  o, lse are the forward's outputs, d_o the gradient of o.  workspace: natsl_softmax_bwd_workspace_bytes()
+ * with respect to a bias on that block's scores as later blocks see them; blocks not typed attention keep 0 unless
+ * flags bit 1 is set (the reference's compute_dnats_for_invalid_blocks_attn, attns.py:1318-1325): then they get
+ * sum min(exp2(s - lse), 1) (dP - delta) over the same (keys) x (later queries), what their keys would contribute if
+ * they were visible.  flags bit 0: same_block_visible, as in the forward.  The caller sums dnats over the query heads
+ * of a selector head.  o, lse are the forward's outputs, d_o the gradient of o.  workspace: natsl_softmax_bwd_workspace_bytes()
  * bytes (delta = rowsum(d_o * o), then the work-queue counters of the dk/dv kernel; nothing to initialise: every call resets
  * them, so calls that share a workspace must not overlap).  T * HQ * max(K, V) * 2 must stay below 2^32 (32-bit row offsets
  * within a sequence).  Regular batches only (no packed-sequence table yet).
@@ -124,7 +126,7 @@ size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ);
 int natsl_softmax_sparse_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* d_o,
                              void* dq, void* dk, void* dv, float* dnats, const void* types, int types_dtype,
                              const int32_t* nats_block_indices, const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV,
-                             int HN, int K, int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                             int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
                              void* workspace, size_t workspace_bytes, natsl_stream_t stream);
 
 /* Bytes of scratch the two linear-branch entry points need for `total_chunks` 64-token chunks

@@ -57,12 +57,11 @@ def parallel_attn_nats_bwd(
     -> (dq [B,T,HQ,K], dk [B,T,H,K], dv [B,T,H,V], None, dnats [B,TNAtS,HNAtS]).
 
     dnats holds, per block typed attention, the summed score gradient of later blocks' queries on its keys (the
-    straight-through gradient of the selector, attns.py:946-961) and 0 for the other blocks; asking for the invalid
-    blocks' gradient too, packed sequences, g_cumsum and sliding windows are not built."""
+    straight-through gradient of the selector, attns.py:946-961); the other blocks get 0, or, with
+    compute_dnats_for_invalid_blocks_attn, what their keys would contribute if they were visible (probabilities against
+    the queries' lse, clamped to 1: attns.py:1318-1325).  Packed sequences, g_cumsum and sliding windows are not built."""
     if g_cumsum is not None or sliding_window_size is not None or not is_causal or OFFSET_ATTN != 0:
         raise NotImplementedError("only the causal backward without g_cumsum / sliding window is built")
-    if compute_dnats_for_invalid_blocks_attn:
-        raise NotImplementedError("compute_dnats_for_invalid_blocks_attn=True is not built")
     if cu_seqlens is not None or cu_seqlens_nats is not None:
         raise NotImplementedError("packed sequences are not supported by the softmax backward yet")
     if scale is None:
@@ -83,7 +82,8 @@ def parallel_attn_nats_bwd(
         _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(o), _capi.ptr(lse.contiguous()), _capi.ptr(do), _capi.ptr(dq),
         _capi.ptr(dk), _capi.ptr(dv), _capi.ptr(dnats), _capi.ptr(ty), _capi.dtype_code(ty.dtype), _capi.ptr(nats_block_indices),
         _capi.ptr(n_nats_blocks), B, T, HQ, H, HN, K, V, TN, NAtS_block_size, float(scale),
-        int(bool(compute_incomplete_chunk_scores)), _capi.dtype_code(q.dtype), _capi.ptr(ws), ws_bytes, _capi.stream_ptr(q.device))
+        int(bool(compute_incomplete_chunk_scores)) | (2 if compute_dnats_for_invalid_blocks_attn else 0), _capi.dtype_code(q.dtype),
+        _capi.ptr(ws), ws_bytes, _capi.stream_ptr(q.device))
     _capi.check(rc, "natsl_softmax_sparse_bwd")
     dnats = dnats.view(B, TN, HN, HQ // HN).sum(-1)          # over the query heads of a selector head (attns.py:1755)
     return dq, dk, dv, None, dnats

@@ -32,6 +32,7 @@ struct SoftmaxBwdParams {
   int B, T, HQ, HKV, HN, TN, block;
   float scale, scale_log2;
   int same_block;
+  int dnats_invalid;   // also give dnats to blocks that are not typed attention (what their keys would contribute, reference attns.py:1318-1325)
 };
 
 NATSL_DEVICE bool bwd_type_is_one(const void* types, int dtype, size_t i) {
@@ -533,7 +534,10 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
     const int hq = hkv * G + g, hn = hq / GN;
     const bool attn = bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + kb) * p.HN + hn) * 2);
     const int n_same = p.same_block ? blk_end_chunk - jc : 0;
-    const int n_later = __builtin_amdgcn_readfirstlane(attn ? max(NTc - blk_end_chunk, 0) : 0);   // (the type was read by a vector load)
+    // a block that is not typed attention walks the later queries only when its dnats is asked for, and then for nothing else
+    const bool walk_later = attn || p.dnats_invalid != 0;
+    const int n_later = __builtin_amdgcn_readfirstlane(walk_later ? max(NTc - blk_end_chunk, 0) : 0);   // (the type was read by a vector load)
+    const bool attn_u = __builtin_amdgcn_readfirstlane(attn ? 1 : 0) != 0;
     const int n_it = n_same + n_later;
     float dn = 0.f;
     auto chunk_of = [&](const int it) { return it < n_same ? jc + it : NTc - 1 - (it - n_same); };
@@ -648,11 +652,15 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
       __builtin_amdgcn_sched_barrier(0);
       f32x16 pr, ds;
       const bool own = jq == jc;
+      // keys the queries do not see: probabilities against the queries' lse, clamped to 1 as the reference does, enter
+      // dnats only (their dV, dK products run on zeros)
+      const bool only_dn = !attn_u && it >= n_same;
       float dsum = 0.f;
       if (!own && jq * 64 + 64 <= len) {   // every (query, key) pair of the tile is visible: no masks
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[r >> 2][r & 3]));
+          float e = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[r >> 2][r & 3]));
+          if (only_dn) e = fminf(e, 1.f);
           pr[r] = e;
           ds[r] = e * (dp[r] - d4[r >> 2][r & 3]);
           dsum += ds[r];
@@ -665,7 +673,8 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
             const int r = 4 * rg + j;
             const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
             const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
-            const float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[rg][j])) : 0.f;
+            float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[rg][j])) : 0.f;
+            if (only_dn) e = fminf(e, 1.f);
             pr[r] = e;
             ds[r] = e * (dp[r] - d4[rg][j]);
             dsum += ds[r];
@@ -676,6 +685,10 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
       bf16x8 PB[2][2];
 #pragma unroll
       for (int ss = 0; ss < 2; ++ss) { PB[ss][0] = pack8(pr, ss); PB[ss][1] = pack8(ds, ss); }
+      if (only_dn) {
+#pragma unroll
+        for (int ss = 0; ss < 2; ++ss) PB[ss][0] = PB[ss][1] = bf16x8{};
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < N2; ++j) {
@@ -845,9 +858,10 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
                                         const void* d_o, void* dq, void* dk, void* dv, float* dnats, const void* types,
                                         int types_dtype, const int32_t* nats_block_indices, const int32_t* n_nats_blocks,
                                         int B, int T, int HQ, int HKV, int HN, int K, int V, int TN, int block, float scale,
-                                        int same_block_visible, int dtype, void* workspace, size_t workspace_bytes,
+                                        int flags, int dtype, void* workspace, size_t workspace_bytes,
                                         natsl_stream_t stream) {
   const char* what = "natsl_softmax_sparse_bwd";
+  const int same_block_visible = flags & 1;
   if (!q || !k || !v || !o || !lse || !d_o || !dq || !dk || !dv || !dnats || !types || !nats_block_indices || !n_nats_blocks)
     return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
@@ -870,6 +884,7 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
   p.types = types; p.types_dtype = types_dtype; p.idx = nats_block_indices; p.nblk = n_nats_blocks;
   p.B = B; p.T = T; p.HQ = HQ; p.HKV = HKV; p.HN = HN; p.TN = TN; p.block = block;
   p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f; p.same_block = same_block_visible ? 1 : 0;
+  p.dnats_invalid = (flags & 2) ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define NATSL_SB(KK, VV) \
   if (K == KK && V == VV) return launch_bwd<KK, VV>(p, s);

@@ -106,7 +106,8 @@ def flops(types: torch.Tensor, T: int, block: int, K: int, V: int, heads_per_sel
     return 2.0 * (K + V) * tot * heads_per_selector
 
 
-def softmax_branch_bwd(q, k, v, types, do, scale, block, same_block_visible=True, dtype=torch.float64, with_magnitude=False):
+def softmax_branch_bwd(q, k, v, types, do, scale, block, same_block_visible=True, dtype=torch.float64, with_magnitude=False,
+                       dnats_invalid=False, clamp_invalid=True):
     """Gradients of the softmax branch in closed form (parallel_attn_nats_bwd, src/nats/ops/attns/attns.py:1562-1759;
     kernels :383-708 for dq, :719-983 for dk, dv and dnats):
         P = softmax(masked scores), delta = rowsum(dO * O) (:357-372), dP = dO V^T, dS = P * (dP - delta)
@@ -116,6 +117,11 @@ def softmax_branch_bwd(q, k, v, types, do, scale, block, same_block_visible=True
         selector head hn, for blocks typed attention (:946-961, :1755); 0 for the other blocks (the default
         compute_dnats_for_invalid_blocks_attn=False).  It is the gradient with respect to a bias added to the
         (natural-log scale) scores of a block's keys as later blocks see them.
+        dnats_invalid (compute_dnats_for_invalid_blocks_attn=True, :1318-1325): a block that is NOT typed attention gets
+        sum min(exp(s - lse), 1) (dP - delta) over the same (keys) x (later queries) instead of 0: the score gradient its
+        keys would have if they were visible, with the probabilities taken against the lse of what the query does see and
+        clamped to 1.  (A query that sees nothing has lse = 0 here, as the forward kernel reports it; the reference leaves
+        that case undefined.)  For a block that is typed attention the expression equals dS, which is how it is pinned.
     -> (dq [B,T,HQ,K], dk [B,T,HKV,K], dv [B,T,HKV,V], dnats [B,NB,HN]); with_magnitude adds the same sums over |dS|
     (the scale rounding errors of dnats are measured against: the signed sums cancel, down to exactly 0 when a query
     sees a single earlier block and nothing else).
@@ -153,6 +159,16 @@ def softmax_branch_bwd(q, k, v, types, do, scale, block, same_block_visible=True
             inter = ds * later                                                  # [query, key]
             per_block = torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter.sum(0))
             dnats[b, :, hn] += per_block * a[b, :, hn].to(dtype)
+            if dnats_invalid:
+                s_all = (qq @ kk.T) * scale
+                lse = torch.where(valid, torch.logsumexp(torch.where(valid, s, torch.zeros_like(s)), -1, keepdim=True), torch.zeros_like(delta))
+                p1 = torch.exp(s_all - lse)
+                if clamp_invalid:   # (False only in the test that pins the unclamped expression as an exact derivative)
+                    p1 = p1.clamp(max=1.0)
+                inter1 = p1 * (dd @ vv.T - delta) * later
+                per_block1 = torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter1.sum(0))
+                dnats[b, :, hn] += per_block1 * (1 - a[b, :, hn].to(dtype))
+                dnats_mag[b, :, hn] += torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter1.abs().sum(0)) * (1 - a[b, :, hn].to(dtype))
             dnats_mag[b, :, hn] += torch.zeros(NB, dtype=dtype).index_add_(0, blk, inter.abs().sum(0)) * a[b, :, hn].to(dtype)
     if with_magnitude:
         return dq, dk, dv, dnats, dnats_mag

@@ -17,21 +17,23 @@ def _close(a, b, what):
     assert rl <= 5e-3 and ma <= 2e-2 * max(top, 1.0), f"{what}: rel-L2 {rl:.3e}, max-abs {ma:.3e} (largest reference value {top:.3e})"
 
 
-def _run(B, T, HQ, H, HN, K, V, block, p_attn, same_block, seed, through_autograd=False):
+def _run(B, T, HQ, H, HN, K, V, block, p_attn, same_block, seed, through_autograd=False, dnats_invalid=False):
     from neuralattentionsearchlinear_amd import nats_util
     from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_bwd, parallel_attn_nats_fwd, parallel_nats_attn
     q, k, v = make_qkv(B, T, H, K, V, seed, HQ=HQ)
     do = torch.randn(B, T, HQ, V, generator=torch.Generator().manual_seed(seed + 7)).bfloat16()
     ty = make_types(B, -(-T // block), HN, p_attn, seed + 1, torch.bfloat16)
     scale = K ** -0.5
-    dq_r, dk_r, dv_r, dn_r, dn_mag = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block, with_magnitude=True)
+    dq_r, dk_r, dv_r, dn_r, dn_mag = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block, with_magnitude=True,
+                                                           dnats_invalid=dnats_invalid)
     qd, kd, vd, dod, tyd = (t.to(DEV) for t in (q, k, v, do, ty))
     r = nats_util.route(tyd, T, block)
     if through_autograd:
         qd, kd, vd = (t.requires_grad_() for t in (qd, kd, vd))
         tyd = tyd.requires_grad_()
         o, _ = parallel_nats_attn(qd, kd, vd, None, tyd, r['nats_block_indices'], r['n_nats_blocks'], scale,
-                                  NAtS_block_size=block, compute_incomplete_chunk_scores=same_block)
+                                  NAtS_block_size=block, compute_incomplete_chunk_scores=same_block,
+                                  compute_dnats_for_invalid_blocks_attn=dnats_invalid)
         o.backward(dod)
         dq, dk, dv, dn = qd.grad, kd.grad, vd.grad, tyd.grad[..., 0]
         assert float(tyd.grad[..., 1:].abs().max()) == 0.0
@@ -39,7 +41,8 @@ def _run(B, T, HQ, H, HN, K, V, block, p_attn, same_block, seed, through_autogra
         o, lse, _ = parallel_attn_nats_fwd(qd, kd, vd, tyd, r['nats_block_indices'], None, scale, block,
                                            compute_incomplete_chunk_scores=same_block, n_nats_blocks=r['n_nats_blocks'])
         dq, dk, dv, _, dn = parallel_attn_nats_bwd(qd, kd, vd, o, tyd, r['nats_block_indices'], r['n_nats_blocks'], None, lse, dod,
-                                                   scale=scale, NAtS_block_size=block, compute_incomplete_chunk_scores=same_block)
+                                                   scale=scale, NAtS_block_size=block, compute_incomplete_chunk_scores=same_block,
+                                                   compute_dnats_for_invalid_blocks_attn=dnats_invalid)
     torch.cuda.synchronize()
     _close(dq.float(), dq_r, "dq")
     _close(dk.float(), dk_r, "dk")
@@ -49,7 +52,8 @@ def _run(B, T, HQ, H, HN, K, V, block, p_attn, same_block, seed, through_autogra
     err = (dn.float().cpu().double() - dn_r).abs()
     assert bool((err <= 2e-3 * dn_mag + 1e-6).all()), f"dnats: error {float(err.max()):.3e} against a magnitude of {float(dn_mag.max()):.3e}"
     lin = torch.round(ty[..., 0].float()) == 0
-    assert float(dn.float().cpu()[lin].abs().max() if lin.any() else 0.0) == 0.0, "blocks not typed attention get no gradient"
+    if not dnats_invalid:
+        assert float(dn.float().cpu()[lin].abs().max() if lin.any() else 0.0) == 0.0, "blocks not typed attention get no gradient"
 
 
 @pytest.mark.parametrize("same_block", [True, False])
@@ -127,3 +131,17 @@ def test_softmax_bwd_repeatable_and_workspace_reuse():
         for name, a, b in zip(("dq", "dk", "dv"), outs[0], outs[rep]):
             assert torch.equal(a, b), f"{name} differs between launches 0 and {rep}"
         assert float((outs[0][3] - outs[rep][3]).abs().max()) <= 1e-3 * float(outs[0][3].abs().max() + 1.0)
+
+
+@pytest.mark.parametrize("same_block", [True, False])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 128)])
+def test_softmax_bwd_dnats_of_blocks_that_are_not_attention(K, V, same_block):
+    """compute_dnats_for_invalid_blocks_attn=True: every block gets a selector gradient; dq, dk, dv are unchanged."""
+    _run(2, 512, 4, 4, 4, K, V, 64, 0.4, same_block, seed=20, dnats_invalid=True)
+
+
+def test_softmax_bwd_dnats_of_blocks_that_are_not_attention_other_shapes():
+    _run(1, 768, 8, 4, 2, 128, 128, 128, 0.5, True, seed=21, dnats_invalid=True)          # grouped heads, two chunks per block
+    _run(2, 600, 2, 2, 2, 64, 64, 64, 0.3, True, seed=22, dnats_invalid=True)             # ragged
+    _run(1, 512, 2, 2, 2, 128, 128, 64, 0.0, True, seed=23, dnats_invalid=True)           # nothing typed attention
+    _run(2, 512, 4, 4, 4, 128, 128, 64, 0.4, True, seed=24, through_autograd=True, dnats_invalid=True)

@@ -247,6 +247,74 @@ def test_softmax_backward_closed_form_equals_autograd(same_block):
         assert float((got - want).abs().max()) < 1e-9, name
 
 
+@pytest.mark.parametrize("same_block", [True, False])
+def test_softmax_backward_dnats_of_blocks_that_are_not_attention(same_block):
+    """compute_dnats_for_invalid_blocks_attn: a block that is not typed attention gets sum min(exp(s - lse), 1) (dP - delta)
+    over its keys and the later queries.  Without the clamp that is an exact derivative: give the block's keys the weight
+    eps * exp(s) in the softmax of later queries, and differentiate the loss with respect to eps at eps = 0 (autograd
+    below, against the oracle with its clamp switched off); the clamped expression is checked against plain loops (a
+    query at the start of its block sees few keys, so earlier keys do exceed its lse)."""
+    from oracle import softmax_branch as sb
+    from tests._util import make_types
+    torch.manual_seed(5)
+    B, T, HQ, HKV, HN, K, V, block = 1, 200, 4, 2, 2, 16, 8, 64
+    NB = -(-T // block)
+    ty = make_types(B, NB, HN, 0.4, 6, force_last=False)
+    a = torch.round(ty[..., 0]).double()
+    blk = torch.arange(T) // block
+    later = (blk.view(-1, 1) > blk.view(1, -1)).double()
+    for big in (False, True):
+        q = torch.randn(B, T, HQ, K, dtype=torch.float64) * (6.0 if big else 0.3)
+        k = torch.randn(B, T, HKV, K, dtype=torch.float64)
+        v = torch.randn(B, T, HKV, V, dtype=torch.float64)
+        do = torch.randn(B, T, HQ, V, dtype=torch.float64)
+        scale = K ** -0.5
+        *_, dn0 = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block)
+        *_, dn1 = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block, dnats_invalid=True)
+        assert torch.equal(dn1 * a, dn0 * a), "attention-typed blocks keep their dnats"
+        if not big:
+            eps = torch.zeros(B, NB, HQ, dtype=torch.float64, requires_grad=True)
+            loss = 0
+            for hq in range(HQ):
+                hn, hk = hq // (HQ // HN), hq // (HQ // HKV)
+                m = sb.visibility_mask(a[0, :, hn], T, block, same_block).double()
+                e = torch.exp((q[0, :, hq] @ k[0, :, hk].T) * scale)
+                w = e * m + e * later * ((1 - a[0, :, hn]) * eps[0, :, hq])[blk].view(1, -1)
+                z = w.sum(-1, keepdim=True)
+                seen = m.sum(-1, keepdim=True) > 0
+                p = torch.where(seen, w / torch.where(seen, z, torch.ones_like(z)), torch.zeros_like(w))
+                loss = loss + ((p @ v[0, :, hk]) * do[0, :, hq]).sum()
+            want = torch.autograd.grad(loss, eps)[0].view(B, NB, HN, HQ // HN).sum(-1) * (1 - a)
+            *_, dn_free = sb.softmax_branch_bwd(q, k, v, ty, do, scale, block, same_block, dnats_invalid=True, clamp_invalid=False)
+            got = dn_free * (1 - a)
+            if same_block:   # (a query that sees nothing has no normaliser: the oracle then uses lse = 0, the gate form 0)
+                assert float((got - want).abs().max()) < 1e-9
+            else:
+                rows_seen = torch.stack([sb.visibility_mask(a[0, :, hn], T, block, same_block).any(-1) for hn in range(HN)])
+                assert not bool(rows_seen.all()), "the case is meant to hold queries that see nothing"
+        else:
+            want = torch.zeros(B, NB, HN, dtype=torch.float64)
+            clamped = 0
+            for hq in range(HQ):
+                hn, hk = hq // (HQ // HN), hq // (HQ // HKV)
+                m = sb.visibility_mask(a[0, :, hn], T, block, same_block)
+                s = (q[0, :, hq] @ k[0, :, hk].T) * scale
+                for t in range(T):
+                    vis = m[t]
+                    lse = torch.logsumexp(s[t][vis], 0) if bool(vis.any()) else torch.zeros((), dtype=torch.float64)
+                    pv = torch.exp(s[t][vis] - lse) if bool(vis.any()) else torch.zeros(0, dtype=torch.float64)
+                    o_t = pv @ v[0, vis, hk] if bool(vis.any()) else torch.zeros(V, dtype=torch.float64)
+                    delta = (do[0, t, hq] * o_t).sum()
+                    for j in range(int(blk[t])):
+                        if a[0, j, hn] == 0:
+                            ks = slice(j * block, min((j + 1) * block, T))
+                            p1 = torch.exp(s[t, ks] - lse)
+                            clamped += int((p1 > 1).sum())
+                            want[0, j, hn] += (p1.clamp(max=1.0) * (v[0, ks, hk] @ do[0, t, hq] - delta)).sum()
+            assert clamped > 0, "the case is meant to need the clamp"
+            assert float((dn1 * (1 - a) - want).abs().max()) < 1e-8 * float(want.abs().max())
+
+
 # --------------------------------------------------------------------------------------------
 # gradients of the linear branches (the oracle of the mixed operators' backward)
 # --------------------------------------------------------------------------------------------
