@@ -119,7 +119,8 @@ int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* 
  * of a selector head.  o, lse are the forward's outputs, d_o the gradient of o.  workspace: natsl_softmax_bwd_workspace_bytes()
  * bytes (delta = rowsum(d_o * o), then the work-queue counters of the dk/dv kernel; nothing to initialise: every call resets
  * them, so calls that share a workspace must not overlap).  T * HQ * max(K, V) * 2 must stay below 2^32 (32-bit row offsets
- * within a sequence).  Regular batches only (no packed-sequence table yet).
+ * within the input).  Packed sequences: B = 1 and `seqs` as in the forward, with total_qtiles the table's count of
+ * 256-query tiles and total_chunks its count of 64-token chunks (n_nats_blocks is [n_seqs,HN,2]); else null, 0, 0, 0.
  * Replaces parallel_attn_nats_bwd (src/nats/ops/attns/attns.py:1562-1759; kernels :357-372, :383-708, :719-983) as
  * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:226-243. */
 size_t natsl_softmax_bwd_workspace_bytes(int B, int T, int HQ);
@@ -127,7 +128,8 @@ int natsl_softmax_sparse_bwd(const void* q, const void* k, const void* v, const 
                              void* dq, void* dk, void* dv, float* dnats, const void* types, int types_dtype,
                              const int32_t* nats_block_indices, const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV,
                              int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
-                             void* workspace, size_t workspace_bytes, natsl_stream_t stream);
+                             void* workspace, size_t workspace_bytes, const natsl_seq_row* seqs, int n_seqs,
+                             int total_qtiles, int total_chunks, natsl_stream_t stream);
 
 /* Bytes of scratch the two linear-branch entry points need for `total_chunks` 64-token chunks
  * (sum over sequences of ceil(len/64)) and H heads. */

@@ -193,7 +193,8 @@ class _MixedFunction(torch.autograd.Function):
         with torch.no_grad():
             o_lin, o_attn, ht, aux = _mixed_forward_impl(
                 cfg['kind'], q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
-                cfg['scale_attn'], cfg['scale_lattn'], None, None, cfg['block'], None, cfg['attn_same_block'], cfg['lin_intra'],
+                cfg['scale_attn'], cfg['scale_lattn'], cfg['cu_seqlens'], cfg['cu_seqlens_nats'], cfg['block'], None,
+                cfg['attn_same_block'], cfg['lin_intra'],
                 cfg['output_final_state'], cfg['decay_non_linear'], True, False, cfg['qk_l2norm'], return_aux=True)
         ctx.cfg = cfg
         ctx.in_dtypes = tuple(None if t is None else t.dtype for t in (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
@@ -217,23 +218,42 @@ class _MixedFunction(torch.autograd.Function):
         beta = beta if beta.numel() else None
         h0 = h0 if ctx.has_h0 else None
         B, NB, HN, _ = types.shape
+        seqs = pack_sequences(cfg['cu_seqlens'], cfg['cu_seqlens_nats'], cfg['block'], types.device)
         if do_attn is not None:
             dq_a, dk_a, dv_a, _, dn_attn = parallel_attn_nats_bwd(
                 q_a, k_a, v_a, o_attn, types, idx, nblk, None, lse, do_attn.to(torch.bfloat16).contiguous(), scale=cfg['scale_attn'],
                 NAtS_block_size=cfg['block'], compute_incomplete_chunk_scores=cfg['attn_same_block'],
-                compute_dnats_for_invalid_blocks_attn=cfg['dnats_invalid_attn'])
+                compute_dnats_for_invalid_blocks_attn=cfg['dnats_invalid_attn'], seqs=seqs)
         else:
             dq_a, dk_a, dv_a = torch.zeros_like(q_a), torch.zeros_like(k_a), torch.zeros_like(v_a)
             dn_attn = torch.zeros(B, NB, HN, dtype=torch.float32, device=types.device)
         if do_lin is None:
             do_lin = torch.zeros(*q_l.shape[:3], v_l.shape[-1], dtype=torch.float32, device=q_l.device)
-        dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
-            cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, cfg['scale_lattn'], cfg['block'], cfg['decay_non_linear'],
-            cfg['qk_l2norm'], cfg['lin_intra'], do_lin, dht, cfg['dnats_invalid_linear'])
+        lin_args = (cfg['scale_lattn'], cfg['block'], cfg['decay_non_linear'], cfg['qk_l2norm'], cfg['lin_intra'])
+        if seqs is None:
+            dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
+                cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, *lin_args, do_lin, dht, cfg['dnats_invalid_linear'])
+        else:
+            # packed sequences: each sequence is its own chain (own initial state, own blocks)
+            parts = []
+            for i in range(seqs.n_seqs):
+                a, b = seqs.cu_seqlens[i], seqs.cu_seqlens[i + 1]
+                na, nb_ = seqs.cu_seqlens_nats[i], seqs.cu_seqlens_nats[i + 1]
+                parts.append(linear_chunk_backward(
+                    cfg['kind'], q_l[:, a:b], k_l[:, a:b], v_l[:, a:b], g[:, a:b], None if beta is None else beta[:, a:b],
+                    None if h0 is None else h0[i:i + 1], types[:, na:nb_], *lin_args, do_lin[:, a:b],
+                    None if dht is None else dht[i:i + 1], cfg['dnats_invalid_linear']))
+            cat = lambda j, dim: None if parts[0][j] is None else torch.cat([p[j] for p in parts], dim)
+            dq_l, dk_l, dv_l, dg, dbeta, dn_lin = cat(0, 1), cat(1, 1), cat(2, 1), cat(3, 1), cat(4, 1), cat(6, 1)
+            dh0 = cat(5, 0)
         d_types = torch.stack([dn_attn.float(), dn_lin.float()], -1)
         grads = [dq_a, dk_a, dv_a, dq_l, dk_l, dv_l, dh0, dg, dbeta, d_types]
         grads = [None if (t is None or dt is None) else t.to(dt) for t, dt in zip(grads, ctx.in_dtypes)]
         return (None, *grads)
+
+
+def _host_list(x):
+    return None if x is None else [int(t) for t in (x.tolist() if torch.is_tensor(x) else x)]
 
 
 def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
@@ -251,12 +271,11 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
                                    attn_sw_size, attn_same_block, lin_intra, output_final_state, decay_non_linear,
                                    incomplete_block_start_with_ht, use_g_for_attn, qk_l2norm, inference, op_type_last_chunk,
                                    n_tokens_in_current_block)
-    if cu_seqlens is not None or cu_seqlens_nats is not None:
-        raise NotImplementedError("packed sequences are not supported by the backward yet")
     if attn_sw_size is not None or use_g_for_attn or not incomplete_block_start_with_ht:
         raise NotImplementedError("attn_sw_size / use_g_for_attn / incomplete_block_start_with_ht=False are not built")
     cfg = dict(kind=kind, scale_attn=float(scale_attn), scale_lattn=float(scale_lattn), block=int(nats_block_size),
                attn_same_block=bool(attn_same_block), lin_intra=bool(lin_intra), output_final_state=bool(output_final_state),
                decay_non_linear=bool(decay_non_linear), qk_l2norm=bool(qk_l2norm), dnats_invalid_attn=bool(dnats_invalid_attn),
-               dnats_invalid_linear=bool(dnats_invalid_linear))
+               dnats_invalid_linear=bool(dnats_invalid_linear), cu_seqlens=_host_list(cu_seqlens),
+               cu_seqlens_nats=_host_list(cu_seqlens_nats))
     return _MixedFunction.apply(cfg, *tensors)

@@ -30,6 +30,8 @@ struct SoftmaxBwdParams {
   const int32_t* idx;
   const int32_t* nblk;
   int B, T, HQ, HKV, HN, TN, block;
+  const SeqRow* seqs;   // packed sequences (B = 1): one row per sequence, else null
+  int n_seqs, total_tiles, total_chunks;   // packed: 256-query table tiles and 64-token chunks over all sequences
   float scale, scale_log2;
   int same_block;
   int dnats_invalid;   // also give dnats to blocks that are not typed attention (what their keys would contribute, reference attns.py:1318-1325)
@@ -151,14 +153,33 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hf = lane >> 5;
-  const int nq_tiles = (p.T + QTILE - 1) / QTILE;
-  // every 8th block index lands on the same XCD: an XCD takes the tiles of one (sequence, head) in turn, last tile
-  // first, so the workgroups that share an L2 walk the same key blocks
-  const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
-  const int pair = (j / nq_tiles) * 8 + xcd, tile = nq_tiles - 1 - j % nq_tiles;
-  if (pair >= p.B * p.HQ) return;   // (the grid is rounded up to whole groups of 8 pairs)
-  const int n = pair / p.HQ, hq = pair % p.HQ;
-  const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
+  int n, hq, tile, len, bos, bos_nats;
+  if (p.seqs == nullptr) {
+    const int nq_tiles = (p.T + QTILE - 1) / QTILE;
+    // every 8th block index lands on the same XCD: an XCD takes the tiles of one (sequence, head) in turn, last tile
+    // first, so the workgroups that share an L2 walk the same key blocks
+    const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
+    const int pair = (j / nq_tiles) * 8 + xcd;
+    tile = nq_tiles - 1 - j % nq_tiles;
+    if (pair >= p.B * p.HQ) return;   // (the grid is rounded up to whole groups of 8 pairs)
+    n = pair / p.HQ;
+    hq = pair % p.HQ;
+    len = p.T;
+    bos = n * p.T;
+    bos_nats = n * p.TN;
+  } else {
+    // packed: the table counts 256-query tiles per sequence, two of this kernel's; last tiles first
+    const int gt = p.total_tiles * 2 - 1 - (int)blockIdx.x / p.HQ;
+    hq = (int)blockIdx.x % p.HQ;
+    n = 0;
+    for (int i = 1; i < p.n_seqs; ++i)
+      if (p.seqs[i].qtile_off * 2 <= gt) n = i;
+    tile = gt - p.seqs[n].qtile_off * 2;
+    bos = p.seqs[n].bos;
+    len = p.seqs[n].eos - bos;
+    bos_nats = p.seqs[n].bos_nats;
+    if (tile * QTILE >= len) return;   // a sequence's last table slot may hold one tile of this size only
+  }
   const int Bs = p.block, per_blk = Bs >> 6;
   const int hkv = hq / (p.HQ / p.HKV), hn = hq / (p.HQ / p.HN);
   const int tile_start = tile * QTILE;
@@ -379,7 +400,7 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hf = lane >> 5;
   const int kh = wave & 1, qh = wave >> 1;
-  const int NTc = (p.T + 63) >> 6;
+  const bool packed = p.seqs != nullptr;
   const int n_pairs = p.B * p.HKV;
   // ---- Persistent workgroups (one per CU; the kernel's registers and LDS admit no more) take units = (sequence, kv
   // head, key chunk) from work queues: starting a workgroup per unit left the CUs idle a quarter of the time.
@@ -387,10 +408,12 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
   // of its own with the key chunks of one (sequence, kv head) after the other, earliest (heaviest) chunk first, and
   // every unit walks the later query chunks from the last one down: units started together stay together in L2.  A
   // workgroup whose queue is empty takes from the other XCDs' queues.
-  __shared__ int unit_pair, unit_jc;
-  const bool per_xcd = n_pairs % 8 == 0;
+  // Packed sequences: one queue, the units of a sequence (kv head after kv head) after those of the one before.
+  __shared__ int unit_pair, unit_jc, unit_seq;
+  const int NT_reg = (p.T + 63) >> 6;
+  const bool per_xcd = !packed && n_pairs % 8 == 0;
   const int n_queues = per_xcd ? 8 : 1;
-  const int queue_len = (per_xcd ? n_pairs / 8 : n_pairs) * NTc;
+  const int queue_len = packed ? p.total_chunks * p.HKV : (per_xcd ? n_pairs / 8 : n_pairs) * NT_reg;
   int q_probe = 0;   // queues found empty so far (they stay empty)
   for (;;) {
     if (tid == 0) {
@@ -399,8 +422,18 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
         const int x = per_xcd ? ((int)blockIdx.x + q_probe) & 7 : 0;
         const int i = atomicAdd(p.queue + x, 1);
         if (i < queue_len) {
-          pr = per_xcd ? (i / NTc) * 8 + x : i / NTc;
-          jj = i % NTc;
+          if (packed) {
+            int sn = 0;
+            for (int u = 1; u < p.n_seqs; ++u)
+              if (p.seqs[u].chunk_off * p.HKV <= i) sn = u;
+            const int r = i - p.seqs[sn].chunk_off * p.HKV, ntc = (p.seqs[sn].eos - p.seqs[sn].bos + 63) >> 6;
+            pr = r / ntc;   // the kv head
+            jj = r % ntc;
+            unit_seq = sn;
+          } else {
+            pr = per_xcd ? (i / NT_reg) * 8 + x : i / NT_reg;
+            jj = i % NT_reg;
+          }
           break;
         }
         ++q_probe;
@@ -409,11 +442,13 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
       unit_jc = jj;
     }
     __syncthreads();
-    const int pair = unit_pair, jc = unit_jc;
+    const int pair = unit_pair, jc = unit_jc, seq = packed ? unit_seq : 0;
     __syncthreads();   // (read before the next round's write)
     if (pair < 0) break;
-  const int n = pair / p.HKV, hkv = pair % p.HKV;
-  const int len = p.T, bos = n * p.T, bos_nats = n * p.TN;
+  const int n = packed ? seq : pair / p.HKV, hkv = packed ? pair : pair % p.HKV;
+  const int bos = packed ? p.seqs[n].bos : n * p.T, len = packed ? p.seqs[n].eos - bos : p.T;
+  const int bos_nats = packed ? p.seqs[n].bos_nats : n * p.TN;
+  const int NTc = (len + 63) >> 6;
   const int Bs = p.block, per_blk = Bs >> 6;
   const int G = p.HQ / p.HKV, GN = p.HQ / p.HN;
   const int kb = (jc * 64) / Bs;
@@ -828,7 +863,7 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     auto kern = dq_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    const long long grid = ((long long)p.B * p.HQ + 7) / 8 * 8 * ((p.T + 127) / 128);
+    const long long grid = p.seqs ? (long long)p.total_tiles * 2 * p.HQ : ((long long)p.B * p.HQ + 7) / 8 * 8 * ((p.T + 127) / 128);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
   }
   {
@@ -838,7 +873,7 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     auto kern = dkdv_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    const long long units = (long long)p.B * p.HKV * ((p.T + 63) / 64);
+    const long long units = p.seqs ? (long long)p.total_chunks * p.HKV : (long long)p.B * p.HKV * ((p.T + 63) / 64);
     long long grid = (cu_count() + 7) / 8 * 8;   // whole groups of 8: block index mod 8 names the XCD and its queue
     if (grid > units) grid = units;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
@@ -859,6 +894,7 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
                                         int types_dtype, const int32_t* nats_block_indices, const int32_t* n_nats_blocks,
                                         int B, int T, int HQ, int HKV, int HN, int K, int V, int TN, int block, float scale,
                                         int flags, int dtype, void* workspace, size_t workspace_bytes,
+                                        const natsl_seq_row* seqs, int n_seqs, int total_tiles, int total_chunks,
                                         natsl_stream_t stream) {
   const char* what = "natsl_softmax_sparse_bwd";
   const int same_block_visible = flags & 1;
@@ -869,7 +905,8 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
   if (B <= 0 || T <= 0 || HQ <= 0 || HKV <= 0 || HN <= 0 || TN <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
   if (HQ % HKV || HQ % HN) return fail(NATSL_ERR_INVALID, "%s: HQ=%d must be a multiple of HKV=%d and HN=%d", what, HQ, HKV, HN);
   if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
-  if (TN != cdiv(T, block)) return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d", what, TN, T, block);
+  if (seqs ? (B != 1 || n_seqs <= 0 || total_tiles <= 0 || total_chunks <= 0) : (TN != cdiv(T, block)))
+    return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   // the dk/dv kernel's DMA requests address the rows of one sequence with 32-bit byte offsets: checked here, before
   // anything is launched
   if ((long long)T * HQ * (K > V ? K : V) * 2 >= (1ll << 32))
@@ -883,6 +920,7 @@ extern "C" int natsl_softmax_sparse_bwd(const void* q, const void* k, const void
   p.queue = reinterpret_cast<int*>(static_cast<char*>(workspace) + bwd_queue_offset(B, T, HQ));
   p.types = types; p.types_dtype = types_dtype; p.idx = nats_block_indices; p.nblk = n_nats_blocks;
   p.B = B; p.T = T; p.HQ = HQ; p.HKV = HKV; p.HN = HN; p.TN = TN; p.block = block;
+  p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0; p.total_tiles = total_tiles; p.total_chunks = total_chunks;
   p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f; p.same_block = same_block_visible ? 1 : 0;
   p.dnats_invalid = (flags & 2) ? 1 : 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

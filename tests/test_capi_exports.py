@@ -51,7 +51,7 @@ def test_argument_validation_needs_no_gpu():
     # the softmax backward's 32-bit row offsets: T * HQ * max(K, V) * 2 bytes must stay below 2^32 -- refused on the host,
     # before any kernel is launched (T = 2^20 tokens x 32 heads x 128 x 2 bytes = 2^33)
     rc = L.natsl_softmax_sparse_bwd(p, p, p, p, p, p, p, p, p, p, p, 1, p, p, 1, 1 << 20, 32, 32, 32, 128, 128, 1 << 14, 64, 0.1, 1, 1,
-                                    p, ctypes.c_size_t(1 << 40), None)
+                                    p, ctypes.c_size_t(1 << 40), None, 0, 0, 0, None)
     assert rc == -2 and b"32-bit" in L.natsl_last_error()
 
 

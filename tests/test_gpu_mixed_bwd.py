@@ -77,6 +77,69 @@ def test_mixed_operator_backward(kind, K, V, block, h0, invalid):
         assert float(dt[..., 1][nonlin].abs().max() if nonlin.any() else 0.0) == 0.0
 
 
+@pytest.mark.parametrize("kind,invalid", [('gdn', False), ('mamba', True)])
+def test_mixed_operator_backward_packed_sequences(kind, invalid):
+    """Packed sequences: the gradients of every sequence equal the oracles' on that sequence alone (own initial state,
+    own final-state gradient, own blocks)."""
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
+    lens, H, HN, K, V, block = [320, 70, 512, 129], 4, 2, 64, 64, 64
+    T, N = sum(lens), len(lens)
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    gen = torch.Generator().manual_seed(77)
+    q, k, v = make_qkv(1, T, H, K, V, 21)
+    if kind == 'mamba':
+        q, k = F.normalize(q.float(), dim=-1).bfloat16(), F.normalize(k.float(), dim=-1).bfloat16()
+    g, beta = make_gates(1, T, H, 22)
+    NB = sum(-(-n // block) for n in lens)
+    ty = make_types(1, NB, HN, 0.4, 23, torch.bfloat16)
+    init = torch.randn(N, H, K, V, generator=gen) * 0.3
+    do_l, do_a = (torch.randn(1, T, H, V, generator=gen).bfloat16() for _ in range(2))
+    dht = torch.randn(N, H, K, V, generator=gen)
+    scale_l = K ** -0.5 if kind == 'gdn' else 1.0
+    leaf = lambda t: None if t is None else t.to(DEV).requires_grad_(True)
+    qa, ka, va, ql, kl, vl, gd, bd, hd, tyd = (leaf(t) for t in (q, k, v, q, k, v, g, beta, init, ty))
+    cud = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    if kind == 'gdn':
+        o_l, o_a, ht = nats_mixed_attn_gdn(qa, ka, va, ql, kl, vl, hd, gd, bd, tyd, None, cu_seqlens=cud, nats_block_size=block,
+                                           ops_for_incomplete_chunks='all', output_final_state_gated_delta=True,
+                                           decay_for_non_gdn_blocks=True, compute_dnats_for_invalid_blocks_linear_att=invalid)
+    else:
+        o_l, o_a, ht = nats_mixed_attn_mamba(qa, ka, va, ql, kl, vl, hd, gd, tyd, None, scale_lattn=1.0, cu_seqlens=cud,
+                                             nats_block_size=block, ops_for_incomplete_chunks='all', output_final_state_mamba=True,
+                                             decay_for_non_mamba_blocks=True, compute_dnats_for_invalid_blocks_linear_att=invalid)
+    ((o_l.float() * do_l.to(DEV).float()).sum() + (o_a.float() * do_a.to(DEV).float()).sum() + (ht * dht.to(DEV)).sum()).backward()
+    torch.cuda.synchronize()
+    dt = tyd.grad.float().cpu().double()
+    nb = 0
+    for i, n in enumerate(lens):
+        a, b, nbi = cu[i], cu[i + 1], -(-n // block)
+        tyi = ty[:, nb:nb + nbi]
+        rl = LB.linear_branch_bwd(kind, q[:, a:b], k[:, a:b], v[:, a:b], g[:, a:b], beta[:, a:b] if kind == 'gdn' else None,
+                                  tyi[..., 1], scale_l, do_l[:, a:b], dht[i:i + 1], init[i:i + 1], block, True, True, True, invalid)
+        dq_a, dk_a, dv_a, dn_a, dn_mag = SB.softmax_branch_bwd(q[:, a:b], k[:, a:b], v[:, a:b], tyi, do_a[:, a:b], K ** -0.5, block,
+                                                               True, with_magnitude=True)
+        w = f" of sequence {i}"
+        _close(ql.grad[:, a:b].float(), rl['dq'], "dq_lattn" + w)
+        _close(kl.grad[:, a:b].float(), rl['dk'], "dk_lattn" + w)
+        _close(vl.grad[:, a:b].float(), rl['dv'], "dv_lattn" + w)
+        _close(gd.grad[:, a:b].float(), rl['dg'], "dg" + w)
+        if kind == 'gdn':
+            _close(bd.grad[:, a:b].float(), rl['dbeta'], "dbeta" + w)
+        _close(hd.grad[i:i + 1].float(), rl['dh0'], "dh0" + w)
+        _close(qa.grad[:, a:b].float(), dq_a, "dq_attn" + w)
+        _close(ka.grad[:, a:b].float(), dk_a, "dk_attn" + w)
+        _close(va.grad[:, a:b].float(), dv_a, "dv_attn" + w)
+        err = (dt[:, nb:nb + nbi, :, 0] - dn_a).abs()
+        assert bool((err <= 2e-3 * dn_mag + 1e-6).all()), f"dnats (softmax op){w}: error {float(err.max()):.3e}"
+        ref, got = rl['dnats'], dt[:, nb:nb + nbi, :, 1]
+        assert float((got - ref).abs().max()) <= 2e-2 * max(float(ref.abs().max()), 1.0) and rel_l2(got, ref) <= 1e-2, \
+            f"dnats (linear op){w}: rel-L2 {rel_l2(got, ref):.3e}"
+        nb += nbi
+
+
 @pytest.mark.parametrize("kind", ['gdn', 'mamba'])
 def test_layer_training_step(kind):
     """One forward + backward of the layer in training mode: every parameter receives a finite gradient, and the gradients

@@ -123,7 +123,7 @@ def test_softmax_bwd_repeatable_and_workspace_reuse():
             _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(o), _capi.ptr(lse), _capi.ptr(do), _capi.ptr(dq), _capi.ptr(dk),
             _capi.ptr(dv), _capi.ptr(dn), _capi.ptr(ty), _capi.dtype_code(ty.dtype), _capi.ptr(r['nats_block_indices']),
             _capi.ptr(r['n_nats_blocks']), B, T, HQ, H, HN, K, V, T // block, block, float(scale), 1, _capi.dtype_code(q.dtype),
-            _capi.ptr(ws), ws_bytes, _capi.stream_ptr(q.device))
+            _capi.ptr(ws), ws_bytes, None, 0, 0, 0, _capi.stream_ptr(q.device))
         _capi.check(rc, "natsl_softmax_sparse_bwd")
         torch.cuda.synchronize()
         outs.append((dq, dk, dv, dn))
@@ -145,3 +145,45 @@ def test_softmax_bwd_dnats_of_blocks_that_are_not_attention_other_shapes():
     _run(2, 600, 2, 2, 2, 64, 64, 64, 0.3, True, seed=22, dnats_invalid=True)             # ragged
     _run(1, 512, 2, 2, 2, 128, 128, 64, 0.0, True, seed=23, dnats_invalid=True)           # nothing typed attention
     _run(2, 512, 4, 4, 4, 128, 128, 64, 0.4, True, seed=24, through_autograd=True, dnats_invalid=True)
+
+
+@pytest.mark.parametrize("dnats_invalid", [False, True])
+@pytest.mark.parametrize("lens,HQ,H,HN,K,V,block", [
+    ([200, 64, 1000, 333, 3], 8, 2, 4, 128, 128, 64),      # ragged lengths, a three-token sequence, grouped heads
+    ([512, 300, 129], 4, 4, 4, 64, 128, 128),              # lengths around the 128-query tile of the dq kernel
+    ([2048, 1536], 16, 16, 16, 128, 64, 256),
+])
+def test_softmax_backward_packed_sequences(lens, HQ, H, HN, K, V, block, dnats_invalid):
+    """Packed sequences (cu_seqlens): every sequence's gradients equal the oracle's on that sequence alone."""
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.attns import parallel_nats_attn
+    T = sum(lens)
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    q, k, v = make_qkv(1, T, H, K, V, 41, HQ=HQ)
+    do = torch.randn(1, T, HQ, V, generator=torch.Generator().manual_seed(48)).bfloat16()
+    TN = sum(-(-n // block) for n in lens)
+    ty = make_types(1, TN, HN, 0.4, 42, torch.bfloat16)
+    scale = K ** -0.5
+    qd, kd, vd, dod, tyd = (t.to(DEV) for t in (q, k, v, do, ty))
+    seqs = nats_util.pack_sequences(cu, None, block, DEV)
+    r = nats_util.route(tyd, T, block, seqs=seqs)
+    qd, kd, vd, tyd = (t.requires_grad_() for t in (qd, kd, vd, tyd))
+    o, _ = parallel_nats_attn(qd, kd, vd, None, tyd, r['nats_block_indices'], r['n_nats_blocks'], scale,
+                              cu_seqlens=torch.tensor(cu, dtype=torch.int32), NAtS_block_size=block,
+                              compute_incomplete_chunk_scores=True, compute_dnats_for_invalid_blocks_attn=dnats_invalid)
+    o.backward(dod)
+    torch.cuda.synchronize()
+    nb = 0
+    for i, n in enumerate(lens):
+        a, b, nbi = cu[i], cu[i + 1], -(-n // block)
+        tyi = ty[:, nb:nb + nbi]
+        dq_r, dk_r, dv_r, dn_r, dn_mag = sb.softmax_branch_bwd(q[:, a:b], k[:, a:b], v[:, a:b], tyi, do[:, a:b], scale, block, True,
+                                                               with_magnitude=True, dnats_invalid=dnats_invalid)
+        _close(qd.grad[:, a:b].float(), dq_r, f"dq of sequence {i}")
+        _close(kd.grad[:, a:b].float(), dk_r, f"dk of sequence {i}")
+        _close(vd.grad[:, a:b].float(), dv_r, f"dv of sequence {i}")
+        err = (tyd.grad[:, nb:nb + nbi, :, 0].float().cpu().double() - dn_r).abs()
+        assert bool((err <= 2e-3 * dn_mag + 1e-6).all()), f"dnats of sequence {i}: error {float(err.max()):.3e}"
+        nb += nbi
