@@ -163,7 +163,7 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
 
 /* Layer tail: y = (rms(x1)*w1*xw[...,0] + rms(x2)*w2*xw[...,1]) * gate*sigmoid(gate) with
  * rms(x) = x*rsqrt(mean(x^2)+eps); x1, x2, gate, y [rows, D] and x_weights [rows, 2] in `dtype`,
- * w1, w2 [D] in `w_dtype`.
+ * w1, w2 [D] in `w_dtype`.  D in {32, 64, 96, 128, 192, 256, 384, 512}.
  * Replaces the forward of FusedMultiInputRMSNormGated (src/nats/modules/fused_norm_gate.py:38-182)
  * as called at src/nats/layers/natsl_attn_gdn.py:652-661. */
 int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const void* x_weights, const void* w1,
@@ -178,7 +178,7 @@ int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const 
  * h_block_start <- S.  q,k [N,T,H,K], v,o [N,T,H,V], beta [N,T,H] in `dtype`; g fp32 [N,T,H];
  * g_cumsum fp32 [N,H] or NULL (0): sum of g over the tokens already in the block; h0 fp32 [N,H,K,V] or NULL
  * (zeros); h_block_start fp32 [N,H,K,V] in/out; ht fp32 [N,H,K,V] or NULL; types [N,1,HN,2] (op 1 = linear);
- * n_tokens_in_block int32 [N] or NULL (then the scalar is used for every sequence).
+ * n_tokens_in_block int32 [N] or NULL (then the scalar is used for every sequence).  K in {64, 128, 192}, V % 16 == 0.
  * Replaces fused_recurrent_gated_delta_rule_nats_fwd, src/nats/ops/gated_delta_rule/fused_recurrent.py:360-470
  * (kernel :28-358) as called with update_hs_for_each_iter=True at
  * src/nats/ops/mixed_ops/mixed_attn_gdn.py:485-503. */

@@ -374,7 +374,9 @@ static int recurrent_fwd(bool delta, const char* what, const void* q, const void
   else if (K == 64 && delta) hipLaunchKernelGGL((gdn_recurrent_kernel<64, true>), grid, dim3(256), 0, s, p);
   else if (K == 128) hipLaunchKernelGGL((gdn_recurrent_kernel<128, false>), grid, dim3(256), 0, s, p);
   else if (K == 64) hipLaunchKernelGGL((gdn_recurrent_kernel<64, false>), grid, dim3(256), 0, s, p);
-  else return fail(NATSL_ERR_UNSUPPORTED, "%s: K=%d not built (supported: 64, 128)", what, K);
+  else if (K == 192 && delta) hipLaunchKernelGGL((gdn_recurrent_kernel<192, true>), grid, dim3(256), 0, s, p);
+  else if (K == 192) hipLaunchKernelGGL((gdn_recurrent_kernel<192, false>), grid, dim3(256), 0, s, p);
+  else return fail(NATSL_ERR_UNSUPPORTED, "%s: K=%d not built (supported: 64, 128, 192)", what, K);
   return check_launch(what);
 }
 

@@ -123,19 +123,19 @@ def test_mask_of_the_next_token():
     assert not bool(m[:, :, 0, -1].any()) and bool(m[:, :, 1, -2:].all())
 
 
-@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
-@pytest.mark.parametrize("T0,T", [(320, 420), (266, 400), (64, 130)])
-def test_layer_generation_matches_whole_forward(kind, T0, T):
+@pytest.mark.parametrize("kind,T0,T,geometry", [(k_, a, b, None) for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (64, 130))]
+                         + [('gdn', 200, 270, '760M')])
+def test_layer_generation_matches_whole_forward(kind, T0, T, geometry):
     """Prefill T0 tokens with a cache, decode up to T token by token (two tokens at a time where the block allows
     it): every output must match the layer's forward over the first T0 tokens resp. the whole sequence at the same
     positions; the selector decisions of the two runs must be identical."""
     from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
-    layer, cfg, w, _ = _layer_case(kind)
+    layer, cfg, w, _ = _layer_case(kind, geometry)
     layer.layer_idx = 0
     layer = layer.to(DEV).to(torch.bfloat16).eval()
     bs = layer.nats_block_size
     torch.manual_seed(T)
-    x = torch.randn(2, T, 256).to(DEV).to(torch.bfloat16)
+    x = torch.randn(2, T, cfg['hidden_size']).to(DEV).to(torch.bfloat16)
     first = lambda out: out[0] if isinstance(out, tuple) else out
     with torch.no_grad():
         whole = first(layer(x))

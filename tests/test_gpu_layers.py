@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
 
 
-@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("D", [64, 96, 128, 192, 256, 384, 512])
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 def test_norm_gate(D, wdtype):
     from neuralattentionsearchlinear_amd.modules import two_inputs_rms_norm_gated
@@ -30,13 +30,21 @@ def test_norm_gate(D, wdtype):
     assert rel_l2(y.float(), ref) <= 5e-3
 
 
-def _layer_case(kind):
+# head geometry of the two published model configurations (experiments/configs/natsl_340M.json, natsl_760M.json):
+# linear heads K 128 / V 256 resp. K 192 / V 384, attention view K 64 / V 128 in both
+PUBLISHED = {'340M': dict(hidden_size=1024, head_dim=128, num_heads=6, num_attn_heads=12, norm_eps=1e-6),
+             '760M': dict(hidden_size=1536, head_dim=192, num_heads=6, num_attn_heads=18, norm_eps=1e-6)}
+
+
+def _layer_case(kind, geometry=None):
     torch.manual_seed(0)
     if kind == 'gdn':
         from neuralattentionsearchlinear_amd.natsl_attn_gdn import NeuralAttentionSearchLinearAttnGDN as L
         # the published ratio: attention view = twice as many heads of half the width (K 64 / V 128 vs K 128 / V 256)
         cfg = dict(hidden_size=256, expand_v=2, head_dim=128, num_heads=2, num_attn_heads=4, nats_block_size=64,
                    ops_for_incomplete_chunks='all', decay_for_non_gdn_blocks=True, norm_eps=1e-5)
+        if geometry is not None:
+            cfg.update(PUBLISHED[geometry])
     else:
         from neuralattentionsearchlinear_amd.natsl_attn_mamba2 import NeuralAttentionSearchLinearAttnMamba as L
         cfg = dict(hidden_size=256, expand_v=0.5, head_dim=128, num_heads=4, num_attn_heads=4, nats_block_size=64,
@@ -47,7 +55,7 @@ def _layer_case(kind):
             if n.endswith('conv1d.weight'):
                 p_.copy_(torch.randn_like(p_) * 0.5)
     w = {k: v.detach().clone().float() for k, v in layer.state_dict().items()}
-    x = torch.randn(2, 320, 256)
+    x = torch.randn(2, 320, cfg['hidden_size'])
     return layer, cfg, w, x
 
 
@@ -86,6 +94,16 @@ def _spy_on_layer(layer, kind):
 @pytest.mark.parametrize("train", [True, False])
 @pytest.mark.parametrize("module_dtype", [torch.float32, torch.bfloat16])
 def test_layer_forward(kind, train, module_dtype):
+    _check_layer_forward(kind, train, module_dtype, None)
+
+
+@pytest.mark.parametrize("geometry", ['340M', '760M'])
+def test_layer_forward_published_head_geometry(geometry):
+    """The GDN layer with the hidden size and head geometry of the published 340M / 760M configurations."""
+    _check_layer_forward('gdn', False, torch.float32, geometry)
+
+
+def _check_layer_forward(kind, train, module_dtype, geometry):
     """The layer on the GPU against the layer oracle.
 
     fp32 module: the torch ops (projections, convolutions, norms) run in fp32 on both sides and the HIP operators compute
@@ -97,7 +115,7 @@ def test_layer_forward(kind, train, module_dtype):
     checked in place, at the stated tolerance, by running the oracle's operators on the GPU's own operator inputs."""
     from neuralattentionsearchlinear_amd import nats_util
     from oracle import mixed as omixed
-    layer, cfg, w, x = _layer_case(kind)
+    layer, cfg, w, x = _layer_case(kind, geometry)
     layer = layer.to(DEV).to(module_dtype).train(train)
     xd = x.to(DEV).to(module_dtype)
     cap, restore = _spy_on_layer(layer, kind)

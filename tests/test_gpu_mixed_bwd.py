@@ -140,14 +140,14 @@ def test_mixed_operator_backward_packed_sequences(kind, invalid):
         nb += nbi
 
 
-@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
-def test_layer_training_step(kind):
+@pytest.mark.parametrize("kind,geometry", [('gdn', None), ('mamba', None), ('gdn', '760M')])
+def test_layer_training_step(kind, geometry):
     """One forward + backward of the layer in training mode: every parameter receives a finite gradient, and the gradients
     of everything outside the selector agree with autograd through the layer oracle on the same (injected) block types.
     The selector's own path (nats_layer) is the straight-through estimator of the operators, checked at operator level."""
     from oracle import layer as olayer
     from tests.test_gpu_layers import _layer_case
-    layer, cfg, w, x = _layer_case(kind)
+    layer, cfg, w, x = _layer_case(kind, geometry)   # ('760M': the published configuration's hidden size and head geometry)
     layer = layer.to(DEV).float().train()
     xd = x.to(DEV).requires_grad_(True)
     out = layer(xd)
