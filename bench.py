@@ -21,6 +21,8 @@ WORKLOADS = {
     "hybrid_gdn_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
     "gdn_only_B4_T4096_H16_d128": dict(B=4, T=4096, H=16, K=128, V=128, p_attn=0.0, block=64),
     "hybrid_gdn_B1_T65536_H32_d128_p10": dict(B=1, T=65536, H=32, K=128, V=128, p_attn=0.10, block=64),
+    # the Mamba2-SSD variant: K = state dim (B, C shared by all heads), V = head dim, selector block 256
+    "hybrid_mamba_B4_T8192_H32_N128_d64_p25": dict(B=4, T=8192, H=32, K=128, V=64, p_attn=0.25, block=256, kind="mamba"),
 }
 # decode: one new token per sequence on cached states, the attention branch over the cached keys/values of the
 # attention-typed blocks (p_attn of the context) plus the current block; not the headline metric
@@ -53,11 +55,21 @@ def make_inputs(w, torch, device):
     import torch.nn.functional as F
     g = torch.Generator().manual_seed(0)
     B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
-    q = torch.randn(B, T, H, K, generator=g).bfloat16()
-    k = torch.randn(B, T, H, K, generator=g).bfloat16()
-    v = torch.randn(B, T, H, V, generator=g).bfloat16()
-    beta = torch.sigmoid(torch.randn(B, T, H, generator=g)).bfloat16()
-    gl = -F.softplus(torch.randn(B, T, H, generator=g))
+    if w.get("kind") == "mamba":
+        # C (as q) and B (as k) ~ N(0,1), one group shared by all heads; X ~ N(0,1); log-decay dt * A with
+        # dt = softplus(N(0,1) - 4), A = -exp(U(0, log 16)) per head
+        q = torch.randn(B, T, 1, K, generator=g).expand(B, T, H, K).contiguous().bfloat16()
+        k = torch.randn(B, T, 1, K, generator=g).expand(B, T, H, K).contiguous().bfloat16()
+        v = torch.randn(B, T, H, V, generator=g).bfloat16()
+        beta = torch.ones(B, T, H).bfloat16()
+        dt = F.softplus(torch.randn(B, T, H, generator=g) - 4.0)
+        gl = -torch.exp(torch.rand(H, generator=g) * math.log(16.0)) * dt
+    else:
+        q = torch.randn(B, T, H, K, generator=g).bfloat16()
+        k = torch.randn(B, T, H, K, generator=g).bfloat16()
+        v = torch.randn(B, T, H, V, generator=g).bfloat16()
+        beta = torch.sigmoid(torch.randn(B, T, H, generator=g)).bfloat16()
+        gl = -F.softplus(torch.randn(B, T, H, generator=g))
     logits = torch.randn(B, T // w["block"], H, 2, generator=g)
     logits[..., 1] += selector_bias(w["p_attn"])
     logits = logits.bfloat16()
@@ -122,11 +134,20 @@ def softmax_flops(types, T, block, K, V):
     return 2.0 * (K + V) * float((n * (n + 1) / 2 + n * block * prior).sum())
 
 
-def gdn_flops(types, K, V, C=64):
+def gdn_flops(types, K, V, C=64, per_block=1):
+    """per 64-token chunk and head: the two Gram products, the solve, w S, T X, q S, P v_new and the state update (kept for
+    chunks of blocks typed linear).  types are per selector block of per_block chunks."""
     lin = types[..., 1].float().round()
-    n_all, n_lin = float(lin.numel()), float(lin.sum())
+    n_all, n_lin = float(lin.numel()) * per_block, float(lin.sum()) * per_block
     per = 2 * C * C * (3 * K + 2 * V) + 6 * C * K * V + (2.0 / 3.0) * C ** 3
     return per * n_all - 2 * C * K * V * (n_all - n_lin)
+
+
+def mamba_flops(types, K, V, C=64, per_block=1):
+    """per chunk and head: q k^T, P v, q S, and the state update for chunks of blocks typed linear."""
+    lin = types[..., 1].float().round()
+    n_all, n_lin = float(lin.numel()) * per_block, float(lin.sum()) * per_block
+    return (2 * C * C * (K + V) + 2 * C * K * V) * n_all + 2 * C * K * V * n_lin
 
 
 def cpu_baseline(host, w, types_host, torch, max_heads=None, max_batch=None):
@@ -140,8 +161,12 @@ def cpu_baseline(host, w, types_host, torch, max_heads=None, max_batch=None):
     q, k, v, beta, g = (sl(host[n]) for n in ("q", "k", "v", "beta", "g"))
     ty = types_host[:Bs, :, :H].contiguous()
     t0 = time.perf_counter()
-    mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, ops_for_incomplete_chunks='all', output_final_state=True,
-                         decay_for_non_gdn_blocks=True, nats_block_size=w["block"])
+    if w.get("kind") == "mamba":
+        mixed.mixed_attn_mamba(q, k, v, q, k, v, None, g, ty, scale_lattn=1.0, ops_for_incomplete_chunks='all', output_final_state=True,
+                               decay_for_non_mamba_blocks=True, nats_block_size=w["block"])
+    else:
+        mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, ops_for_incomplete_chunks='all', output_final_state=True,
+                             decay_for_non_gdn_blocks=True, nats_block_size=w["block"])
     dt = time.perf_counter() - t0
     tok_s = Bs * w["T"] / dt * (H / w["H"])
     sample = (f"{Bs} of {w['B']} sequences, {H} of {w['H']} heads, full T={w['T']}; {dt:.1f} s of the fp32 torch-CPU oracle, "
@@ -316,12 +341,14 @@ def main():
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
         sys.exit(2)
     _capi.lib()
     device = torch.device("cuda:0")
     w = WORKLOADS[args.workload]
+    is_mamba = w.get("kind") == "mamba"
     host, dev = make_inputs(w, torch, device)
 
     events = []
@@ -333,6 +360,10 @@ def main():
 
     def step():
         ty, nb = nats_util.hard_select(dev["logits"], force_last_block=True)
+        if is_mamba:
+            return nats_mixed_attn_mamba(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v"], None, dev["g"], ty, nb,
+                                         scale_lattn=1.0, nats_block_size=w["block"], ops_for_incomplete_chunks="all",
+                                         output_final_state_mamba=True, decay_for_non_mamba_blocks=True), ty
         return nats_mixed_attn_gdn(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v"], None, dev["g"], dev["beta"], ty,
                                    nb, nats_block_size=w["block"], ops_for_incomplete_chunks="all",
                                    output_final_state_gated_delta=True, decay_for_non_gdn_blocks=True), ty
@@ -392,11 +423,12 @@ def main():
     sm_alone_ms, lin_alone_ms = avg_ms("softmax", events[n_timed_events:]), avg_ms("linear", events[n_timed_events:])
     types_host = ty.cpu()
     f_attn = softmax_flops(types_host, w["T"], w["block"], w["K"], w["V"])
-    f_gdn = gdn_flops(types_host, w["K"], w["V"])
+    f_gdn = (mamba_flops if is_mamba else gdn_flops)(types_host, w["K"], w["V"], per_block=w["block"] // 64)
     B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
     traffic, traffic_source = measured_traffic(args.workload)
     # the linear branch (prep + scan kernels): algorithmic bytes = q, k, v read once, o written once, g and beta, final state
-    lin_bytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * 6 + B * H * K * V * 4
+    # (the Mamba workload's B and C are stored per head here, as the operator takes them, and counted so)
+    lin_bytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * (4 if is_mamba else 6) + B * H * K * V * 4
     roof_lin = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=lin_bytes / (lin_ms * 1e-3) / 1e9,
                     peak=PEAK_HBM_GBS, unit="GB/s", frac=lin_bytes / (lin_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     traffic=(traffic or {}).get("linear_bytes"), launch_ms=lin_ms, algorithmic_bytes=lin_bytes,
@@ -404,7 +436,7 @@ def main():
                     launch_ms_alone=lin_alone_ms)
     if f_attn >= f_gdn:
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", kernel="softmax_stream_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
+        roof = dict(bound="mfma", kernel="softmax_stream_kernel" if T % 256 == 0 and B * H * (T // 256) >= 512 else "softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
                     unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=(traffic or {}).get("softmax_bytes"),
                     traffic_source=traffic_source, launch_ms=sm_ms, algorithmic_flops=f_attn,
                     # the same kernel with the GPU to itself (branches launched one after the other, outside the timed region)
