@@ -134,7 +134,10 @@ def test_errors_mirror_reference():
     with pytest.raises(NotImplementedError):
         nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, attn_sw_size=128)
     with pytest.raises(NotImplementedError):
-        nats_mixed_attn_gdn(q.requires_grad_(), k, v, q, k, v, None, g, beta, ty, None)
+        nats_mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, None, use_g_for_attn=True)
+    # inputs that require grad go through the differentiable operator
+    o_l, o_a, _ = nats_mixed_attn_gdn(q.clone().requires_grad_(), k, v, q, k, v, None, g, beta, ty, None)
+    assert o_l.requires_grad and o_a.requires_grad
 
 
 @pytest.mark.parametrize("decay", [True, False])
