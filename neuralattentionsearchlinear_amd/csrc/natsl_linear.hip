@@ -72,112 +72,59 @@ NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
 // =============================================================================================
 // prep
 // =============================================================================================
-// index of A operand (t, s) of TmB / P among the six that the scan keeps in LDS (the two above the diagonal are skipped)
-NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t : 2 * t - 2 + s; }
-
-// What the prep of one chunk reads from memory, in registers: a caller can fetch it a step ahead of its use.
-// Thread t of 256: the 16-byte pieces seg + 4 i of row t / 4 (seg = t % 4); threads 0..63 also token t's g and beta.
-template <int DK>
-struct PrepRegs {
-  u32x4 q[DK / 32], k[DK / 32];
-  float g, beta;
-};
-
 template <int DK, bool DELTA>
-NATSL_DEVICE void prep_fetch(const LinearParams& p, PrepRegs<DK>& r, const int t, const int bos, const int len, const int t0, const int h) {
-  constexpr int KL = DK / 32;
-  const int row = t >> 2, seg = t & 3;
-  const bool ok = t0 + row < len;
-  const size_t off = ((size_t)(bos + t0 + row) * p.H + h) * DK;
-  const u32x4* qr = reinterpret_cast<const u32x4*>(p.q + off);
-  const u32x4* kr = reinterpret_cast<const u32x4*>(p.k + off);
-  const u32x4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-  for (int i = 0; i < KL; ++i) {
-    r.q[i] = ok ? qr[seg + 4 * i] : z;
-    r.k[i] = ok ? kr[seg + 4 * i] : z;
-  }
-  r.g = 0.f;
-  r.beta = 0.f;
-  if (t < C) {
-    const bool ok1 = t0 + t < len;
-    const size_t gi = (size_t)(bos + t0 + t) * p.H + h;
-    r.g = ok1 ? p.g[gi] : 0.f;
-    if (DELTA) r.beta = ok1 ? bf16_to_f32(p.beta[gi]) : 0.f;
-  }
-}
-
-// LDS of the prep: region0 holds the q, k tiles (rows of DK + 8 bf16) and, once the Gram products are done, the blocks of
-// the solve in their place; vec holds gamma, 1/|q|, 1/|k|, beta (64 floats each).
-template <int DK, bool DELTA>
-struct PrepLds {
-  static constexpr int KP = DK + 8;   // bf16 row pitch
-  // The 64x64 fp32 matrices of the solve are kept as their ten lower 16x16 blocks, block (i, k) at index i(i+1)/2 + k,
-  // rows of BP floats.  A = strictly lower system matrix; X = (I+A)^-1 row-major; Xt = the four DIAGONAL blocks of X
-  // transposed (so that such a block serves as an MFMA B operand with one 16-byte read).
-  static constexpr int BP = 20, BLK = 16 * BP, NBLK = 10;
-  static constexpr int TILE_BYTES = 2 * C * KP * 2, SOLVE_BYTES = (2 * NBLK + 4) * BLK * 4;
-  static constexpr int REGION0 = (DELTA && SOLVE_BYTES > TILE_BYTES) ? SOLVE_BYTES : TILE_BYTES;
-  static constexpr int VEC_BYTES = 4 * C * 4;
-};
-
-// Where a chunk's results go: the workspace in global memory (8 operand slots of 1 KiB per matrix, slot 2 t + s), or,
-// FUSED, the scan's stage in LDS (6 slots, tri_slot(t, s)) as byte addresses.
-struct PrepOut {
-  bf16_t* P; bf16_t* T; float* SC;
-  unsigned lds_P, lds_T, lds_SC;
-};
-
-// Arrival counter in LDS for the helper waves of the fused kernel: the hardware barrier belongs to the whole workgroup
-// (one per step), so the four prep waves meet among themselves through this counter.  The wait is bounded: a wave that
-// never sees the others arrive goes on after about 2^20 polls instead of hanging the GPU.
-struct HelperSync {
-  unsigned addr, target;
-};
-NATSL_DEVICE void helper_barrier(HelperSync& hs) {
-  hs.target += 4;
-  // this wave's LDS writes, and its reads of what the others overwrite next, are done before it is counted
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  if ((threadIdx.x & 63) == 0) asm volatile("ds_add_u32 %0, %1" ::"v"(hs.addr), "v"(1u) : "memory");
-  for (int spin = 0; spin < (1 << 20); ++spin) {
-    unsigned v;
-    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(hs.addr) : "memory");
-    if ((int)((unsigned)__builtin_amdgcn_readfirstlane((int)v) - hs.target) >= 0) break;
-    __builtin_amdgcn_s_sleep(1);
-  }
-}
-
-// The prep of one chunk by 256 threads (tid 0..255).  `sync` is the meeting of those four waves; `after_consume` runs
-// once the registers in `r` have been used up (the fused kernel fetches the next chunk's there).
-template <int DK, bool DELTA, bool FUSED, class Sync, class AfterConsume>
-NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const int tid, unsigned char* region0, float* vec,
-                             const PrepOut out, const size_t type_idx, Sync sync, AfterConsume after_consume) {
-  using M = PrepLds<DK, DELTA>;
-  constexpr int KP = M::KP, KL = DK / 32, BP = M::BP, BLK = M::BLK, NBLK = M::NBLK;
-  typedef __attribute__((address_space(3))) u32x4* lds_w16;
-  typedef __attribute__((address_space(3))) u32x2* lds_w8;
-  typedef __attribute__((address_space(3))) float* lds_w4;
+__global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) {
+  constexpr int KP = DK + 8;   // bf16 row pitch
+  constexpr int KL = DK / 32;  // 16-byte loads per thread per tile
+  // The 64x64 fp32 matrices of the solve are kept as their ten lower 16x16 blocks, block (i, k) at
+  // index i(i+1)/2 + k, rows of BP floats.  A = strictly lower system matrix; X = (I+A)^-1 row-major;
+  // Xt = the four DIAGONAL blocks of X transposed (so that such a block serves as an MFMA B operand with one 16-byte read).
+  constexpr int BP = 20, BLK = 16 * BP, NBLK = 10;
+  constexpr int TILE_BYTES = 2 * C * KP * 2, SOLVE_BYTES = (2 * NBLK + 4) * BLK * 4;
+  // LDS: the q, k tiles are dead once the Gram products are done; the solve reuses their space
+  constexpr int REGION0 = (DELTA && SOLVE_BYTES > TILE_BYTES) ? SOLVE_BYTES : TILE_BYTES;
+  __shared__ __align__(16) unsigned char region0[REGION0];
+  __shared__ __align__(16) float gam[C], rq[C], rk[C], bet[C];
   bf16_t* Qs = reinterpret_cast<bf16_t*>(region0);
   bf16_t* Ks = Qs + C * KP;
   float* Ab = reinterpret_cast<float*>(region0);
   float* Xb = Ab + NBLK * BLK;
   float* Xt = Xb + NBLK * BLK;
-  float *gam = vec, *rq = vec + C, *rk = vec + 2 * C, *bet = vec + 3 * C;
   auto bidx = [](int i, int k) { return i * (i + 1) / 2 + k; };
-  const int wave = tid >> 6, lane = tid & 63;
-  const bool l2 = (p.flags & NATSL_QK_L2NORM) != 0;
-  auto put_sc = [&](const int idx, const float x) {
-    if constexpr (FUSED) *reinterpret_cast<lds_w4>(out.lds_SC + 4u * idx) = x;
-    else out.SC[idx] = x;
-  };
 
-  // ---- q, k tiles; row sums of squares from the registers -----------------------------------
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
+  int bos, len, c, bos_nats;
+  if (p.seqs == nullptr) {
+    const int n = gc / p.nt;
+    c = gc - n * p.nt;
+    bos = n * p.T;
+    len = p.T;
+    bos_nats = n * p.TN;
+  } else {
+    int n = 0;
+    for (int i = 1; i < p.n_seqs; ++i)
+      if (p.seqs[i].chunk_off <= gc) n = i;
+    c = gc - p.seqs[n].chunk_off;
+    bos = p.seqs[n].bos;
+    len = p.seqs[n].eos - bos;
+    bos_nats = p.seqs[n].bos_nats;
+  }
+  const int t0 = c * C;
+  const bool l2 = (p.flags & NATSL_QK_L2NORM) != 0;
+
+  // ---- load q, k tiles; row sums of squares from the registers just loaded -----------------
   {
     const int row = tid >> 2, seg = tid & 3;
+    const bool ok = t0 + row < len;
+    const size_t off = ((size_t)(bos + t0 + row) * p.H + h) * DK;
+    const u32x4* qr = reinterpret_cast<const u32x4*>(p.q + off);
+    const u32x4* kr = reinterpret_cast<const u32x4*>(p.k + off);
+    const u32x4 z = {0u, 0u, 0u, 0u};
     float sq = 0.f, sk = 0.f;
 #pragma unroll
     for (int i = 0; i < KL; ++i) {
-      const u32x4 a = r.q[i], b = r.k[i];
+      const u32x4 a = ok ? qr[seg + 4 * i] : z, b = ok ? kr[seg + 4 * i] : z;
       *reinterpret_cast<u32x4*>(Qs + row * KP + (seg + 4 * i) * 8) = a;
       *reinterpret_cast<u32x4*>(Ks + row * KP + (seg + 4 * i) * 8) = b;
 #pragma unroll
@@ -197,33 +144,39 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
   }
   // ---- gamma = inclusive cumsum of g over the chunk (wave 0), beta -------------------------
   if (wave == 0) {
-    float x = r.g;
+    const bool ok = t0 + lane < len;
+    const size_t gi = (size_t)(bos + t0 + lane) * p.H + h;
+    float x = ok ? p.g[gi] : 0.f;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const float y = __shfl_up(x, d);
       if (lane >= d) x += y;
     }
     gam[lane] = x;
-    if (DELTA) bet[lane] = r.beta;
+    if (DELTA) bet[lane] = ok ? bf16_to_f32(p.beta[gi]) : 0.f;
   }
-  after_consume();
-  sync();
+  __syncthreads();
+
+  const size_t unit = (size_t)gc * p.H + h;
+  bf16_t* Pout = p.ws_p + unit * (C * C);
+  bf16_t* Tout = p.ws_tm + unit * (C * C);
+  float* Sout = p.ws_sc + unit * (4 * C);
 
   // ---- Gram products on the matrix cores: wave w owns the 32x32 tile (w/2, w%2) ------------
   // P and TmB are stored as the scan kernel's MFMA A operands (16x16x32: 16 rows x 32 contraction tokens), 1 KiB each,
-  // operand (t, s) = rows 16t.., tokens 32s..; in it, scan-lane (row i%16, group g) finds its 16 bytes
+  // operand (t, s) = rows 16t.., tokens 32s.. at index 2t + s; in it, scan-lane (row i%16, group g) finds its 16 bytes
   // at (16 g + i%16) * 16.  The scan feeds the other operand from accumulator registers, where lane group g holds
   // tokens 4g..4g+3 of a 16-token tile, so slot j of group g stands for token 32s + 16(j/4) + 4g + j%4.
   // Operands (0,1) and (1,1) lie above the diagonal: never written, never read.
   {
     const int ti = wave >> 1, tj = wave & 1, l32 = lane & 31, hf = lane >> 5;
     const int i = 32 * ti + l32;  // P row owned by this lane
-    const int p_elem = ((FUSED ? tri_slot(i >> 4, tj) : 2 * (i >> 4) + tj) * 64 + (i & 15)) * 8;
+    bf16_t* prow = Pout + ((size_t)((2 * (i >> 4) + tj) * 64 + (i & 15))) * 8;
     f32x16 gk;
     if (ti >= tj) {
       f32x16 gq;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) gk[e] = gq[e] = 0.f;
+      for (int r = 0; r < 16; ++r) gk[r] = gq[r] = 0.f;
 #pragma unroll
       for (int s = 0; s < DK / 16; ++s) {
         const bf16x8 kb = ld8(Ks + (32 * tj + l32) * KP + 16 * s + 8 * hf);
@@ -250,18 +203,13 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
           w[q4 & 1][2 * (q4 >> 1)] = pack_bf16x2(pv[0], pv[1]);
           w[q4 & 1][2 * (q4 >> 1) + 1] = pack_bf16x2(pv[2], pv[3]);
         }
-        if constexpr (FUSED) {
-          *reinterpret_cast<lds_w16>(out.lds_P + 2u * (p_elem + hf * 128)) = w[0];
-          *reinterpret_cast<lds_w16>(out.lds_P + 2u * (p_elem + (2 + hf) * 128)) = w[1];
-        } else {
-          *reinterpret_cast<u32x4*>(out.P + p_elem + hf * 128) = w[0];
-          *reinterpret_cast<u32x4*>(out.P + p_elem + (2 + hf) * 128) = w[1];
-        }
+        *reinterpret_cast<u32x4*>(prow + hf * 128) = w[0];
+        *reinterpret_cast<u32x4*>(prow + (2 + hf) * 128) = w[1];
       }
     }
     if (DELTA) {
       // all waves are done reading the q, k tiles before the A blocks overwrite them
-      sync();
+      __syncthreads();
       if (ti >= tj) {
         const int j = 32 * tj + l32;
         const float gj = gam[j], rkj = rk[j];
@@ -285,16 +233,20 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
     const float gl = gam[C - 1], gt = gam[lane], eg = __expf(gt);
     float dk = gl - gt;
     if (!DELTA) dk = fminf(dk, 0.f);  // src/nats/ops/mamba/chunk_h.py:177
-    put_sc(lane, eg * rk[lane]);
-    put_sc(C + lane, p.scale * rq[lane] * eg);
-    put_sc(2 * C + lane, rk[lane] * __expf(dk));
-    if (lane == 0) put_sc(3 * C, __expf(gl));
-    if (lane == 1) put_sc(3 * C + 1, gl);
-    // is this chunk's selector block typed linear?  (kept next to the decay so the scan finds it with it)
-    if (lane == 2) put_sc(3 * C + 2, lin_type(p.types, p.types_dtype, type_idx) ? 1.f : 0.f);
+    Sout[lane] = eg * rk[lane];
+    Sout[C + lane] = p.scale * rq[lane] * eg;
+    Sout[2 * C + lane] = rk[lane] * __expf(dk);
+    if (lane == 0) Sout[3 * C] = __expf(gl);
+    if (lane == 1) Sout[3 * C + 1] = gl;
+    if (lane == 2) {
+      // is this chunk's selector block typed linear?  (kept next to the decay so the scan finds it
+      // in the cache line it prefetches anyway)
+      const int hn = h / (p.H / p.HN);
+      Sout[3 * C + 2] = lin_type(p.types, p.types_dtype, ((size_t)(bos_nats + (c * C) / p.block) * p.HN + hn) * 2 + 1) ? 1.f : 0.f;
+    }
   }
   if (!DELTA) return;
-  sync();
+  __syncthreads();
 
   // ---- X = (I + A)^-1 in fp32, 4x4 blocks of 16x16 ------------------------------------------
   // diagonal blocks by forward substitution: wave b owns block (b, b), one column per lane
@@ -303,32 +255,33 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
     const float* Ad = Ab + bidx(wave, wave) * BLK;
     f32x4 arow[16][4];
 #pragma unroll
-    for (int rr = 1; rr < 16; ++rr)
+    for (int r = 1; r < 16; ++r)
 #pragma unroll
-      for (int j4 = 0; j4 < (rr + 3) / 4; ++j4) arow[rr][j4] = *reinterpret_cast<const f32x4*>(Ad + rr * BP + 4 * j4);
+      for (int j4 = 0; j4 < (r + 3) / 4; ++j4) arow[r][j4] = *reinterpret_cast<const f32x4*>(Ad + r * BP + 4 * j4);
     float x[16];
 #pragma unroll
-    for (int rr = 0; rr < 16; ++rr) {
-      float acc = rr == x16 ? 1.f : 0.f;
+    for (int r = 0; r < 16; ++r) {
+      float acc = r == x16 ? 1.f : 0.f;
 #pragma unroll
-      for (int j = 0; j < rr; ++j) acc -= arow[rr][j >> 2][j & 3] * x[j];
-      x[rr] = acc;
+      for (int j = 0; j < r; ++j) acc -= arow[r][j >> 2][j & 3] * x[j];
+      x[r] = acc;
     }
     float* Xd = Xb + bidx(wave, wave) * BLK;
     float* Xtd = Xt + wave * BLK;
 #pragma unroll
-    for (int rr = 0; rr < 16; ++rr) Xd[rr * BP + x16] = x[rr];
+    for (int r = 0; r < 16; ++r) Xd[r * BP + x16] = x[r];
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4)
       *reinterpret_cast<f32x4*>(Xtd + x16 * BP + 4 * r4) = (f32x4){x[4 * r4], x[4 * r4 + 1], x[4 * r4 + 2], x[4 * r4 + 3]};
   }
-  sync();
+  __syncthreads();
   // off-diagonal blocks on the fp32 matrix cores, wave k down its own block column:
   //   X_ik = -X_ii * sum_{j=k}^{i-1} A_ij X_jk        (i = k+1 .. 3)
   // MFMA 16x16x4: lane (x, g) supplies A[x][kk] and B[kk][x].  With kk = 4g + s in step s, the A operand of all four
   // steps is one 16-byte row read, and an accumulator (lane = column x, registers = rows 4g..4g+3) is already a B
   // operand: the X_jk of the column stay in registers (only the diagonal block comes from LDS), and the inner sum feeds
-  // the second product from registers too.  Nothing a wave reads here was written by another wave after the meeting above.
+  // the second product from registers too.  Nothing a wave reads here was written by another wave after the barrier above,
+  // so the column needs no barrier of its own.
   {
     const int k = wave;
     f32x4 Xcol[4];
@@ -336,7 +289,7 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
     for (int i = 1; i < 4; ++i) {
       Xcol[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
       if (i > k) {
-        f32x4 Mx = {0.f, 0.f, 0.f, 0.f};
+        f32x4 M = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < i; ++j) {
           if (j >= k) {
@@ -344,21 +297,21 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
             f32x4 b4 = Xcol[j];
             if (j == k) b4 = *reinterpret_cast<const f32x4*>(Xt + k * BLK + x16 * BP + 4 * g4);
 #pragma unroll
-            for (int st = 0; st < 4; ++st) Mx = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[st], b4[st], Mx, 0, 0, 0);
+            for (int st = 0; st < 4; ++st) M = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[st], b4[st], M, 0, 0, 0);
           }
         }
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(Xb + bidx(i, i) * BLK + x16 * BP + 4 * g4);
         f32x4 Xa = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int st = 0; st < 4; ++st) Xa = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[st], Mx[st], Xa, 0, 0, 0);
+        for (int st = 0; st < 4; ++st) Xa = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[st], M[st], Xa, 0, 0, 0);
         Xcol[i] = (f32x4){-Xa[0], -Xa[1], -Xa[2], -Xa[3]};
         float* Xo = Xb + bidx(i, k) * BLK;
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) Xo[(4 * g4 + rr) * BP + x16] = Xcol[i][rr];
+        for (int r = 0; r < 4; ++r) Xo[(4 * g4 + r) * BP + x16] = Xcol[i][r];
       }
     }
   }
-  sync();
+  __syncthreads();
   // TmB = Tm * diag(beta), bf16, in the scan kernel's A-operand order (see above): this thread's 16 columns are one
   // half (cb % 2) of the 32 tokens of operand (row / 16, cb / 2); columns 4g..4g+3 of them are the lower (upper) 8 bytes
   // of scan-lane group g.  Blocks above the diagonal are zero; operands (0,1), (1,1) are not stored at all.
@@ -374,53 +327,16 @@ NATSL_DEVICE void prep_chunk(const LinearParams& p, const PrepRegs<DK>& r, const
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[4 * e4 + e] = xv[e] * bv[e];
       }
-      const int t_elem = ((FUSED ? tri_slot(row >> 4, cb >> 1) : 2 * (row >> 4) + (cb >> 1)) * 64 + (row & 15)) * 8 + 4 * (cb & 1);
+      bf16_t* trow = Tout + ((size_t)((2 * (row >> 4) + (cb >> 1)) * 64 + (row & 15))) * 8 + 4 * (cb & 1);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 w;
         w[0] = pack_bf16x2(x[4 * g], x[4 * g + 1]);
         w[1] = pack_bf16x2(x[4 * g + 2], x[4 * g + 3]);
-        if constexpr (FUSED) *reinterpret_cast<lds_w8>(out.lds_T + 2u * (t_elem + g * 128)) = w;
-        else *reinterpret_cast<u32x2*>(out.T + t_elem + g * 128) = w;
+        *reinterpret_cast<u32x2*>(trow + g * 128) = w;
       }
     }
   }
-}
-
-template <int DK, bool DELTA>
-__global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) {
-  using M = PrepLds<DK, DELTA>;
-  __shared__ __align__(16) unsigned char region0[M::REGION0];
-  __shared__ __align__(16) float vec[4 * C];
-  const int tid = threadIdx.x;
-  const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
-  int bos, len, c, bos_nats;
-  if (p.seqs == nullptr) {
-    const int n = gc / p.nt;
-    c = gc - n * p.nt;
-    bos = n * p.T;
-    len = p.T;
-    bos_nats = n * p.TN;
-  } else {
-    int n = 0;
-    for (int i = 1; i < p.n_seqs; ++i)
-      if (p.seqs[i].chunk_off <= gc) n = i;
-    c = gc - p.seqs[n].chunk_off;
-    bos = p.seqs[n].bos;
-    len = p.seqs[n].eos - bos;
-    bos_nats = p.seqs[n].bos_nats;
-  }
-  PrepRegs<DK> r;
-  prep_fetch<DK, DELTA>(p, r, tid, bos, len, c * C, h);
-  const size_t unit = (size_t)gc * p.H + h;
-  PrepOut out;
-  out.P = p.ws_p + unit * (C * C);
-  out.T = p.ws_tm + unit * (C * C);
-  out.SC = p.ws_sc + unit * (4 * C);
-  out.lds_P = out.lds_T = out.lds_SC = 0;
-  const int hn = h / (p.H / p.HN);
-  const size_t type_idx = ((size_t)(bos_nats + (c * C) / p.block) * p.HN + hn) * 2 + 1;
-  prep_chunk<DK, DELTA, false>(p, r, tid, region0, vec, out, type_idx, [] { __syncthreads(); }, [] {});
 }
 
 // =============================================================================================
@@ -478,6 +394,9 @@ struct ScanLds {
   static constexpr int NSTAGE = 3 * STAGE + 2 * OB <= 160 * 1024 ? 3 : 2;
   static constexpr int TOTAL = NSTAGE * STAGE + 2 * OB;
 };
+
+// index of A operand (t, s) of TmB / P among the six that are stored (the two above the diagonal are skipped)
+NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t : 2 * t - 2 + s; }
 
 // Registers per wave: with DK <= 128 the kernel fits 256, so it asks for the two-waves-per-SIMD register budget even though
 // LDS admits one workgroup per CU: within that budget the matrix instructions take their accumulators in ordinary vector
