@@ -150,11 +150,17 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
 
         if cache is not None and mode != 'chunk' and q_len > 1:
             # refuse BEFORE the cache is touched: a refused step must leave it as it was
-            if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
-                raise NotImplementedError("a decode step of several tokens that crosses a selector-block boundary is not built: "
-                                          "split it at the boundary")
             if self.ops_for_incomplete_chunks == 'gated_delta_net':
                 raise NotImplementedError("several new tokens per decode step are not built for ops_for_incomplete_chunks=gated_delta_net")
+            if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
+                # the step crosses a selector-block boundary: the tokens that complete the block first (the block gets its
+                # type and the cache is updated), then the rest as the start of the next block -- what the reference's
+                # recurrent kernel does with two blocks in one call (src/nats/ops/gated_delta_rule/fused_recurrent.py:144-358)
+                first = self.nats_block_size - cache._n_tokens_in_nats_block
+                kw = dict(past_key_values=past_key_values, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
+                o1 = self.forward(hidden_states[:, :first], attention_mask, **kw)[0]
+                o2 = self.forward(hidden_states[:, first:], attention_mask, **kw)[0]
+                return torch.cat([o1, o2], 1), None, past_key_values
         # selector: on a cache, over the tokens of the incomplete block + the new ones, once they complete a block
         if cache is not None:
             selector_input = cache.update_attn_types(input_hidden_states=hidden_states)

@@ -127,11 +127,15 @@ class NeuralAttentionSearchLinearAttnMamba(nn.Module):
 
         if cache is not None and mode != 'chunk' and q_len > 1:
             # refuse BEFORE the cache is touched: a refused step must leave it as it was
-            if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
-                raise NotImplementedError("a decode step of several tokens that crosses a selector-block boundary is not built: "
-                                          "split it at the boundary")
             if self.ops_for_incomplete_chunks == 'mamba':
                 raise NotImplementedError("several new tokens per decode step are not built for ops_for_incomplete_chunks=mamba")
+            if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
+                # the step crosses a selector-block boundary: the tokens that complete the block first, then the rest as the
+                # start of the next block (src/nats/ops/mamba/fused_recurrent.py handles the two blocks in one call)
+                first = self.nats_block_size - cache._n_tokens_in_nats_block
+                kw = dict(cache_params=cache_params, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
+                return torch.cat([self.forward(hidden_states[:, :first], attention_mask, **kw),
+                                  self.forward(hidden_states[:, first:], attention_mask, **kw)], 1)
         selector_input = cache.update_attn_types(input_hidden_states=hidden_states) if cache is not None else hidden_states
         if selector_input is not None:
             raw_types, _, _ = self.select_ops(selector_input, cu_seqlens, force_last_block=False)

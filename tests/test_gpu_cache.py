@@ -174,8 +174,6 @@ def test_layer_rejects_what_the_cache_cannot_do():
         layer(xd[:, :100], past_key_values=cache, use_cache=True)
         with pytest.raises(NotImplementedError):
             layer(xd[:, 100:200], past_key_values=cache, use_cache=True)      # a second chunked forward
-        with pytest.raises(NotImplementedError):
-            layer(xd[:, 100:140], past_key_values=cache, use_cache=True)      # 36 + 40 tokens cross a block boundary
         # a refused step leaves the cache as it was: the same tokens fed one at a time afterwards give what an
         # untouched cache gives
         fresh = NAtSCache()
@@ -184,3 +182,31 @@ def test_layer_rejects_what_the_cache_cannot_do():
             a = layer(xd[:, t:t + 1], past_key_values=cache, use_cache=True)[0]
             b = layer(xd[:, t:t + 1], past_key_values=fresh, use_cache=True)[0]
             assert torch.equal(a, b), f"token {t} differs after a refused step"
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+def test_decode_step_across_a_block_boundary(kind):
+    """A decode step of several tokens that crosses a selector-block boundary (36 cached tokens of the block + 40 new ones)
+    gives what the same tokens give one at a time, and leaves the cache in the same state."""
+    from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
+    layer, cfg, w, x = _layer_case(kind)
+    layer.layer_idx = 0
+    layer = layer.to(DEV).to(torch.bfloat16).eval()
+    xd = x.to(DEV).bfloat16()
+    first = lambda out: out[0] if isinstance(out, tuple) else out
+    mk = (lambda: NAtSCache()) if kind == 'gdn' else (lambda: NAtSMamba2Cache())
+    kw = lambda h: dict(past_key_values=h, use_cache=True) if kind == 'gdn' else dict(cache_params=h, use_cache=True)
+    with torch.no_grad():
+        a_h, b_h = mk(), mk()
+        layer(xd[:, :100], **kw(a_h))
+        layer(xd[:, :100], **kw(b_h))
+        a = first(layer(xd[:, 100:140], **kw(a_h)))
+        b = torch.cat([first(layer(xd[:, t:t + 1], **kw(b_h))) for t in range(100, 140)], 1)
+        assert a.shape == b.shape
+        assert rel_l2(a.float(), b.float()) <= 1e-3, f"rel-L2 {rel_l2(a.float(), b.float()):.3e}"
+        ca, cb = (h[0] if kind == 'gdn' else h.nats_cache[0] for h in (a_h, b_h))
+        assert ca.n_observed_tokens == cb.n_observed_tokens == 140 and ca._n_tokens_in_nats_block == cb._n_tokens_in_nats_block == 12
+        assert torch.equal(ca.n_attn_blocks, cb.n_attn_blocks)
+        # and the two caches go on alike
+        a2, b2 = first(layer(xd[:, 140:141], **kw(a_h))), first(layer(xd[:, 140:141], **kw(b_h)))
+        assert rel_l2(a2.float(), b2.float()) <= 1e-3
