@@ -5,8 +5,9 @@ Projections, short convolutions and norms are torch; block pooling, the selector
 and the output norm-gate are the HIP kernels of this package.  Training works: the softmax branch's backward is a HIP
 kernel, the linear branch, the pooling and the norm-gate differentiate through torch operations.  With a NAtSCache
 the layer prefills once in chunk mode on the empty cache and then decodes in steps of fewer than 64 tokens;
-continuing a chunked prefill on a cache that already holds tokens raises NotImplementedError (the reference's
-attention operator cannot do it either: it sizes its output by the keys, src/nats/ops/attns/attns.py:1439,1491).
+64 or more new tokens on a cache that already holds tokens run through that decode path in steps (there is no chunked
+kernel that starts from cached keys; the reference's attention operator cannot run this case at all: it sizes its
+output by the keys, src/nats/ops/attns/attns.py:1439,1491).
 """
 from __future__ import annotations
 
@@ -143,8 +144,16 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
         if cache is None and mode != 'chunk':
             raise ValueError("fewer than 64 tokens are decoded on a cache: pass past_key_values")
         if cache is not None and mode == 'chunk' and cache.n_observed_tokens > 0:
-            raise NotImplementedError("a chunked forward that continues a non-empty cache is not built: prefill once, then "
-                                      "decode in steps of fewer than 64 tokens")
+            if cu_seqlens is not None:
+                raise NotImplementedError("packed sequences are not supported together with a cache")
+            # 64 or more new tokens on a cache that already holds tokens (a second prompt): there is no chunked kernel that
+            # starts from cached keys (the reference's attention operator cannot run this case either,
+            # src/nats/ops/attns/attns.py:1439,1491), so the tokens go through the decode path in steps of fewer than 64
+            # (one token per step where the mode's decode operator takes a single token)
+            step = 1 if self.ops_for_incomplete_chunks == 'gated_delta_net' else 63
+            kw = dict(past_key_values=past_key_values, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
+            outs = [self.forward(hidden_states[:, t:t + step], attention_mask, **kw)[0] for t in range(0, q_len, step)]
+            return torch.cat(outs, 1), None, past_key_values
         if cache is not None and cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported together with a cache")
 

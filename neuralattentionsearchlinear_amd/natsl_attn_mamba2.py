@@ -2,7 +2,7 @@
 the reference layer (src/nats/layers/natsl_attn_mamba2.py:100-599).  Same scope as the Gated-DeltaNet
 layer: trainable (the linear branch, the pooling and the norm-gate differentiate through torch operations, the
 softmax branch through its HIP backward); with a cache, one chunked prefill on the empty cache and then decode steps of
-fewer than 64 tokens."""
+fewer than 64 tokens (longer inputs on a filled cache are fed through the decode path in such steps)."""
 from __future__ import annotations
 
 import math
@@ -120,8 +120,15 @@ class NeuralAttentionSearchLinearAttnMamba(nn.Module):
         if cache is None and mode != 'chunk':
             raise ValueError("fewer than 64 tokens are decoded on a cache: pass cache_params")
         if cache is not None and mode == 'chunk' and cache.n_observed_tokens > 0:
-            raise NotImplementedError("a chunked forward that continues a non-empty cache is not built: prefill once, then "
-                                      "decode in steps of fewer than 64 tokens")
+            if cu_seqlens is not None:
+                raise NotImplementedError("packed sequences are not supported together with a cache")
+            # 64 or more new tokens on a cache that already holds tokens (a second prompt): there is no chunked kernel that
+            # starts from cached keys (the reference's attention operator cannot run this case either,
+            # src/nats/ops/attns/attns.py:1439,1491), so the tokens go through the decode path in steps of fewer than 64
+            # (one token per step where the mode's decode operator takes a single token)
+            step = 1 if self.ops_for_incomplete_chunks == 'mamba' else 63
+            kw = dict(cache_params=cache_params, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
+            return torch.cat([self.forward(hidden_states[:, t:t + step], attention_mask, **kw) for t in range(0, q_len, step)], 1)
         if cache is not None and cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported together with a cache")
 

@@ -163,7 +163,7 @@ def test_layer_generation_matches_whole_forward(kind, T0, T, geometry):
     assert rl0 <= 2e-2, f"prefilled tokens: rel-L2 {rl0:.3e}"
 
 
-def test_layer_rejects_what_the_cache_cannot_do():
+def test_single_token_steps_after_a_prefill_are_repeatable():
     from neuralattentionsearchlinear_amd.cache import NAtSCache
     layer, cfg, w, x = _layer_case('gdn')
     layer.layer_idx = 0
@@ -172,8 +172,6 @@ def test_layer_rejects_what_the_cache_cannot_do():
     cache = NAtSCache()
     with torch.no_grad():
         layer(xd[:, :100], past_key_values=cache, use_cache=True)
-        with pytest.raises(NotImplementedError):
-            layer(xd[:, 100:200], past_key_values=cache, use_cache=True)      # a second chunked forward
         # a refused step leaves the cache as it was: the same tokens fed one at a time afterwards give what an
         # untouched cache gives
         fresh = NAtSCache()
@@ -210,3 +208,29 @@ def test_decode_step_across_a_block_boundary(kind):
         # and the two caches go on alike
         a2, b2 = first(layer(xd[:, 140:141], **kw(a_h))), first(layer(xd[:, 140:141], **kw(b_h)))
         assert rel_l2(a2.float(), b2.float()) <= 1e-3
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+def test_long_continuation_on_a_filled_cache(kind):
+    """64 or more new tokens on a cache that already holds tokens (a second prompt) run through the decode path in steps:
+    same outputs and cache state as the tokens one at a time, and close to the whole forward."""
+    from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
+    layer, cfg, w, x = _layer_case(kind)
+    layer.layer_idx = 0
+    layer = layer.to(DEV).to(torch.bfloat16).eval()
+    xd = x.to(DEV).bfloat16()                                           # 320 tokens
+    first = lambda out: out[0] if isinstance(out, tuple) else out
+    mk = (lambda: NAtSCache()) if kind == 'gdn' else (lambda: NAtSMamba2Cache())
+    kw = lambda h: dict(past_key_values=h, use_cache=True) if kind == 'gdn' else dict(cache_params=h, use_cache=True)
+    with torch.no_grad():
+        whole = first(layer(xd))
+        a_h, b_h = mk(), mk()
+        layer(xd[:, :100], **kw(a_h))
+        layer(xd[:, :100], **kw(b_h))
+        a = first(layer(xd[:, 100:300], **kw(a_h)))                     # 200 tokens at once
+        b = torch.cat([first(layer(xd[:, t:t + 1], **kw(b_h))) for t in range(100, 300)], 1)
+    assert a.shape == b.shape == (2, 200, xd.shape[-1])
+    assert rel_l2(a.float(), b.float()) <= 1e-3, f"against single-token steps: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
+    assert rel_l2(a.float(), whole[:, 100:300].float()) <= 2e-2, f"against the whole forward: rel-L2 {rel_l2(a.float(), whole[:, 100:300].float()):.3e}"
+    ca, cb = (h[0] if kind == 'gdn' else h.nats_cache[0] for h in (a_h, b_h))
+    assert ca.n_observed_tokens == cb.n_observed_tokens == 300 and torch.equal(ca.n_attn_blocks, cb.n_attn_blocks)
