@@ -57,23 +57,26 @@ def make_inputs(w, torch, device):
     B, T, H, K, V = w["B"], w["T"], w["H"], w["K"], w["V"]
     if w.get("kind") == "mamba":
         # C (as q) and B (as k) ~ N(0,1), one group shared by all heads; X ~ N(0,1); log-decay dt * A with
-        # dt = softplus(N(0,1) - 4), A = -exp(U(0, log 16)) per head
+        # dt = softplus(N(0,1) - 4), A = -exp(U(0, log 16)) per head.  The linear branch takes X * dt as its values, the
+        # attention branch the unscaled X (src/nats/layers/natsl_attn_mamba2.py:391-393, :473).
         q = torch.randn(B, T, 1, K, generator=g).expand(B, T, H, K).contiguous().bfloat16()
         k = torch.randn(B, T, 1, K, generator=g).expand(B, T, H, K).contiguous().bfloat16()
-        v = torch.randn(B, T, H, V, generator=g).bfloat16()
+        x = torch.randn(B, T, H, V, generator=g)
         beta = torch.ones(B, T, H).bfloat16()
         dt = F.softplus(torch.randn(B, T, H, generator=g) - 4.0)
         gl = -torch.exp(torch.rand(H, generator=g) * math.log(16.0)) * dt
+        v, v_l = x.bfloat16(), (x * dt[..., None]).bfloat16()
     else:
         q = torch.randn(B, T, H, K, generator=g).bfloat16()
         k = torch.randn(B, T, H, K, generator=g).bfloat16()
         v = torch.randn(B, T, H, V, generator=g).bfloat16()
         beta = torch.sigmoid(torch.randn(B, T, H, generator=g)).bfloat16()
         gl = -F.softplus(torch.randn(B, T, H, generator=g))
+        v_l = v
     logits = torch.randn(B, T // w["block"], H, 2, generator=g)
     logits[..., 1] += selector_bias(w["p_attn"])
     logits = logits.bfloat16()
-    host = dict(q=q, k=k, v=v, beta=beta, g=gl, logits=logits)
+    host = dict(q=q, k=k, v=v, v_l=v_l, beta=beta, g=gl, logits=logits)
     dev = {n: t.to(device) for n, t in host.items()}
     return host, dev
 
@@ -158,11 +161,11 @@ def cpu_baseline(host, w, types_host, torch, max_heads=None, max_batch=None):
     H = w["H"] if max_heads is None else min(w["H"], max_heads)
     Bs = w["B"] if max_batch is None else min(w["B"], max_batch)
     sl = lambda t: t[:Bs, :, :H].contiguous()
-    q, k, v, beta, g = (sl(host[n]) for n in ("q", "k", "v", "beta", "g"))
+    q, k, v, v_l, beta, g = (sl(host[n]) for n in ("q", "k", "v", "v_l", "beta", "g"))
     ty = types_host[:Bs, :, :H].contiguous()
     t0 = time.perf_counter()
     if w.get("kind") == "mamba":
-        mixed.mixed_attn_mamba(q, k, v, q, k, v, None, g, ty, scale_lattn=1.0, ops_for_incomplete_chunks='all', output_final_state=True,
+        mixed.mixed_attn_mamba(q, k, v, q, k, v_l, None, g, ty, scale_lattn=1.0, ops_for_incomplete_chunks='all', output_final_state=True,
                                decay_for_non_mamba_blocks=True, nats_block_size=w["block"])
     else:
         mixed.mixed_attn_gdn(q, k, v, q, k, v, None, g, beta, ty, ops_for_incomplete_chunks='all', output_final_state=True,
@@ -361,7 +364,7 @@ def main():
     def step():
         ty, nb = nats_util.hard_select(dev["logits"], force_last_block=True)
         if is_mamba:
-            return nats_mixed_attn_mamba(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v"], None, dev["g"], ty, nb,
+            return nats_mixed_attn_mamba(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v_l"], None, dev["g"], ty, nb,
                                          scale_lattn=1.0, nats_block_size=w["block"], ops_for_incomplete_chunks="all",
                                          output_final_state_mamba=True, decay_for_non_mamba_blocks=True), ty
         return nats_mixed_attn_gdn(dev["q"], dev["k"], dev["v"], dev["q"], dev["k"], dev["v"], None, dev["g"], dev["beta"], ty,
