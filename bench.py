@@ -432,7 +432,7 @@ def main():
     # the linear branch (prep + scan kernels): algorithmic bytes = q, k, v read once, o written once, g and beta, final state
     # (the Mamba workload's B and C are stored per head here, as the operator takes them, and counted so)
     lin_bytes = B * T * H * (2 * K + 2 * V) * 2 + B * T * H * (4 if is_mamba else 6) + B * H * K * V * 4
-    roof_lin = dict(bound="hbm", kernel="linear_prep_kernel+linear_scan_kernel", achieved=lin_bytes / (lin_ms * 1e-3) / 1e9,
+    roof_lin = dict(bound="hbm", kernel=("mamba_scale_kernel" if is_mamba else "linear_prep_kernel") + "+linear_scan_kernel", achieved=lin_bytes / (lin_ms * 1e-3) / 1e9,
                     peak=PEAK_HBM_GBS, unit="GB/s", frac=lin_bytes / (lin_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     traffic=(traffic or {}).get("linear_bytes"), launch_ms=lin_ms, algorithmic_bytes=lin_bytes,
                     algorithmic_flops=f_gdn, frac_of_mfma_peak=f_gdn / (lin_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,

@@ -31,6 +31,9 @@
 //                        A block that is not typed linear leaves S rolled back at its end (times
 //                        e^{sum g} when decay is on), which is all the reference's carry logic
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
+//
+// The Mamba form has no solve: its prep is mamba_scale_kernel (the scale vectors only; q and k are not read), and the
+// scan forms P itself, in registers, from the k and q tiles of the stage.
 #include "natsl_device.h"
 #include "natsl_host.h"
 
@@ -339,6 +342,50 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) 
   }
 }
 
+// The Mamba form needs no Gram products ahead of the scan (its intra-chunk matrix is formed in the scan from the k, q tiles
+// that are in LDS anyway): what is left of the prep is the chunk's scale vectors, one wave per chunk-head, nothing read
+// but g and the block type:  sc = { gamma log2(e), scale e^{gamma}, e^{min(gamma_last - gamma, 0)}, {e^{gamma_last}, gamma_last, is_linear} }.
+__global__ __launch_bounds__(256) void mamba_scale_kernel(const LinearParams p) {
+  const int lane = threadIdx.x & 63;
+  const long long unit = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= (long long)p.total_chunks * p.H) return;
+  const int gc = (int)(unit / p.H), h = (int)(unit % p.H);
+  int bos, len, c, bos_nats;
+  if (p.seqs == nullptr) {
+    const int n = gc / p.nt;
+    c = gc - n * p.nt;
+    bos = n * p.T;
+    len = p.T;
+    bos_nats = n * p.TN;
+  } else {
+    int n = 0;
+    for (int i = 1; i < p.n_seqs; ++i)
+      if (p.seqs[i].chunk_off <= gc) n = i;
+    c = gc - p.seqs[n].chunk_off;
+    bos = p.seqs[n].bos;
+    len = p.seqs[n].eos - bos;
+    bos_nats = p.seqs[n].bos_nats;
+  }
+  const int t0 = c * C;
+  float x = t0 + lane < len ? p.g[(size_t)(bos + t0 + lane) * p.H + h] : 0.f;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const float y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  const float gl = __shfl(x, C - 1);
+  float* Sout = p.ws_sc + (size_t)unit * (4 * C);
+  Sout[lane] = x * 1.4426950408889634f;   // in log2 units: the scan forms e^{gamma_i - gamma_j} with one exp2 per element
+  Sout[C + lane] = p.scale * __expf(x);
+  Sout[2 * C + lane] = __expf(fminf(gl - x, 0.f));  // src/nats/ops/mamba/chunk_h.py:177
+  if (lane == 0) Sout[3 * C] = __expf(gl);
+  if (lane == 1) Sout[3 * C + 1] = gl;
+  if (lane == 2) {
+    const int hn = h / (p.H / p.HN);
+    Sout[3 * C + 2] = lin_type(p.types, p.types_dtype, ((size_t)(bos_nats + (c * C) / p.block) * p.HN + hn) * 2 + 1) ? 1.f : 0.f;
+  }
+}
+
 // =============================================================================================
 // scan
 // =============================================================================================
@@ -507,8 +554,10 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
 #pragma unroll
           for (int v = 0; v < 6; ++v) dma16(tb, ws_off[v], st + L::OFF_T + 1024 * v);
         }
+        if (DELTA) {
 #pragma unroll
-        for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
+          for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
+        }
       }
       kb += qk_step; vb += v_step; tb += ws_step; sb += sc_step;
     };
@@ -551,7 +600,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     // stores issued after them) may still be in flight at the barrier: vector memory operations complete in the order
     // they were issued, so allowing as many outstanding as one step issues leaves exactly the older step's complete.
     constexpr int AHEAD = L::NSTAGE - 1;
-    constexpr int PER_STEP_FIRST = 1 + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? 6 : 0) + 6 + O_PASSES;
+    constexpr int PER_STEP_FIRST = 1 + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? 12 : 0) + O_PASSES;
     static_assert(PER_STEP_FIRST <= 63 && PER_STEP_SECOND <= 63, "the wait counter has six bits");
     constexpr int VM_FIRST = (PER_STEP_FIRST & 15) | ((PER_STEP_FIRST >> 4) << 14) | 0x0f70;
     constexpr int VM_SECOND = (PER_STEP_SECOND & 15) | ((PER_STEP_SECOND >> 4) << 14) | 0x0f70;
@@ -620,6 +669,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
   const unsigned a_sc = 16u * g4;    // this lane group's four tokens in a row of sc
 
   float gsum = 0.f;
+  const float log2_scale = __builtin_amdgcn_logf(p.scale);
   __syncthreads();   // chunk 0 has landed
 
   for (int c = 0; c < NT; ++c) {
@@ -752,8 +802,48 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
 #pragma unroll
       for (int t = 0; t < 4; ++t) O[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * C + a_sc + 64 * t);
       if (intra) {
+        if constexpr (DELTA) {
 #pragma unroll
-        for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>(st + L::OFF_P + 1024 * v + 16 * lane);
+          for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>(st + L::OFF_P + 1024 * v + 16 * lane);
+        } else {
+          // P = scale tril(q k^T e^{gamma_i - gamma_j}) formed here, from the tiles of this stage: Z^T = k_tile(t') q_tile(t)^T
+          // leaves lane (i16, g4) with query 16 t + i16 against keys 16 t' + 4 g4 .. + 3 -- the four slots this lane holds of
+          // A operand (t, t' / 2), half t' % 2 (see the operand order above); both inputs are plain row reads, the k rows as
+          // A operand, the q rows as B operand (a lane's eight contraction slots = 16 bytes of its row).
+          f32x4 gj[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) gj[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + a_sc + 64 * t);
+          f32x4 Wt[4][4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            // (gamma comes in log2 units; the scale rides along as log2(scale))
+            const float gi = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (16 * t + i16)) + log2_scale;
+#pragma unroll
+            for (int t2 = 0; t2 < 4; ++t2) {
+              Wt[t][t2] = (f32x4){0.f, 0.f, 0.f, 0.f};
+              if (t2 <= t) {
+                f32x4 Z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KS; ++s) {
+                  const bf16x8 ka = *reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + t2 * 16 * L::KROW);
+                  const bf16x8 qb = *reinterpret_cast<lds_b128_t>(st + L::OFF_Q + a_kq[s] + t * 16 * L::KROW);
+                  Z = mfma16(ka, qb, Z);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  const float w = Z[r] * __builtin_amdgcn_exp2f(gi - gj[t2][r]);
+                  Wt[t][t2][r] = (t2 < t || i16 >= 4 * g4 + r) ? w : 0.f;
+                }
+              }
+            }
+          }
+          PA[tri_slot(0, 0)] = pack8(Wt[0][0], Wt[0][1]);
+          PA[tri_slot(1, 0)] = pack8(Wt[1][0], Wt[1][1]);
+          PA[tri_slot(2, 0)] = pack8(Wt[2][0], Wt[2][1]);
+          PA[tri_slot(2, 1)] = pack8(Wt[2][2], Wt[2][3]);
+          PA[tri_slot(3, 0)] = pack8(Wt[3][0], Wt[3][1]);
+          PA[tri_slot(3, 1)] = pack8(Wt[3][2], Wt[3][3]);
+        }
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t)
@@ -825,7 +915,8 @@ template <int DK, bool DELTA>
 static int launch_linear(const LinearParams& p, hipStream_t stream, const char* what) {
   const long long units = (long long)p.total_chunks * p.H;
   if (units <= 0) return NATSL_OK;
-  hipLaunchKernelGGL((linear_prep_kernel<DK, DELTA>), dim3((unsigned)units), dim3(256), 0, stream, p);
+  if constexpr (DELTA) hipLaunchKernelGGL((linear_prep_kernel<DK, true>), dim3((unsigned)units), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(mamba_scale_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, p);
   int rc = check_launch(what);
   if (rc != NATSL_OK) return rc;
   // Waves per workgroup (16 state columns each): the widest workgroup that still gives every CU one, so that the
