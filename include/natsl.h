@@ -170,6 +170,25 @@ int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const 
                         const void* w2, void* y, int64_t rows, int D, int dtype, float eps, int w_dtype,
                         natsl_stream_t stream);
 
+/* Layer glue, depthwise causal short convolution with its activation, on the layer's token-major tensors:
+ * y[b,t,d] = act(bias[d] + sum_j w[d,j] e[b, t-(W-1)+j, d]) where e is x preceded by the W-1 inputs before it: the last
+ * W-1 entries of `state` [B,D,W] (the cache of a previous call, in `state_dtype`), or zeros when state is NULL.
+ * x, y [B,T,D] in `dtype` (f32 or bf16; sums in f32, one rounding); weight [D,W] (the [D,1,W] of a Conv1d), bias [D] or NULL
+ * in `w_dtype`; activation 0 = none, 1 = silu; W in {2, 3, 4}; D % 8 == 0.
+ * Replaces the forward of flash-linear-attention's ShortConvolution as called at
+ * src/nats/layers/natsl_attn_gdn.py:425-491 and src/nats/layers/natsl_attn_mamba2.py:368-425. */
+int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, int B, int T, int D,
+                         int W, int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream);
+
+/* Layer glue, row normalisation: y = x * rsqrt(mean(x^2) + eps) * weight (l2 = 0, RMSNorm; weight [D] in `w_dtype` or NULL
+ * for none) or y = x * rsqrt(sum(x^2) + eps) (l2 = 1).  x, y [rows, D] in `dtype` (f32 or bf16), arithmetic in f32.
+ * D in {32, 64, 96, 128, 192, 256, 384, 512}.
+ * Replaces the RMSNorm of the attention view's q and k (flash-linear-attention's, called at
+ * src/nats/layers/natsl_attn_gdn.py:504-505) and the L2 normalisation of the Mamba layer's B and C
+ * (src/nats/layers/natsl_attn_mamba2.py:469-470). */
+int natsl_row_norm_fwd(const void* x, const void* weight, void* y, int64_t rows, int D, float eps, int l2, int dtype,
+                       int w_dtype, natsl_stream_t stream);
+
 /* Decode: T tokens that continue the current (incomplete) selector block of N cached sequences, token by
  * token.  Per token: S *= e^g; d = beta (v - S^T k); S += k d^T; o = scale S^T q (k, q L2-normalised with
  * NATSL_QK_L2NORM).  Only the first min(T, block - n_tokens_in_block) tokens are processed.  If they

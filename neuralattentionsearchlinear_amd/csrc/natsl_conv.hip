@@ -1,0 +1,215 @@
+// Layer glue around the mixed operator, forward: the depthwise causal short convolution with its activation, and the
+// RMS / L2 normalisation of head rows.  Both are HBM-bound and work on the layer's own token-major tensors ([B,T,D] and
+// [rows,D]): no transposed copies, one read and one write of the activations.
+//
+//   short_conv_kernel   y[b,t,d] = act(bias[d] + sum_j w[d,j] e[b, t-(W-1)+j, d]),  e = the W-1 inputs before the
+//                       sequence (from a cached state, else zeros) followed by x.  This is what the reference's
+//                       ShortConvolution (flash-linear-attention, called at src/nats/layers/natsl_attn_gdn.py:425-491)
+//                       computes: a causal cross-correlation with the kernel's last tap on the current token.
+//   row_norm_kernel     y = x * rsqrt(mean(x^2) + eps) * weight   (RMSNorm, src/nats/layers/natsl_attn_gdn.py:504-505)
+//                       y = x * rsqrt(sum(x^2) + eps)             (L2Norm of the Mamba layer's B and C)
+#include "natsl_device.h"
+#include "natsl_host.h"
+
+namespace natsl {
+
+NATSL_DEVICE void unpack8_bf16(const u32x4 w, float* f) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = __uint_as_float(w[j] << 16);
+    f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+  }
+}
+
+// eight adjacent channels of one row, as floats
+template <bool F32>
+NATSL_DEVICE void load8(const void* base, const size_t elem, float* f) {
+  if constexpr (F32) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { f[j] = a[j]; f[4 + j] = b[j]; }
+  } else {
+    unpack8_bf16(*reinterpret_cast<const u32x4*>(reinterpret_cast<const bf16_t*>(base) + elem), f);
+  }
+}
+template <bool F32>
+NATSL_DEVICE void store8(void* base, const size_t elem, const float* f) {
+  if constexpr (F32) {
+    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem) = (f32x4){f[0], f[1], f[2], f[3]};
+    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem + 4) = (f32x4){f[4], f[5], f[6], f[7]};
+  } else {
+    u32x4 w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
+    *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(base) + elem) = w;
+  }
+}
+NATSL_DEVICE float ld1(const void* p, const bool f32, const size_t i) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : bf16_to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+
+// A thread owns 8 adjacent channels for a run of `run` consecutive tokens of one sequence and slides a window of the last
+// W-1 rows through registers: every row is read once (plus W-1 rows at the start of each run).  Adjacent threads take
+// adjacent channel groups, so a row is read and written in whole 16-byte (bf16) or 32-byte (fp32) pieces side by side.
+template <int W, bool F32>
+__global__ __launch_bounds__(256) void short_conv_kernel(const void* x, const void* w, const void* bias, const void* state,
+                                                         void* y, const int B, const int T, const int D, const int run,
+                                                         const int silu, const bool w_f32, const bool state_f32) {
+  const int groups = D / 8, runs = (T + run - 1) / run;
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (long long)B * runs * groups) return;
+  const int cg = (int)(gid % groups);
+  const int r = (int)((gid / groups) % runs), b = (int)(gid / ((long long)groups * runs));
+  const int d0 = 8 * cg, t0 = r * run, t1 = min(T, t0 + run);
+  float wt[W][8], bs[8], win[W][8];   // win[j] = the input W-1-j rows back; win[W-1] is the current row
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+#pragma unroll
+    for (int j = 0; j < W; ++j) wt[j][c] = ld1(w, w_f32, (size_t)(d0 + c) * W + j);
+    bs[c] = bias ? ld1(bias, w_f32, d0 + c) : 0.f;
+  }
+  // the W-1 rows before the run: earlier tokens, else the cached state [B,D,W] (its last W-1 entries), else zeros
+#pragma unroll
+  for (int j = 0; j < W - 1; ++j) {
+    const int s = t0 - (W - 1) + j;
+    if (s >= 0) {
+      load8<F32>(x, ((size_t)b * T + s) * D + d0, win[j]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) win[j][c] = state ? ld1(state, state_f32, ((size_t)b * D + d0 + c) * W + (W + s)) : 0.f;
+    }
+  }
+  // eight rows are requested before the first of them is used: a thread's loads are otherwise one dependent round trip
+  // to memory per row
+  constexpr int AHEAD = 8;
+  auto one_row = [&](const float* in, const int t) __attribute__((always_inline)) {
+    float o[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      win[W - 1][c] = in[c];
+      float acc = bs[c];
+#pragma unroll
+      for (int j = 0; j < W; ++j) acc += wt[j][c] * win[j][c];
+      o[c] = silu ? acc / (1.f + __expf(-acc)) : acc;
+    }
+    store8<F32>(y, ((size_t)b * T + t) * D + d0, o);
+#pragma unroll
+    for (int j = 0; j < W - 1; ++j)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) win[j][c] = win[j + 1][c];
+  };
+  int tb = t0;
+  for (; tb + AHEAD <= t1; tb += AHEAD) {   // (no conditions around the loads: they all go out before the first wait)
+    float rows[AHEAD][8];
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) load8<F32>(x, ((size_t)b * T + tb + a) * D + d0, rows[a]);
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) one_row(rows[a], tb + a);
+  }
+  for (; tb < t1; ++tb) {
+    float row[8];
+    load8<F32>(x, ((size_t)b * T + tb) * D + d0, row);
+    one_row(row, tb);
+  }
+}
+
+// A row is handled by LANES adjacent lanes with PER pieces of 8 elements each (D = 8 LANES PER).
+template <int LANES, int PER, bool F32>
+__global__ __launch_bounds__(256) void row_norm_kernel(const void* x, const void* weight, void* y, const long long rows, const float eps,
+                                                       const int l2, const bool w_f32) {
+  constexpr int D = LANES * PER * 8;
+  const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / LANES;
+  const int seg = threadIdx.x % LANES;
+  if (row >= rows) return;  // whole row groups exit together: LANES divides 64
+  float v[PER][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    load8<F32>(x, (size_t)row * D + (u * LANES + seg) * 8, v[u]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += v[u][j] * v[u][j];
+  }
+#pragma unroll
+  for (int d = 1; d < LANES; d <<= 1) ss += __shfl_xor(ss, d);
+  const float rs = rsqrtf((l2 ? ss : ss / D) + eps);
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int col = (u * LANES + seg) * 8;
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = v[u][j] * rs * (weight ? ld1(weight, w_f32, col + j) : 1.f);
+    store8<F32>(y, (size_t)row * D + col, o);
+  }
+}
+
+}  // namespace natsl
+
+using namespace natsl;
+
+extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, int B, int T, int D,
+                                    int W, int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream) {
+  const char* what = "natsl_short_conv_fwd";
+  if (!x || !weight || !y) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: activations must be f32 or bf16", what);
+  if (w_dtype != NATSL_BF16 && w_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: weights must be f32 or bf16", what);
+  if (state && state_dtype != NATSL_BF16 && state_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: the state must be f32 or bf16", what);
+  if (B <= 0 || T <= 0 || D <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
+  if (D % 8) return fail(NATSL_ERR_UNSUPPORTED, "%s: D=%d must be a multiple of 8", what, D);
+  if (activation != 0 && activation != 1) return fail(NATSL_ERR_INVALID, "%s: activation must be 0 (none) or 1 (silu)", what);
+  // long runs read the fewest rows twice; short ones are needed to give every CU work on small inputs
+  int run = 32;
+  while (run > 8 && (long long)B * cdiv(T, run) * (D / 8) < 256 * 256) run >>= 1;
+  const long long threads = (long long)B * cdiv(T, run) * (D / 8);
+  const dim3 grid((unsigned)((threads + 255) / 256));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool f32 = dtype == NATSL_F32;
+#define NATSL_CONV(WW)                                                                                                        \
+  {                                                                                                                           \
+    if (f32) hipLaunchKernelGGL((short_conv_kernel<WW, true>), grid, dim3(256), 0, s, x, weight, bias, state, y, B, T, D, run, \
+                                activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                   \
+    else hipLaunchKernelGGL((short_conv_kernel<WW, false>), grid, dim3(256), 0, s, x, weight, bias, state, y, B, T, D, run,    \
+                            activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                       \
+    return check_launch(what);                                                                                                \
+  }
+  switch (W) {
+    case 2: NATSL_CONV(2)
+    case 3: NATSL_CONV(3)
+    case 4: NATSL_CONV(4)
+    default: return fail(NATSL_ERR_UNSUPPORTED, "%s: kernel size %d not built (2, 3, 4)", what, W);
+  }
+#undef NATSL_CONV
+}
+
+extern "C" int natsl_row_norm_fwd(const void* x, const void* weight, void* y, int64_t rows, int D, float eps, int l2, int dtype,
+                                  int w_dtype, natsl_stream_t stream) {
+  const char* what = "natsl_row_norm_fwd";
+  if (!x || !y) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: activations must be f32 or bf16", what);
+  if (weight && w_dtype != NATSL_BF16 && w_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: weights must be f32 or bf16", what);
+  if (rows <= 0) return NATSL_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool f32 = dtype == NATSL_F32;
+#define NATSL_RN(L, P)                                                                                                          \
+  {                                                                                                                             \
+    const long long threads = rows * (L);                                                                                       \
+    const dim3 grid((unsigned)((threads + 255) / 256));                                                                         \
+    if (f32) hipLaunchKernelGGL((row_norm_kernel<L, P, true>), grid, dim3(256), 0, s, x, weight, y, (long long)rows, eps, l2,    \
+                                w_dtype == NATSL_F32);                                                                           \
+    else hipLaunchKernelGGL((row_norm_kernel<L, P, false>), grid, dim3(256), 0, s, x, weight, y, (long long)rows, eps, l2,       \
+                            w_dtype == NATSL_F32);                                                                               \
+    return check_launch(what);                                                                                                  \
+  }
+  switch (D) {
+    case 32: NATSL_RN(4, 1)
+    case 64: NATSL_RN(8, 1)
+    case 96: NATSL_RN(4, 3)
+    case 128: NATSL_RN(16, 1)
+    case 192: NATSL_RN(8, 3)
+    case 256: NATSL_RN(32, 1)
+    case 384: NATSL_RN(16, 3)
+    case 512: NATSL_RN(64, 1)
+    default: return fail(NATSL_ERR_UNSUPPORTED, "%s: row width %d not built (32, 64, 96, 128, 192, 256, 384, 512)", what, D);
+  }
+#undef NATSL_RN
+}

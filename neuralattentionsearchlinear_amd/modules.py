@@ -2,8 +2,9 @@
 
 The reference takes these from flash-linear-attention (ShortConvolution, RMSNorm, L2Norm) and from
 src/nats/modules/fused_norm_gate.py (FusedMultiInputRMSNormGated); parameter names are kept so that
-reference checkpoints load.  Projections and the short convolution stay torch ops (rocBLAS / MIOpen);
-the two-input norm-gate runs the HIP kernel natsl_norm_gate_fwd.
+reference checkpoints load.  Projections stay torch ops (rocBLAS); the short convolution, the RMS / L2 row norms and the
+two-input norm-gate run HIP kernels (natsl_short_conv_fwd, natsl_row_norm_fwd, natsl_norm_gate_fwd) in the forward, with
+torch-evaluated gradients.
 """
 from __future__ import annotations
 
@@ -16,6 +17,63 @@ import torch.nn.functional as F
 from . import _capi
 
 
+_ROW_NORM_WIDTHS = (32, 64, 96, 128, 192, 256, 384, 512)
+
+
+def _row_norm_torch(x, weight, eps, l2):
+    xf = x.float()
+    ss = xf.pow(2).sum(-1, keepdim=True) if l2 else xf.pow(2).mean(-1, keepdim=True)
+    y = xf * torch.rsqrt(ss + eps)
+    if weight is not None:
+        y = y * weight.float()
+    return y.to(x.dtype)
+
+
+def _row_norm_fwd(x, weight, eps, l2):
+    """natsl_row_norm_fwd on [..., D] (fp32 arithmetic, result in x's dtype)."""
+    D = x.shape[-1]
+    xc = x.detach().contiguous()
+    w = None if weight is None else weight.detach().contiguous()
+    if w is not None and w.dtype not in (torch.float32, torch.bfloat16):
+        w = w.float()
+    y = torch.empty_like(xc)
+    rc = _capi.lib().natsl_row_norm_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(y), xc.numel() // D, D, float(eps), int(l2),
+                                        _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype) if w is not None else _capi.F32,
+                                        _capi.stream_ptr(xc.device))
+    _capi.check(rc, "natsl_row_norm_fwd")
+    return y
+
+
+class _RowNorm(torch.autograd.Function):
+    """The HIP forward with the gradients of the same formula evaluated as fp32 torch operations."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps, l2):
+        ctx.save_for_backward(x, weight)
+        ctx.eps, ctx.l2 = eps, l2
+        return _row_norm_fwd(x, weight, eps, l2)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        with torch.enable_grad():
+            xf = x.detach().float().requires_grad_(True)
+            wf = None if weight is None else weight.detach().float().requires_grad_(True)
+            y = _row_norm_torch(xf, wf, ctx.eps, ctx.l2)
+            grads = torch.autograd.grad(y, (xf,) if wf is None else (xf, wf), dy.float())
+        return grads[0].to(x.dtype), (None if wf is None else grads[1].to(weight.dtype)), None, None
+
+
+def row_norm(x, weight, eps: float, l2: bool):
+    """RMSNorm (l2=False, optional weight) or L2 normalisation (l2=True) of the last dimension: the HIP kernel for f32 / bf16
+    tensors on the GPU with a supported width, else the same formula as torch operations."""
+    if not (x.is_cuda and x.dtype in (torch.float32, torch.bfloat16) and x.shape[-1] in _ROW_NORM_WIDTHS and x.numel() > 0):
+        return _row_norm_torch(x, weight, eps, l2)
+    if torch.is_grad_enabled() and (x.requires_grad or (weight is not None and weight.requires_grad)):
+        return _RowNorm.apply(x, weight, eps, l2)
+    return _row_norm_fwd(x, weight, eps, l2)
+
+
 class RMSNorm(nn.Module):
     def __init__(self, hidden_size: int, eps: float = 1e-5):
         super().__init__()
@@ -23,9 +81,7 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size))
 
     def forward(self, x):
-        xf = x.float()
-        y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
-        return y.to(x.dtype)
+        return row_norm(x, self.weight, self.eps, False)
 
 
 class L2Norm(nn.Module):
@@ -34,12 +90,71 @@ class L2Norm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        xf = x.float()
-        return (xf * torch.rsqrt(xf.pow(2).sum(-1, keepdim=True) + self.eps)).to(x.dtype)
+        return row_norm(x, None, self.eps, True)
+
+
+def _short_conv_torch(x, weight, bias, cache, activation):
+    """[B,T,D] -> [B,T,D]: the causal depthwise convolution as torch operations (weight [D,1,W])."""
+    B, T, D = x.shape
+    W = weight.shape[-1]
+    xt = x.transpose(1, 2)
+    if cache is not None:
+        xt = torch.cat([cache.to(xt.dtype), xt], -1)
+        y = F.conv1d(xt, weight, bias, groups=D)[..., -T:]
+    else:
+        y = F.conv1d(xt, weight, bias, padding=W - 1, groups=D)[..., :T]
+    if activation is not None:
+        y = F.silu(y)
+    return y.transpose(1, 2)
+
+
+def _short_conv_fwd(x, weight, bias, cache, activation):
+    """natsl_short_conv_fwd: token-major in, token-major out, no transposed copies."""
+    B, T, D = x.shape
+    W = weight.shape[-1]
+    xc = x.detach().contiguous()
+    w = weight.detach().reshape(D, W).contiguous()
+    b = None if bias is None else bias.detach().to(w.dtype).contiguous()
+    if w.dtype not in (torch.float32, torch.bfloat16):
+        w, b = w.float(), (None if b is None else b.float())
+    st = None
+    if cache is not None:
+        st = cache.detach().contiguous()
+        if st.dtype not in (torch.float32, torch.bfloat16):
+            st = st.float()
+    y = torch.empty_like(xc)
+    rc = _capi.lib().natsl_short_conv_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(y), B, T, D, W,
+                                          0 if activation is None else 1, _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
+                                          _capi.dtype_code(st.dtype) if st is not None else _capi.F32, _capi.stream_ptr(xc.device))
+    _capi.check(rc, "natsl_short_conv_fwd")
+    return y
+
+
+class _ShortConv(torch.autograd.Function):
+    """The HIP forward with the gradients of the same convolution evaluated as torch operations."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, cache, activation):
+        ctx.save_for_backward(x, weight, bias, cache)
+        ctx.activation = activation
+        return _short_conv_fwd(x, weight, bias, cache, activation)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, bias, cache = ctx.saved_tensors
+        with torch.enable_grad():
+            xf = x.detach().float().requires_grad_(True)
+            wf = weight.detach().float().requires_grad_(True)
+            bf = None if bias is None else bias.detach().float().requires_grad_(True)
+            y = _short_conv_torch(xf, wf, bf, None if cache is None else cache.detach().float(), ctx.activation)
+            wrt = (xf, wf) if bf is None else (xf, wf, bf)
+            grads = torch.autograd.grad(y, wrt, dy.float())
+        return (grads[0].to(x.dtype), grads[1].to(weight.dtype), None if bf is None else grads[2].to(bias.dtype), None, None)
 
 
 class ShortConvolution(nn.Conv1d):
-    """Depthwise causal convolution over time with optional SiLU; weight [hidden, 1, kernel] as in fla."""
+    """Depthwise causal convolution over time with optional SiLU; weight [hidden, 1, kernel] as in fla.  On the GPU the
+    forward is the HIP kernel natsl_short_conv_fwd (kernel sizes 2-4, hidden % 8 == 0, f32 / bf16), else torch's conv1d."""
 
     def __init__(self, hidden_size: int, kernel_size: int, bias: bool = False, activation: Optional[str] = 'silu'):
         super().__init__(hidden_size, hidden_size, kernel_size, groups=hidden_size, bias=bias, padding=kernel_size - 1)
@@ -52,20 +167,23 @@ class ShortConvolution(nn.Conv1d):
         if cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported by this ShortConvolution")
         B, T, D = x.shape
-        xt = x.transpose(1, 2)
         W = self.kernel_size[0]
-        if cache is not None:
-            xt = torch.cat([cache.to(xt.dtype), xt], -1)
-            y = F.conv1d(xt, self.weight, self.bias, groups=D)[..., -T:]
+        hip = x.is_cuda and W in (2, 3, 4) and D % 8 == 0 and x.dtype in (torch.float32, torch.bfloat16) and x.numel() > 0
+        if not hip:
+            y = _short_conv_torch(x, self.weight, self.bias, cache, self.activation)
+        elif torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad):
+            y = _ShortConv.apply(x, self.weight, self.bias, cache, self.activation)
         else:
-            y = F.conv1d(xt, self.weight, self.bias, padding=W - 1, groups=D)[..., :T]
+            y = _short_conv_fwd(x, self.weight, self.bias, cache, self.activation)
         final = None
         if output_final_state:
-            src = xt if cache is not None else F.pad(xt, (W, 0))
-            final = src[..., -W:].contiguous()
-        if self.activation is not None:
-            y = F.silu(y)
-        return y.transpose(1, 2), final
+            # the last W inputs, [B,D,W]: what the next call sees before its first token
+            tail = x[:, -W:].transpose(1, 2)
+            if T < W:
+                prev = cache.to(x.dtype)[..., -(W - T):] if cache is not None else x.new_zeros(B, D, W - T)
+                tail = torch.cat([prev, tail], -1)
+            final = tail.contiguous()
+        return y, final
 
 
 class FusedMultiInputRMSNormGated(nn.Module):

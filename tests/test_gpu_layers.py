@@ -1,6 +1,7 @@
 """GPU parity: layer tail (two-input norm-gate) and the two hybrid layer modules vs the oracle."""
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import layer as olayer
 from oracle import norm_gate as ong
@@ -176,3 +177,77 @@ def test_layer_rejects_unbuilt_paths():
     layer = layer.to(DEV).to(torch.bfloat16).eval()
     with pytest.raises(ValueError):
         layer(x[:, :32].to(DEV).bfloat16())                       # decoding needs a cache
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("W,D,act,bias", [(4, 768, 'silu', False), (4, 1536, 'silu', True), (3, 64, None, True), (2, 8, 'silu', False)])
+def test_short_convolution(W, D, act, bias, dtype):
+    """natsl_short_conv_fwd against the oracle's convolution (torch conv1d in fp32 on the same inputs): whole sequences,
+    a continuation from a cached state (two pieces == one piece), pieces shorter than the kernel, and the gradients."""
+    from neuralattentionsearchlinear_amd.modules import ShortConvolution
+    g = torch.Generator().manual_seed(W * D)
+    conv = ShortConvolution(D, W, bias=bias, activation=act)
+    with torch.no_grad():
+        conv.weight.copy_(torch.randn(conv.weight.shape, generator=g) * 0.5)
+        if bias:
+            conv.bias.copy_(torch.randn(D, generator=g) * 0.1)
+    conv = conv.to(DEV).to(dtype)
+    B, T = 3, 333
+    x = torch.randn(B, T, D, generator=g).to(dtype)
+    wf, bf = conv.weight.detach().float().cpu(), (conv.bias.detach().float().cpu() if bias else None)
+    ref = F.conv1d(x.float().transpose(1, 2), wf, bf, padding=W - 1, groups=D)[..., :T].transpose(1, 2)
+    if act is not None:
+        ref = F.silu(ref)
+    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    def close(a, what):
+        err = (a.float().cpu() - what).abs()
+        assert bool((err <= tol * what.abs() + tol).all()), f"short convolution: max-abs {float(err.max()):.3e}"
+    with torch.no_grad():
+        y, final = conv(x.to(DEV), output_final_state=True)
+        assert y.is_contiguous() and y.dtype == dtype and final.shape == (B, D, W)
+        close(y, ref)
+        assert torch.equal(final.cpu(), x[:, -W:].transpose(1, 2))
+        # two pieces through the state, the second shorter than the kernel, then single tokens
+        cut = 200
+        y1, st = conv(x[:, :cut].to(DEV), output_final_state=True)
+        y2, st = conv(x[:, cut:cut + 2].to(DEV), cache=st, output_final_state=True)
+        outs = [y1, y2]
+        for t in range(cut + 2, cut + 7):
+            yt, st = conv(x[:, t:t + 1].to(DEV), cache=st, output_final_state=True)
+            outs.append(yt)
+        y3, st = conv(x[:, cut + 7:].to(DEV), cache=st, output_final_state=True)
+        outs.append(y3)
+        close(torch.cat(outs, 1), ref)
+        assert torch.equal(st.cpu(), x[:, -W:].transpose(1, 2))
+    # gradients (HIP forward, torch-evaluated backward) against autograd through the fp32 formula
+    xd = x.to(DEV).requires_grad_(True)
+    yg, _ = conv(xd)
+    dy = torch.randn(B, T, D, generator=g)
+    (yg.float() * dy.to(DEV)).sum().backward()
+    xr = x.float().requires_grad_(True)
+    wr = wf.clone().requires_grad_(True)
+    yr = F.conv1d(xr.transpose(1, 2), wr, bf, padding=W - 1, groups=D)[..., :T].transpose(1, 2)
+    ((F.silu(yr) if act is not None else yr) * dy).sum().backward()
+    assert rel_l2(xd.grad.float(), xr.grad) <= 5e-3 and rel_l2(conv.weight.grad.float(), wr.grad) <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("D", [32, 64, 96, 128, 192, 256, 384, 512])
+def test_row_norms(D, dtype):
+    """natsl_row_norm_fwd: RMSNorm with weight and L2 normalisation of head rows against the fp32 formulas."""
+    from neuralattentionsearchlinear_amd.modules import L2Norm, RMSNorm
+    g = torch.Generator().manual_seed(D)
+    x = (torch.randn(2, 77, 5, D, generator=g) * 3).to(dtype)
+    rms, l2 = RMSNorm(D, eps=1e-5).to(DEV).to(dtype), L2Norm(eps=1e-6)
+    with torch.no_grad():
+        rms.weight.copy_((1 + 0.2 * torch.randn(D, generator=g)).to(dtype))
+        y1, y2 = rms(x.to(DEV)), l2(x.to(DEV))
+    xf, wf = x.float(), rms.weight.detach().float().cpu()
+    r1 = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5) * wf
+    r2 = xf * torch.rsqrt(xf.pow(2).sum(-1, keepdim=True) + 1e-6)
+    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    for y, r in ((y1, r1), (y2, r2)):
+        assert y.dtype == dtype and bool(((y.float().cpu() - r).abs() <= tol * r.abs() + 1e-6).all())
+    xd = x.to(DEV).requires_grad_(True)
+    (rms(xd).float().sum() + l2(xd).float().pow(2).sum()).backward()
+    assert xd.grad is not None and bool(torch.isfinite(xd.grad).all()) and rms.weight.grad is not None
