@@ -174,11 +174,13 @@ int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const 
  * y[b,t,d] = act(bias[d] + sum_j w[d,j] e[b, t-(W-1)+j, d]) where e is x preceded by the W-1 inputs before it: the last
  * W-1 entries of `state` [B,D,W] (the cache of a previous call, in `state_dtype`), or zeros when state is NULL.
  * x, y [B,T,D] in `dtype` (f32 or bf16; sums in f32, one rounding); weight [D,W] (the [D,1,W] of a Conv1d), bias [D] or NULL
- * in `w_dtype`; activation 0 = none, 1 = silu; W in {2, 3, 4}; D % 8 == 0.
+ * in `w_dtype`; activation 0 = none, 1 = silu; W in {2, 3, 4}; D % 8 == 0.  state_out [B,D,W] in `dtype`, or NULL: the
+ * last W inputs of (state ++ x), what the next call takes as `state`; it must not alias `state`.
  * Replaces the forward of flash-linear-attention's ShortConvolution as called at
  * src/nats/layers/natsl_attn_gdn.py:425-491 and src/nats/layers/natsl_attn_mamba2.py:368-425. */
-int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, int B, int T, int D,
-                         int W, int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream);
+int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, void* state_out,
+                         int B, int T, int D, int W, int activation, int dtype, int w_dtype, int state_dtype,
+                         natsl_stream_t stream);
 
 /* Layer glue, row normalisation: y = x * rsqrt(mean(x^2) + eps) * weight (l2 = 0, RMSNorm; weight [D] in `w_dtype` or NULL
  * for none) or y = x * rsqrt(sum(x^2) + eps) (l2 = 1).  x, y [rows, D] in `dtype` (f32 or bf16), arithmetic in f32.
@@ -222,13 +224,14 @@ int natsl_mamba_recurrent_fwd(const void* q, const void* k, const void* v, const
  * visible, HM divides HQ; query head hq uses kv head hq/(HQ/HKV) and mask head hq/(HQ/HM).  A query that sees
  * no key gives 0.  With a workspace of natsl_attn_masked_workspace_bytes() the keys of one query are split over
  * several workgroups (needed to fill the GPU when B*TQ*HQ is small); with workspace = NULL one workgroup
- * handles a query.
+ * handles a query.  k_batch_stride / v_batch_stride: elements from one sequence's keys / values to the next, for keys that
+ * are the front part of a larger cache buffer [B,capacity,HKV,D] (a multiple of 8, at least TK*HKV*D); 0 = dense.
  * Replaces repeat_masks + torch.nn.functional.scaled_dot_product_attention at
  * src/nats/ops/mixed_ops/mixed_attn_gdn.py:475-481. */
 size_t natsl_attn_masked_workspace_bytes(int B, int TQ, int TK, int HQ, int V);
 int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
                           int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
-                          size_t workspace_bytes, natsl_stream_t stream);
+                          size_t workspace_bytes, int64_t k_batch_stride, int64_t v_batch_stride, natsl_stream_t stream);
 
 /* natsl_attn_masked_fwd for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc): the same kernels with the split scratch in a device array of the library itself, so the caller

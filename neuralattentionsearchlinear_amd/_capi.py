@@ -42,8 +42,8 @@ _SIGNATURES = {
                                       c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_size_t,
                                       c_int, c_void_p, c_int, c_int, c_void_p]),
-    "natsl_short_conv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                     c_int, c_void_p]),
+    "natsl_short_conv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_int, c_int, c_void_p]),
     "natsl_row_norm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_int, c_int, c_int, c_void_p]),
     "natsl_norm_gate_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                     c_float, c_int, c_void_p]),
@@ -55,7 +55,7 @@ _SIGNATURES = {
                                           c_float, c_int, c_int, c_void_p]),
     "natsl_attn_masked_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "natsl_attn_masked_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                      c_int, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+                                      c_int, c_int, c_float, c_int, c_void_p, c_size_t, c_int64, c_int64, c_void_p]),
     "natsl_attn_masked_static_scratch_bytes": (c_size_t, []),
     "natsl_attn_masked_fwd_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                              c_int, c_int, c_float, c_int, c_void_p]),

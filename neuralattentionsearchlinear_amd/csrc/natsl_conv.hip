@@ -54,7 +54,7 @@ NATSL_DEVICE float ld1(const void* p, const bool f32, const size_t i) {
 // adjacent channel groups, so a row is read and written in whole 16-byte (bf16) or 32-byte (fp32) pieces side by side.
 template <int W, bool F32>
 __global__ __launch_bounds__(256) void short_conv_kernel(const void* x, const void* w, const void* bias, const void* state,
-                                                         void* y, const int B, const int T, const int D, const int run,
+                                                         void* y, void* state_out, const int B, const int T, const int D, const int run,
                                                          const int silu, const bool w_f32, const bool state_f32) {
   const int groups = D / 8, runs = (T + run - 1) / run;
   const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -78,6 +78,27 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const void* x, const vo
     } else {
 #pragma unroll
       for (int c = 0; c < 8; ++c) win[j][c] = state ? ld1(state, state_f32, ((size_t)b * D + d0 + c) * W + (W + s)) : 0.f;
+    }
+  }
+  // the state the next call starts from: the last W inputs of (state ++ x), [B,D,W] in x's dtype, by the thread that owns
+  // the sequence's last run
+  if (state_out && r == runs - 1) {
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const int s = T - W + j;
+      float e[8];
+      if (s >= 0) {
+        load8<F32>(x, ((size_t)b * T + s) * D + d0, e);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) e[c] = state ? ld1(state, state_f32, ((size_t)b * D + d0 + c) * W + (W + s)) : 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const size_t o = ((size_t)b * D + d0 + c) * W + j;
+        if constexpr (F32) reinterpret_cast<float*>(state_out)[o] = e[c];
+        else reinterpret_cast<bf16_t*>(state_out)[o] = f32_to_bf16(e[c]);
+      }
     }
   }
   // eight rows are requested before the first of them is used: a thread's loads are otherwise one dependent round trip
@@ -147,8 +168,9 @@ __global__ __launch_bounds__(256) void row_norm_kernel(const void* x, const void
 
 using namespace natsl;
 
-extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, int B, int T, int D,
-                                    int W, int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream) {
+extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, void* state_out,
+                                    int B, int T, int D, int W, int activation, int dtype, int w_dtype, int state_dtype,
+                                    natsl_stream_t stream) {
   const char* what = "natsl_short_conv_fwd";
   if (!x || !weight || !y) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: activations must be f32 or bf16", what);
@@ -157,6 +179,7 @@ extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const voi
   if (B <= 0 || T <= 0 || D <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
   if (D % 8) return fail(NATSL_ERR_UNSUPPORTED, "%s: D=%d must be a multiple of 8", what, D);
   if (activation != 0 && activation != 1) return fail(NATSL_ERR_INVALID, "%s: activation must be 0 (none) or 1 (silu)", what);
+  if (state_out && state_out == state) return fail(NATSL_ERR_INVALID, "%s: state_out must not alias state (other threads still read it)", what);
   // long runs read the fewest rows twice; short ones are needed to give every CU work on small inputs
   int run = 32;
   while (run > 8 && (long long)B * cdiv(T, run) * (D / 8) < 256 * 256) run >>= 1;
@@ -166,9 +189,9 @@ extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const voi
   const bool f32 = dtype == NATSL_F32;
 #define NATSL_CONV(WW)                                                                                                        \
   {                                                                                                                           \
-    if (f32) hipLaunchKernelGGL((short_conv_kernel<WW, true>), grid, dim3(256), 0, s, x, weight, bias, state, y, B, T, D, run, \
+    if (f32) hipLaunchKernelGGL((short_conv_kernel<WW, true>), grid, dim3(256), 0, s, x, weight, bias, state, y, state_out, B, T, D, run, \
                                 activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                   \
-    else hipLaunchKernelGGL((short_conv_kernel<WW, false>), grid, dim3(256), 0, s, x, weight, bias, state, y, B, T, D, run,    \
+    else hipLaunchKernelGGL((short_conv_kernel<WW, false>), grid, dim3(256), 0, s, x, weight, bias, state, y, state_out, B, T, D, run,    \
                             activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                       \
     return check_launch(what);                                                                                                \
   }

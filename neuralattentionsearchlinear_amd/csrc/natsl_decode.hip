@@ -138,6 +138,7 @@ struct MaskedAttnParams {
   float scale_log2;
   int nsplit;        // workgroups per query, each owning every nsplit-th group of ATTN_WAVES chunks
   float* partials;   // nsplit > 1: [B, TQ, HQ, nsplit, 2 + DV] running (max, sum, accumulator) of each split
+  size_t k_bs, v_bs; // elements from one sequence's keys / values to the next (TK * HKV * D when dense)
 };
 
 template <int DK, int DV>
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
 #pragma unroll 4
       for (int pass = 0; pass < 16; ++pass) {
         const int kidx = min(k0 + 4 * pass + rowg, p.TK - 1);
-        const size_t kb = (((size_t)b * p.TK + kidx) * p.HKV + hkv) * DK + EPL * sub;
+        const size_t kb = (size_t)b * p.k_bs + ((size_t)kidx * p.HKV + hkv) * DK + EPL * sub;
         float d = 0.f;
         if (p.dtype == NATSL_BF16) {
           if (EPL == 8) {
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
 #pragma unroll 4
       for (int pass = 0; pass < 16; ++pass) {
         const int kidx = min(k0 + 4 * pass + rowg, p.TK - 1);   // keys past the end are clamped (their probability is 0)
-        const bf16_t* vrow = reinterpret_cast<const bf16_t*>(p.v) + (((size_t)b * p.TK + kidx) * p.HKV + hkv) * DV + EV * sub;
+        const bf16_t* vrow = reinterpret_cast<const bf16_t*>(p.v) + (size_t)b * p.v_bs + ((size_t)kidx * p.HKV + hkv) * DV + EV * sub;
         const float pk = sc[wave][4 * pass + rowg];
         u32x4 w;
         if (EV == 8) {
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_masked_kernel(const Mask
 #pragma unroll
       for (int u = 0; u < ATTN_VROWS; ++u) {
         const int kidx = min(k0 + kk + u, p.TK - 1);
-        const size_t vb = (((size_t)b * p.TK + kidx) * p.HKV + hkv) * DV + CPL * lane;
+        const size_t vb = (size_t)b * p.v_bs + ((size_t)kidx * p.HKV + hkv) * DV + CPL * lane;
         if (p.dtype == NATSL_BF16) {
           if (CPL == 2) {
             const unsigned w = *reinterpret_cast<const unsigned*>(reinterpret_cast<const bf16_t*>(p.v) + vb);
@@ -417,7 +418,8 @@ extern "C" size_t natsl_attn_masked_workspace_bytes(int B, int TQ, int TK, int H
 // instead of a silent fall-back to one workgroup per query.
 static int attn_masked_run(const char* what, const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
                            int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
-                           size_t workspace_bytes, bool strict, natsl_stream_t stream) {
+                           size_t workspace_bytes, bool strict, long long k_batch_stride, long long v_batch_stride,
+                           natsl_stream_t stream) {
   if (!q || !k || !v || !mask || !o) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: tensors must be f32 or bf16", what);
   if (B <= 0 || TQ <= 0 || TK <= 0 || HQ <= 0 || HKV <= 0 || HM <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
@@ -426,6 +428,11 @@ static int attn_masked_run(const char* what, const void* q, const void* k, const
   p.q = q; p.k = k; p.v = v; p.mask = mask; p.o = o;
   p.B = B; p.TQ = TQ; p.TK = TK; p.HQ = HQ; p.HKV = HKV; p.HM = HM; p.dtype = dtype;
   p.scale_log2 = scale * 1.4426950408889634f;
+  if ((k_batch_stride && k_batch_stride < (long long)TK * HKV * K) || (v_batch_stride && v_batch_stride < (long long)TK * HKV * V) ||
+      k_batch_stride % 8 || v_batch_stride % 8)
+    return fail(NATSL_ERR_INVALID, "%s: a batch stride must be 0 (dense) or at least TK*HKV*D, and a multiple of 8 elements", what);
+  p.k_bs = k_batch_stride ? (size_t)k_batch_stride : (size_t)TK * HKV * K;
+  p.v_bs = v_batch_stride ? (size_t)v_batch_stride : (size_t)TK * HKV * V;
   // without a workspace (or with one that is too small) every query is handled by one workgroup
   p.nsplit = attn_masked_splits(B, TQ, TK, HQ);
   const size_t need = natsl_attn_masked_workspace_bytes(B, TQ, TK, HQ, V);
@@ -454,9 +461,10 @@ static int attn_masked_run(const char* what, const void* q, const void* k, const
 
 extern "C" int natsl_attn_masked_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, int B, int TQ,
                                      int TK, int HQ, int HKV, int HM, int K, int V, float scale, int dtype, void* workspace,
-                                     size_t workspace_bytes, natsl_stream_t stream) {
+                                     size_t workspace_bytes, int64_t k_batch_stride, int64_t v_batch_stride,
+                                     natsl_stream_t stream) {
   return attn_masked_run("natsl_attn_masked_fwd", q, k, v, mask, o, B, TQ, TK, HQ, HKV, HM, K, V, scale, dtype, workspace,
-                         workspace_bytes, false, stream);
+                         workspace_bytes, false, k_batch_stride, v_batch_stride, stream);
 }
 
 // ---- the variant that allocates nothing -----------------------------------------------------------------------------
@@ -503,5 +511,5 @@ extern "C" int natsl_attn_masked_fwd_static(const void* q, const void* k, const 
   void* ws = scratch_device_address(what, &rc);
   if (!ws) return rc;
   return attn_masked_run(what, q, k, v, mask, o, B, TQ, TK, HQ, HKV, HM, K, V, scale, dtype, ws, NATSL_ATTN_STATIC_SCRATCH_BYTES,
-                         true, stream);
+                         true, 0, 0, stream);
 }

@@ -160,7 +160,16 @@ def masked_attention(q, k, v, attn_msk, scale):
     TK, HKV, V = k.shape[1], k.shape[2], v.shape[-1]
     if attn_msk.dim() != 4 or attn_msk.shape[0] != B or attn_msk.shape[2] != TQ or attn_msk.shape[3] != TK:
         raise ValueError(f"attn_msk must be [B, heads, {TQ}, {TK}], got {tuple(attn_msk.shape)}")
-    q, k, v = (t.contiguous() for t in (q, k, v))
+    q = q.contiguous()
+
+    def cache_view(t):
+        # the front part [:, :TK] of a cache buffer [B, capacity, H, D] is read in place (only its batch stride differs
+        # from a dense tensor's); anything else is made contiguous
+        D = t.shape[-1]
+        if t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == HKV * D and t.stride(0) >= TK * HKV * D and t.stride(0) % 8 == 0:
+            return t, t.stride(0)
+        return t.contiguous(), 0
+    (k, k_bs), (v, v_bs) = cache_view(k), cache_view(v)
     if not (q.dtype == k.dtype == v.dtype):
         raise ValueError("q, k, v must share a dtype")
     mask = attn_msk.to(torch.bool).contiguous().view(torch.uint8)
@@ -170,7 +179,7 @@ def masked_attention(q, k, v, attn_msk, scale):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     rc = L.natsl_attn_masked_fwd(_capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(mask), _capi.ptr(o), B, TQ, TK, HQ,
                                  HKV, mask.shape[1], K, V, float(scale), _capi.dtype_code(q.dtype), _capi.ptr(ws), ws_bytes,
-                                 _capi.stream_ptr(q.device))
+                                 k_bs, v_bs, _capi.stream_ptr(q.device))
     _capi.check(rc, "natsl_attn_masked_fwd")
     return o
 

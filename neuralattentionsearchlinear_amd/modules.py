@@ -108,8 +108,8 @@ def _short_conv_torch(x, weight, bias, cache, activation):
     return y.transpose(1, 2)
 
 
-def _short_conv_fwd(x, weight, bias, cache, activation):
-    """natsl_short_conv_fwd: token-major in, token-major out, no transposed copies."""
+def _short_conv_fwd(x, weight, bias, cache, activation, want_state=False):
+    """natsl_short_conv_fwd: token-major in, token-major out, no transposed copies -> (y, next state [B,D,W] or None)."""
     B, T, D = x.shape
     W = weight.shape[-1]
     xc = x.detach().contiguous()
@@ -123,11 +123,12 @@ def _short_conv_fwd(x, weight, bias, cache, activation):
         if st.dtype not in (torch.float32, torch.bfloat16):
             st = st.float()
     y = torch.empty_like(xc)
-    rc = _capi.lib().natsl_short_conv_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(y), B, T, D, W,
-                                          0 if activation is None else 1, _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
+    nxt = torch.empty(B, D, W, dtype=xc.dtype, device=xc.device) if want_state else None
+    rc = _capi.lib().natsl_short_conv_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(y), _capi.ptr(nxt), B, T, D,
+                                          W, 0 if activation is None else 1, _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
                                           _capi.dtype_code(st.dtype) if st is not None else _capi.F32, _capi.stream_ptr(xc.device))
     _capi.check(rc, "natsl_short_conv_fwd")
-    return y
+    return y, nxt
 
 
 class _ShortConv(torch.autograd.Function):
@@ -137,7 +138,7 @@ class _ShortConv(torch.autograd.Function):
     def forward(ctx, x, weight, bias, cache, activation):
         ctx.save_for_backward(x, weight, bias, cache)
         ctx.activation = activation
-        return _short_conv_fwd(x, weight, bias, cache, activation)
+        return _short_conv_fwd(x, weight, bias, cache, activation)[0]
 
     @staticmethod
     def backward(ctx, dy):
@@ -169,14 +170,14 @@ class ShortConvolution(nn.Conv1d):
         B, T, D = x.shape
         W = self.kernel_size[0]
         hip = x.is_cuda and W in (2, 3, 4) and D % 8 == 0 and x.dtype in (torch.float32, torch.bfloat16) and x.numel() > 0
+        final = None
         if not hip:
             y = _short_conv_torch(x, self.weight, self.bias, cache, self.activation)
         elif torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad):
             y = _ShortConv.apply(x, self.weight, self.bias, cache, self.activation)
         else:
-            y = _short_conv_fwd(x, self.weight, self.bias, cache, self.activation)
-        final = None
-        if output_final_state:
+            y, final = _short_conv_fwd(x, self.weight, self.bias, cache, self.activation, want_state=output_final_state)
+        if output_final_state and final is None:
             # the last W inputs, [B,D,W]: what the next call sees before its first token
             tail = x[:, -W:].transpose(1, 2)
             if T < W:

@@ -82,6 +82,25 @@ def test_masked_attention_against_oracle(K, V, TQ, TK, HM, dtype):
     assert float(o[0, 0, :HQ // HM].abs().max()) == 0.0
 
 
+def test_masked_attention_reads_a_cache_buffer_in_place():
+    """Keys / values that are the front part of a larger cache buffer [B, capacity, H, D] are read where they are (batch
+    stride = capacity * H * D): same result as on a dense copy, bit for bit, and the buffer's tail is never touched."""
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import masked_attention
+    B, HQ, HKV, HM, K, V, TQ, TK, cap = 3, 8, 4, 2, 64, 128, 2, 777, 1024
+    gen = torch.Generator().manual_seed(9)
+    q = torch.randn(B, TQ, HQ, K, generator=gen).bfloat16().to(DEV)
+    kbuf = torch.randn(B, cap, HKV, K, generator=gen).bfloat16().to(DEV)
+    vbuf = torch.randn(B, cap, HKV, V, generator=gen).bfloat16().to(DEV)
+    kbuf[:, TK:], vbuf[:, TK:] = float('nan'), float('nan')       # reading past TK would poison the result
+    mask = (torch.rand(B, HM, TQ, TK, generator=gen) < 0.4).to(DEV)
+    kv, vv = kbuf[:, :TK], vbuf[:, :TK]
+    assert not kv.is_contiguous()
+    a = masked_attention(q, kv, vv, mask, K ** -0.5)
+    b = masked_attention(q, kv.contiguous(), vv.contiguous(), mask, K ** -0.5)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(a.float()).all()) and torch.equal(a, b)
+
+
 @pytest.mark.parametrize("decay", [True, False])
 def test_prefill_then_decode_matches_whole_sequence(decay):
     """Prefill 3 blocks + 10 tokens with the chunked operator, then decode token by token through the end of

@@ -36,7 +36,7 @@ def _run(static, q, k, v, mask, K, V):
         need = L.natsl_attn_masked_workspace_bytes(B, TQ, TK, HQ, V)
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=DEV)
         rc = L.natsl_attn_masked_fwd(P(q), P(k), P(v), P(mask), P(o), B, TQ, TK, HQ, HKV, HM, K, V, scale, _capi.BF16, P(ws), need,
-                                     _capi.stream_ptr(q.device))
+                                     0, 0, _capi.stream_ptr(q.device))
         _capi.check(rc, "natsl_attn_masked_fwd")
     torch.cuda.synchronize()
     return o, need if not static else None
