@@ -182,6 +182,16 @@ int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, co
                          int B, int T, int D, int W, int activation, int dtype, int w_dtype, int state_dtype,
                          natsl_stream_t stream);
 
+/* Backward of natsl_short_conv_fwd: dx [B,T,D] in `dtype` (gradient of x; the cached state gets none), dweight fp32 [D,W],
+ * dbias fp32 [D] or NULL, from x, weight, bias, state as given to the forward and dy [B,T,D] in `dtype`.  The pre-activation
+ * is recomputed; the weight sums are reduced in a fixed order through the workspace
+ * (natsl_short_conv_bwd_workspace_bytes(), fp32 partial sums per run of tokens): no atomics, repeatable bits.
+ * Replaces the backward of flash-linear-attention's ShortConvolution under the same call sites. */
+size_t natsl_short_conv_bwd_workspace_bytes(int B, int T, int D, int W);
+int natsl_short_conv_bwd(const void* x, const void* weight, const void* bias, const void* state, const void* dy, void* dx,
+                         float* dweight, float* dbias, void* workspace, size_t workspace_bytes, int B, int T, int D, int W,
+                         int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream);
+
 /* Layer glue, row normalisation: y = x * rsqrt(mean(x^2) + eps) * weight (l2 = 0, RMSNorm; weight [D] in `w_dtype` or NULL
  * for none) or y = x * rsqrt(sum(x^2) + eps) (l2 = 1).  x, y [rows, D] in `dtype` (f32 or bf16), arithmetic in f32.
  * D in {32, 64, 96, 128, 192, 256, 384, 512}.

@@ -44,6 +44,9 @@ _SIGNATURES = {
                                       c_int, c_void_p, c_int, c_int, c_void_p]),
     "natsl_short_conv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_void_p]),
+    "natsl_short_conv_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "natsl_short_conv_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "natsl_row_norm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_int, c_int, c_int, c_void_p]),
     "natsl_norm_gate_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                     c_float, c_int, c_void_p]),

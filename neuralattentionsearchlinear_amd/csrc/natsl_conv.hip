@@ -135,6 +135,110 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const void* x, const vo
   }
 }
 
+// Backward of the short convolution.  With pre[t] = bias + sum_j w[j] e[t-(W-1)+j] and y = act(pre):
+//   dpre[t] = dy[t] act'(pre[t]);   dx[s] = sum_i w[W-1-i] dpre[s+i];   dw[j] = sum_{b,t} dpre[t] e[t-(W-1)+j];   dbias = sum dpre.
+// Same decomposition as the forward: a thread owns 8 channels for a run of tokens, recomputes pre from a sliding window of
+// inputs, keeps the last W dpre rows, and emits dx[s] once dpre[s .. s+W-1] exist (it reads W-1 rows past its run for that,
+// without adding them to its weight sums).  Its weight / bias sums go to part[run id][W+1][D] (fp32) and are added up by
+// conv_wgrad_reduce_kernel in a fixed order: no atomics, the same bits on every run.
+template <int W, bool F32>
+__global__ __launch_bounds__(256) void short_conv_bwd_kernel(const void* x, const void* w, const void* bias, const void* state,
+                                                             const void* dy, void* dx, float* part, const int B, const int T,
+                                                             const int D, const int run, const int silu, const bool w_f32,
+                                                             const bool state_f32) {
+  const int groups = D / 8, runs = (T + run - 1) / run;
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (long long)B * runs * groups) return;
+  const int cg = (int)(gid % groups);
+  const int r = (int)((gid / groups) % runs), b = (int)(gid / ((long long)groups * runs));
+  const int d0 = 8 * cg, t0 = r * run, t1 = min(T, t0 + run);
+  float wt[W][8], bs[8], win[W][8], dwin[W][8], dws[W + 1][8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+#pragma unroll
+    for (int j = 0; j < W; ++j) { wt[j][c] = ld1(w, w_f32, (size_t)(d0 + c) * W + j); dws[j][c] = 0.f; dwin[j][c] = 0.f; }
+    bs[c] = bias ? ld1(bias, w_f32, d0 + c) : 0.f;
+    dws[W][c] = 0.f;
+  }
+#pragma unroll
+  for (int j = 0; j < W - 1; ++j) {
+    const int s = t0 - (W - 1) + j;
+    if (s >= 0) {
+      load8<F32>(x, ((size_t)b * T + s) * D + d0, win[j]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) win[j][c] = state ? ld1(state, state_f32, ((size_t)b * D + d0 + c) * W + (W + s)) : 0.f;
+    }
+  }
+  // t runs W-1 rows past the run: dx of the run's last tokens needs the dpre of the next run's first ones
+  const int t_end = min(T, t1 + W - 1);
+  for (int t = t0; t < t1 + W - 1; ++t) {
+    float dp[8];
+    if (t < t_end) {
+      float g[8];
+      load8<F32>(x, ((size_t)b * T + t) * D + d0, win[W - 1]);
+      load8<F32>(dy, ((size_t)b * T + t) * D + d0, g);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        float acc = bs[c];
+#pragma unroll
+        for (int j = 0; j < W; ++j) acc += wt[j][c] * win[j][c];
+        float da = 1.f;
+        if (silu) {
+          const float sg = 1.f / (1.f + __expf(-acc));
+          da = sg * (1.f + acc * (1.f - sg));
+        }
+        dp[c] = g[c] * da;
+        if (t < t1) {   // this run's own tokens: weight and bias sums
+#pragma unroll
+          for (int j = 0; j < W; ++j) dws[j][c] += dp[c] * win[j][c];
+          dws[W][c] += dp[c];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) dp[c] = 0.f;
+    }
+    // dwin[i] = dpre[t-(W-1)+i]
+#pragma unroll
+    for (int c = 0; c < 8; ++c) dwin[W - 1][c] = dp[c];
+    const int sx = t - (W - 1);
+    if (sx >= t0) {
+      float o[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < W; ++i) acc += wt[W - 1 - i][c] * dwin[i][c];
+        o[c] = acc;
+      }
+      store8<F32>(dx, ((size_t)b * T + sx) * D + d0, o);
+    }
+#pragma unroll
+    for (int j = 0; j < W - 1; ++j)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) { win[j][c] = win[j + 1][c]; dwin[j][c] = dwin[j + 1][c]; }
+  }
+  float* pr = part + ((size_t)(b * runs + r) * (W + 1)) * D + d0;
+#pragma unroll
+  for (int j = 0; j <= W; ++j) {
+    *reinterpret_cast<f32x4*>(pr + (size_t)j * D) = (f32x4){dws[j][0], dws[j][1], dws[j][2], dws[j][3]};
+    *reinterpret_cast<f32x4*>(pr + (size_t)j * D + 4) = (f32x4){dws[j][4], dws[j][5], dws[j][6], dws[j][7]};
+  }
+}
+
+// dw[d][j] = sum over run ids of part[id][j][d], dbias[d] = the same of part[id][W][d]; a thread per (j, d)
+__global__ __launch_bounds__(256) void conv_wgrad_reduce_kernel(const float* part, float* dw, float* dbias, const int n_part, const int D,
+                                                                const int W) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= (W + 1) * D) return;
+  const int j = i / D, d = i % D;
+  float acc = 0.f;
+  for (int k = 0; k < n_part; ++k) acc += part[((size_t)k * (W + 1) + j) * D + d];
+  if (j < W) dw[(size_t)d * W + j] = acc;
+  else if (dbias) dbias[d] = acc;
+}
+
 // A row is handled by LANES adjacent lanes with PER pieces of 8 elements each (D = 8 LANES PER).
 template <int LANES, int PER, bool F32>
 __global__ __launch_bounds__(256) void row_norm_kernel(const void* x, const void* weight, void* y, const long long rows, const float eps,
@@ -168,6 +272,13 @@ __global__ __launch_bounds__(256) void row_norm_kernel(const void* x, const void
 
 using namespace natsl;
 
+static int conv_run_length(int B, int T, int D) {
+  // long runs read the fewest rows twice; short ones are needed to give every CU work on small inputs
+  int run = 32;
+  while (run > 8 && (long long)B * cdiv(T, run) * (D / 8) < 256 * 256) run >>= 1;
+  return run;
+}
+
 extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const void* bias, const void* state, void* y, void* state_out,
                                     int B, int T, int D, int W, int activation, int dtype, int w_dtype, int state_dtype,
                                     natsl_stream_t stream) {
@@ -180,9 +291,7 @@ extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const voi
   if (D % 8) return fail(NATSL_ERR_UNSUPPORTED, "%s: D=%d must be a multiple of 8", what, D);
   if (activation != 0 && activation != 1) return fail(NATSL_ERR_INVALID, "%s: activation must be 0 (none) or 1 (silu)", what);
   if (state_out && state_out == state) return fail(NATSL_ERR_INVALID, "%s: state_out must not alias state (other threads still read it)", what);
-  // long runs read the fewest rows twice; short ones are needed to give every CU work on small inputs
-  int run = 32;
-  while (run > 8 && (long long)B * cdiv(T, run) * (D / 8) < 256 * 256) run >>= 1;
+  const int run = conv_run_length(B, T, D);
   const long long threads = (long long)B * cdiv(T, run) * (D / 8);
   const dim3 grid((unsigned)((threads + 255) / 256));
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -202,6 +311,47 @@ extern "C" int natsl_short_conv_fwd(const void* x, const void* weight, const voi
     default: return fail(NATSL_ERR_UNSUPPORTED, "%s: kernel size %d not built (2, 3, 4)", what, W);
   }
 #undef NATSL_CONV
+}
+
+extern "C" size_t natsl_short_conv_bwd_workspace_bytes(int B, int T, int D, int W) {
+  if (B <= 0 || T <= 0 || D <= 0 || W <= 0) return 0;
+  return (size_t)B * cdiv(T, conv_run_length(B, T, D)) * (W + 1) * D * sizeof(float);
+}
+
+extern "C" int natsl_short_conv_bwd(const void* x, const void* weight, const void* bias, const void* state, const void* dy, void* dx,
+                                    float* dweight, float* dbias, void* workspace, size_t workspace_bytes, int B, int T, int D, int W,
+                                    int activation, int dtype, int w_dtype, int state_dtype, natsl_stream_t stream) {
+  const char* what = "natsl_short_conv_bwd";
+  if (!x || !weight || !dy || !dx || !dweight) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: activations must be f32 or bf16", what);
+  if (w_dtype != NATSL_BF16 && w_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: weights must be f32 or bf16", what);
+  if (state && state_dtype != NATSL_BF16 && state_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: the state must be f32 or bf16", what);
+  if (B <= 0 || T <= 0 || D <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
+  if (D % 8) return fail(NATSL_ERR_UNSUPPORTED, "%s: D=%d must be a multiple of 8", what, D);
+  if (activation != 0 && activation != 1) return fail(NATSL_ERR_INVALID, "%s: activation must be 0 (none) or 1 (silu)", what);
+  if (W < 2 || W > 4) return fail(NATSL_ERR_UNSUPPORTED, "%s: kernel size %d not built (2, 3, 4)", what, W);
+  const size_t need = natsl_short_conv_bwd_workspace_bytes(B, T, D, W);
+  if (!workspace || workspace_bytes < need) return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
+  if (reinterpret_cast<uintptr_t>(workspace) & 15) return fail(NATSL_ERR_INVALID, "%s: workspace must be 16-byte aligned", what);
+  const int run = conv_run_length(B, T, D), runs = cdiv(T, run);
+  const long long threads = (long long)B * runs * (D / 8);
+  const dim3 grid((unsigned)((threads + 255) / 256));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* part = reinterpret_cast<float*>(workspace);
+  const bool f32 = dtype == NATSL_F32;
+#define NATSL_CONVB(WW)                                                                                                            \
+  {                                                                                                                                \
+    if (f32) hipLaunchKernelGGL((short_conv_bwd_kernel<WW, true>), grid, dim3(256), 0, s, x, weight, bias, state, dy, dx, part, B, T, \
+                                D, run, activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                \
+    else hipLaunchKernelGGL((short_conv_bwd_kernel<WW, false>), grid, dim3(256), 0, s, x, weight, bias, state, dy, dx, part, B, T,    \
+                            D, run, activation, w_dtype == NATSL_F32, state_dtype == NATSL_F32);                                    \
+  }
+  if (W == 2) NATSL_CONVB(2) else if (W == 3) NATSL_CONVB(3) else NATSL_CONVB(4)
+#undef NATSL_CONVB
+  int rc = check_launch(what);
+  if (rc != NATSL_OK) return rc;
+  hipLaunchKernelGGL(conv_wgrad_reduce_kernel, dim3((unsigned)(((W + 1) * D + 255) / 256)), dim3(256), 0, s, part, dweight, dbias, B * runs, D, W);
+  return check_launch(what);
 }
 
 extern "C" int natsl_row_norm_fwd(const void* x, const void* weight, void* y, int64_t rows, int D, float eps, int l2, int dtype,

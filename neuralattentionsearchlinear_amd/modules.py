@@ -112,6 +112,19 @@ def _short_conv_fwd(x, weight, bias, cache, activation, want_state=False):
     """natsl_short_conv_fwd: token-major in, token-major out, no transposed copies -> (y, next state [B,D,W] or None)."""
     B, T, D = x.shape
     W = weight.shape[-1]
+    xc, w, b, st = _conv_operands(x, weight, bias, cache)
+    y = torch.empty_like(xc)
+    nxt = torch.empty(B, D, W, dtype=xc.dtype, device=xc.device) if want_state else None
+    rc = _capi.lib().natsl_short_conv_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(y), _capi.ptr(nxt), B, T, D,
+                                          W, 0 if activation is None else 1, _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
+                                          _capi.dtype_code(st.dtype) if st is not None else _capi.F32, _capi.stream_ptr(xc.device))
+    _capi.check(rc, "natsl_short_conv_fwd")
+    return y, nxt
+
+
+def _conv_operands(x, weight, bias, cache):
+    B, T, D = x.shape
+    W = weight.shape[-1]
     xc = x.detach().contiguous()
     w = weight.detach().reshape(D, W).contiguous()
     b = None if bias is None else bias.detach().to(w.dtype).contiguous()
@@ -122,17 +135,11 @@ def _short_conv_fwd(x, weight, bias, cache, activation, want_state=False):
         st = cache.detach().contiguous()
         if st.dtype not in (torch.float32, torch.bfloat16):
             st = st.float()
-    y = torch.empty_like(xc)
-    nxt = torch.empty(B, D, W, dtype=xc.dtype, device=xc.device) if want_state else None
-    rc = _capi.lib().natsl_short_conv_fwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(y), _capi.ptr(nxt), B, T, D,
-                                          W, 0 if activation is None else 1, _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
-                                          _capi.dtype_code(st.dtype) if st is not None else _capi.F32, _capi.stream_ptr(xc.device))
-    _capi.check(rc, "natsl_short_conv_fwd")
-    return y, nxt
+    return xc, w, b, st
 
 
 class _ShortConv(torch.autograd.Function):
-    """The HIP forward with the gradients of the same convolution evaluated as torch operations."""
+    """The HIP forward with the HIP backward (natsl_short_conv_bwd: dx, and dweight / dbias reduced in a fixed order)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, cache, activation):
@@ -143,14 +150,22 @@ class _ShortConv(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, weight, bias, cache = ctx.saved_tensors
-        with torch.enable_grad():
-            xf = x.detach().float().requires_grad_(True)
-            wf = weight.detach().float().requires_grad_(True)
-            bf = None if bias is None else bias.detach().float().requires_grad_(True)
-            y = _short_conv_torch(xf, wf, bf, None if cache is None else cache.detach().float(), ctx.activation)
-            wrt = (xf, wf) if bf is None else (xf, wf, bf)
-            grads = torch.autograd.grad(y, wrt, dy.float())
-        return (grads[0].to(x.dtype), grads[1].to(weight.dtype), None if bf is None else grads[2].to(bias.dtype), None, None)
+        B, T, D = x.shape
+        W = weight.shape[-1]
+        xc, w, b, st = _conv_operands(x, weight, bias, cache)
+        dyc = dy.detach().to(xc.dtype).contiguous()
+        dx = torch.empty_like(xc)
+        dw = torch.empty(D, W, dtype=torch.float32, device=xc.device)
+        db = torch.empty(D, dtype=torch.float32, device=xc.device) if bias is not None else None
+        L = _capi.lib()
+        ws_bytes = L.natsl_short_conv_bwd_workspace_bytes(B, T, D, W)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=xc.device)
+        rc = L.natsl_short_conv_bwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(b), _capi.ptr(st), _capi.ptr(dyc), _capi.ptr(dx), _capi.ptr(dw),
+                                    _capi.ptr(db), _capi.ptr(ws), ws_bytes, B, T, D, W, 0 if ctx.activation is None else 1,
+                                    _capi.dtype_code(xc.dtype), _capi.dtype_code(w.dtype),
+                                    _capi.dtype_code(st.dtype) if st is not None else _capi.F32, _capi.stream_ptr(xc.device))
+        _capi.check(rc, "natsl_short_conv_bwd")
+        return (dx.to(x.dtype), dw.view(weight.shape).to(weight.dtype), None if bias is None else db.to(bias.dtype), None, None)
 
 
 class ShortConvolution(nn.Conv1d):

@@ -226,9 +226,12 @@ def test_short_convolution(W, D, act, bias, dtype):
     (yg.float() * dy.to(DEV)).sum().backward()
     xr = x.float().requires_grad_(True)
     wr = wf.clone().requires_grad_(True)
-    yr = F.conv1d(xr.transpose(1, 2), wr, bf, padding=W - 1, groups=D)[..., :T].transpose(1, 2)
+    br = bf.clone().requires_grad_(True) if bias else None
+    yr = F.conv1d(xr.transpose(1, 2), wr, br, padding=W - 1, groups=D)[..., :T].transpose(1, 2)
     ((F.silu(yr) if act is not None else yr) * dy).sum().backward()
     assert rel_l2(xd.grad.float(), xr.grad) <= 5e-3 and rel_l2(conv.weight.grad.float(), wr.grad) <= 5e-3
+    if bias:
+        assert rel_l2(conv.bias.grad.float(), br.grad) <= 5e-3
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
