@@ -1,11 +1,22 @@
 """Backward of the linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for training.
 
-NOT a HIP kernel yet: the gradients are obtained by re-running the chunked forward as differentiable torch operations on
-the GPU (fp32, batched over sequences and heads, one step per 64-token chunk) and calling autograd on it.  It is the
-same algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong to the forward that was
-actually computed, up to its bf16 rounding.  It replaces chunk_gated_delta_rule_nats_bwd
-(src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart (src/nats/ops/mamba/chunk.py:112-260) in
-function, not in speed.
+NOT HIP kernels yet: fp32 torch operations on the GPU, organised so that nothing but two short loops over the chunks is
+sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
+to the forward that was actually computed, up to its bf16 rounding.  It replaces chunk_gated_delta_rule_nats_bwd
+(src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart (src/nats/ops/mamba/chunk.py:112-260) in function.
+
+Per 64-token chunk c with entering state S_c (notation of the forward):
+    X = v - W S_c,  v_new = T X,  o = Q~ S_c + P v_new,  S_{c+1} = e^{gamma_last} S_c + gate * K~^T v_new
+(a block that is not typed linear ends in S = f * S_blockstart + gate_off * K~^T v_new instead, f = e^{sum of g over the
+block} or 1).  Three steps:
+  1. the states S_c of all chunks: one loop over the chunks without autograd (three small products per chunk);
+  2. the state gradients: the reverse recurrence
+         dv_new = P^T dO + K~ dS',   dX = T^T dv_new,   dS_c = e^{gamma_last} dS' + Q~^T dO - W^T dX
+     (dS' = gradient of S_{c+1}; at the end of a block that is not typed linear it goes to the block's first chunk times f
+     instead of into the chain), again one loop without autograd;
+  3. everything else in ONE batched autograd call over all chunks at once: with S_c and dS' of every chunk as constants, the
+     gradients of  sum_c <dO_c, o_c> + <dS'_c, S_{c+1}>  with respect to q, k, v, g, beta and the gates are the exact
+     gradients of the whole recurrence (the chain rule split at the states).
 
 The selector's straight-through gradient for the linear operator (src/nats/ops/common/chunk_o.py:438-443, :487-492) is the
 inner product of the state gradient behind a chunk with that chunk's additive state update k~^T v_new: the derivative
@@ -29,13 +40,11 @@ def _chunks(x, NT):
     return x.permute(0, 3, 1, 2, *range(4, x.dim()))
 
 
-def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, decay, l2norm, intra, gate_on, gate_off):
-    """Differentiable chunked forward.  q,k [B,T,H,K], v [B,T,H,V], g,beta [B,T,H] (fp32), h0 [B,H,K,V] or None,
-    lin bool [B,NB,H] (block typed linear), gate_on / gate_off [B,NT,H] (ones / zeros).  -> (o [B,T,H,V], S [B,H,K,V])."""
-    B, T, H, K = q.shape
-    V = v.shape[-1]
+def _chunk_local(kind, q, k, v, g, beta, scale, l2norm):
+    """Everything of a chunk that does not depend on the state, for all chunks at once (differentiable):
+    qe, kd [B,H,NT,C,K], P [B,H,NT,C,C], vc [B,H,NT,C,V], dec, glast [B,H,NT], and for the delta rule TmB [..,C,C], w [..,C,K]."""
+    T = q.shape[1]
     NT = -(-T // C)
-    per = block // C
     delta = kind == 'gdn'
     if l2norm and delta:
         q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6)
@@ -53,31 +62,41 @@ def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, de
     if not delta:
         dk = torch.clamp(dk, max=0.0)                                       # src/nats/ops/mamba/chunk_h.py:177
     kd = kc * torch.exp(dk).unsqueeze(-1)
-    dec = torch.exp(glast)
+    out = dict(qe=qe, kd=kd, P=P, vc=vc, dec=torch.exp(glast), glast=glast)
     if delta:
         bc = _chunks(beta, NT)
         A = torch.tril(bc.unsqueeze(-1) * (kc @ kc.transpose(-1, -2)) * Lm, -1)
         eye = torch.eye(C, dtype=q.dtype, device=q.device)
         Tm = torch.linalg.solve_triangular(eye + A, eye.expand_as(A).contiguous(), upper=False)
-        TmB = Tm * bc.unsqueeze(-2)
-        w = kc * eg
+        out['TmB'] = Tm * bc.unsqueeze(-2)
+        out['w'] = kc * eg
+    return out
+
+
+def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, decay, l2norm, intra, gate_on, gate_off):
+    """Differentiable chunked forward (the whole recurrence under autograd; kept as the plain statement of the algorithm).
+    q,k [B,T,H,K], v [B,T,H,V], g,beta [B,T,H] (fp32), h0 [B,H,K,V] or None, lin bool [B,NB,H] (block typed linear),
+    gate_on / gate_off [B,NT,H] (ones / zeros).  -> (o [B,T,H,V], S [B,H,K,V])."""
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    NT = -(-T // C)
+    per = block // C
+    delta = kind == 'gdn'
+    m = _chunk_local(kind, q, k, v, g, beta, scale, l2norm)
     S = torch.zeros(B, H, K, V, dtype=q.dtype, device=q.device) if h0 is None else h0
     outs = []
     S_start, gsum = S, None
     for c in range(NT):
         if c % per == 0:
             S_start, gsum = S, torch.zeros(B, H, dtype=q.dtype, device=q.device)
-        if delta:
-            vn = TmB[:, :, c] @ (vc[:, :, c] - w[:, :, c] @ S)
-        else:
-            vn = vc[:, :, c]
-        o = qe[:, :, c] @ S
+        vn = m['TmB'][:, :, c] @ (m['vc'][:, :, c] - m['w'][:, :, c] @ S) if delta else m['vc'][:, :, c]
+        o = m['qe'][:, :, c] @ S
         if intra:
-            o = o + P[:, :, c] @ vn
+            o = o + m['P'][:, :, c] @ vn
         outs.append(o)
-        upd = kd[:, :, c].transpose(-1, -2) @ vn                            # the chunk's additive state update
-        gsum = gsum + glast[:, :, c]
-        S_up = dec[:, :, c, None, None] * S + gate_on[:, c, :, None, None] * upd
+        upd = m['kd'][:, :, c].transpose(-1, -2) @ vn                       # the chunk's additive state update
+        gsum = gsum + m['glast'][:, :, c]
+        S_up = m['dec'][:, :, c, None, None] * S + gate_on[:, c, :, None, None] * upd
         if (c + 1) % per == 0 or c == NT - 1:
             keep = lin[:, (c * C) // block][..., None, None]
             back = S_start * torch.exp(gsum)[..., None, None] if decay else S_start
@@ -94,42 +113,105 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
     """Gradients of the chunked linear branch: -> (dq, dk, dv, dg fp32, dbeta or None, dh0 or None, dnats fp32 [B,NB,HN]).
     types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None."""
     B, T, H, K = q.shape
-    HN = types.shape[2]
+    V = v.shape[-1]
+    HN, NB = types.shape[2], types.shape[1]
     NT = -(-T // C)
     per = block // C
     f32 = torch.float32
+    delta = kind == 'gdn'
+    dev = q.device
+    lin = (torch.round(types[..., 1].detach().float()) == 1).repeat_interleave(H // HN, dim=2)            # [B,NB,H]
+    blk_of = torch.arange(NT, device=dev) * C // block                                                     # chunk -> block
+    first_of = blk_of * per                                                                               # chunk -> first chunk of its block
+    last = ((torch.arange(NT, device=dev) + 1) % per == 0) | (torch.arange(NT, device=dev) == NT - 1)      # chunk ends its block
+    keep_c = lin[:, blk_of].permute(0, 2, 1)                                                               # [B,H,NT]: the chunk's block is typed linear
+    rolled = last.view(1, 1, NT) & ~keep_c                                                                # the state is rolled back behind this chunk
+    last_l = [((c + 1) % per == 0) or c == NT - 1 for c in range(NT)]
+    first_l = [(c * C // block) * per for c in range(NT)]
+
+    def block_factor(glast):
+        # e^{sum of gamma_last over the chunks of the block} per chunk (the roll-back's decay), or 1
+        if not decay:
+            return torch.ones_like(glast)
+        pad = NB * per - NT
+        gl = torch.cat([glast, glast.new_zeros(B, H, pad)], -1) if pad else glast
+        return torch.exp(gl.view(B, H, NB, per).sum(-1))[:, :, blk_of]
+
+    with torch.no_grad():
+        qf, kf, vf, gf = (t.detach().to(f32) for t in (q, k, v, g))
+        bf = beta.detach().to(f32) if delta else None
+        m = _chunk_local(kind, qf, kf, vf, gf, bf, scale, l2norm)
+        dO = _chunks(do.detach().to(f32), NT)                                                             # [B,H,NT,C,V]
+        f_c = block_factor(m['glast'])
+        # ---- 1. the entering state of every chunk ---------------------------------------------------------------------
+        S_all = torch.empty(B, H, NT, K, V, dtype=f32, device=dev)
+        S = torch.zeros(B, H, K, V, dtype=f32, device=dev) if h0 is None else h0.detach().to(f32)
+        for c in range(NT):
+            S_all[:, :, c] = S
+            vn = m['TmB'][:, :, c] @ (m['vc'][:, :, c] - m['w'][:, :, c] @ S) if delta else m['vc'][:, :, c]
+            S_up = m['dec'][:, :, c, None, None] * S + m['kd'][:, :, c].transpose(-1, -2) @ vn
+            if last_l[c]:
+                back = S_all[:, :, first_l[c]] * f_c[:, :, c, None, None]
+                S = torch.where(keep_c[:, :, c, None, None], S_up, back)
+            else:
+                S = S_up
+        # ---- 2. the gradient of the state behind every chunk ----------------------------------------------------------
+        dSp = torch.empty(B, H, NT, K, V, dtype=f32, device=dev)
+        dS = torch.zeros(B, H, K, V, dtype=f32, device=dev) if dht is None else dht.detach().to(f32)
+        pending = None                                   # f * dS' of a rolled-back block, owed to the block's first chunk
+        for c in range(NT - 1, -1, -1):
+            dSp[:, :, c] = dS
+            if last_l[c]:
+                rb = rolled[:, :, c, None, None]
+                pending = torch.where(rb, dS * f_c[:, :, c, None, None], torch.zeros_like(dS))
+                dS_up = torch.where(rb, torch.zeros_like(dS), dS)
+            else:
+                dS_up = dS
+            dvn = m['kd'][:, :, c] @ dS_up
+            if intra:
+                dvn = dvn + m['P'][:, :, c].transpose(-1, -2) @ dO[:, :, c]
+            dS = m['dec'][:, :, c, None, None] * dS_up + m['qe'][:, :, c].transpose(-1, -2) @ dO[:, :, c]
+            if delta:
+                dX = m['TmB'][:, :, c].transpose(-1, -2) @ dvn
+                dS = dS - m['w'][:, :, c].transpose(-1, -2) @ dX
+            if c % per == 0:
+                dS = dS + pending
+        dh0 = dS if h0 is not None else None
+        S_first = S_all[:, :, first_of]                                                                   # each chunk's block-start state
+        del m
+
+    # ---- 3. everything else: one batched autograd call with the states as constants ----------------------------------
     with torch.enable_grad():
         leaves = [t.detach().to(f32).requires_grad_(True) for t in (q, k, v, g)]
         qf, kf, vf, gf = leaves
-        bf = beta.detach().to(f32).requires_grad_(True) if kind == 'gdn' else None
-        hf = h0.detach().to(f32).requires_grad_(True) if h0 is not None else None
-        lin = (torch.round(types[..., 1].detach().float()) == 1).repeat_interleave(H // HN, dim=2)       # [B,NB,H]
-        gate_on = torch.ones(B, NT, H, dtype=f32, device=q.device, requires_grad=True)
-        gate_off = torch.zeros(B, NT, H, dtype=f32, device=q.device, requires_grad=dnats_for_invalid_blocks)
-        o, S = linear_chunk_forward_torch(kind, qf, kf, vf, gf, bf, hf, lin, scale, block, decay, l2norm, intra, gate_on, gate_off)
-        outs, grads_out = [o], [do.to(f32)]
-        if dht is not None:
-            outs.append(S)
-            grads_out.append(dht.to(f32))
+        bf = beta.detach().to(f32).requires_grad_(True) if delta else None
+        gate_on = torch.ones(B, NT, H, dtype=f32, device=dev, requires_grad=True)
+        gate_off = torch.zeros(B, NT, H, dtype=f32, device=dev, requires_grad=dnats_for_invalid_blocks)
+        m = _chunk_local(kind, qf, kf, vf, gf, bf, scale, l2norm)
+        vn = m['TmB'] @ (m['vc'] - m['w'] @ S_all) if delta else m['vc']
+        o = m['qe'] @ S_all
+        if intra:
+            o = o + m['P'] @ vn
+        upd = m['kd'].transpose(-1, -2) @ vn
+        S_up = m['dec'][..., None, None] * S_all + gate_on.permute(0, 2, 1)[..., None, None] * upd
+        S_back = block_factor(m['glast'])[..., None, None] * S_first + gate_off.permute(0, 2, 1)[..., None, None] * upd
+        S_next = torch.where(rolled[..., None, None], S_back, S_up)
+        total = (o * dO).sum() + (S_next * dSp).sum()
         wrt = [qf, kf, vf, gf, gate_on]
         if bf is not None:
             wrt.append(bf)
-        if hf is not None:
-            wrt.append(hf)
         if dnats_for_invalid_blocks:
             wrt.append(gate_off)
-        grads = list(torch.autograd.grad(outs, wrt, grads_out, allow_unused=True))
+        grads = list(torch.autograd.grad(total, wrt, allow_unused=True))
     dq, dk, dv, dg, dgate = grads[:5]
     rest = grads[5:]
     dbeta = rest.pop(0) if bf is not None else None
-    dh0 = rest.pop(0) if hf is not None else None
     # a gate acts where its block's update is kept (typed linear), the zero gate where it is not
     lin_c = lin.repeat_interleave(per, dim=1)[:, :NT]                                                     # per chunk
     dn = torch.where(lin_c, dgate, torch.zeros_like(dgate))
     if dnats_for_invalid_blocks:
         dgo = rest.pop(0)
         dn = dn + torch.where(lin_c, torch.zeros_like(dgo), dgo)
-    NB = types.shape[1]
     pad = NB * per - NT
     if pad:
         dn = torch.cat([dn, dn.new_zeros(B, pad, H)], 1)
