@@ -142,21 +142,25 @@ size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H);
  * sequence's last selector block, g_block_sum [N,H] fp32 = the sum of g over that block (the two
  * quantities chunk_gated_delta_rule_nats_inference_fwd derives at
  * src/nats/ops/gated_delta_rule/chunk_fwd.py:178-206); pass NULL for both in training.
+ * chunk_states (optional, for a backward): the state ENTERING every 64-token chunk, transposed and rounded as the kernel
+ * uses it, bf16 [total_chunks][H][V][K] (total_chunks as for natsl_linear_workspace_bytes; the reference keeps the same
+ * per-chunk states as `h`, src/nats/ops/common/chunk_delta_h.py:681-683); NULL = not stored.
  * Replaces l2norm_fwd + chunk_gated_delta_rule_nats_fwd
  * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:119-164, src/nats/ops/gated_delta_rule/chunk.py:22-167). */
 int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
                         const float* h0, void* o, float* ht, float* h_block_start, float* g_block_sum,
-                        const void* types, int types_dtype, int B,
+                        void* chunk_states, const void* types, int types_dtype, int B,
                         int T, int H, int HN, int K, int V, int TN, int block, float scale, int flags,
                         void* workspace, size_t workspace_bytes, int dtype, const natsl_seq_row* seqs,
                         int n_seqs, int total_units, natsl_stream_t stream);
 
 /* Mamba2-style SSD branch, chunked forward (q = C, k = B, v = X*dt, g = A*dt).
- * h_block_start / g_block_sum as for the Gated DeltaNet entry (src/nats/ops/mamba/chunk_fwd.py:22-157).
+ * h_block_start / g_block_sum / chunk_states as for the Gated DeltaNet entry (src/nats/ops/mamba/chunk_fwd.py:22-157).
  * Replaces chunk_mamba2_fwd (src/nats/ops/mamba/chunk.py:21-109) as called at
  * src/nats/ops/mixed_ops/mixed_attn_mamba.py:140-161. */
 int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* h0,
-                          void* o, float* ht, float* h_block_start, float* g_block_sum, const void* types, int types_dtype, int B, int T, int H,
+                          void* o, float* ht, float* h_block_start, float* g_block_sum, void* chunk_states, const void* types,
+                          int types_dtype, int B, int T, int H,
                           int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
                           size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs,
                           int total_units, natsl_stream_t stream);

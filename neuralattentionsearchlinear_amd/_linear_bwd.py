@@ -1,7 +1,7 @@
 """Backward of the linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for training.
 
-NOT HIP kernels yet: fp32 torch operations on the GPU, organised so that nothing but two short loops over the chunks is
-sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
+NOT HIP kernels yet except for the states: fp32 torch operations on the GPU, organised so that nothing but one short loop
+over the chunks is sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
 to the forward that was actually computed, up to its bf16 rounding.  It replaces chunk_gated_delta_rule_nats_bwd
 (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart (src/nats/ops/mamba/chunk.py:112-260) in function.
 
@@ -9,11 +9,12 @@ Per 64-token chunk c with entering state S_c (notation of the forward):
     X = v - W S_c,  v_new = T X,  o = Q~ S_c + P v_new,  S_{c+1} = e^{gamma_last} S_c + gate * K~^T v_new
 (a block that is not typed linear ends in S = f * S_blockstart + gate_off * K~^T v_new instead, f = e^{sum of g over the
 block} or 1).  Three steps:
-  1. the states S_c of all chunks: one loop over the chunks without autograd (three small products per chunk);
+  1. the states S_c of all chunks: the forward kernel run once more with its per-chunk state output (bf16, as the forward
+     used them);
   2. the state gradients: the reverse recurrence
          dv_new = P^T dO + K~ dS',   dX = T^T dv_new,   dS_c = e^{gamma_last} dS' + Q~^T dO - W^T dX
      (dS' = gradient of S_{c+1}; at the end of a block that is not typed linear it goes to the block's first chunk times f
-     instead of into the chain), again one loop without autograd;
+     instead of into the chain), one loop without autograd;
   3. everything else in ONE batched autograd call over all chunks at once: with S_c and dS' of every chunk as constants, the
      gradients of  sum_c <dO_c, o_c> + <dS'_c, S_{c+1}>  with respect to q, k, v, g, beta and the gates are the exact
      gradients of the whole recurrence (the chain rule split at the states).
@@ -143,18 +144,20 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
         m = _chunk_local(kind, qf, kf, vf, gf, bf, scale, l2norm)
         dO = _chunks(do.detach().to(f32), NT)                                                             # [B,H,NT,C,V]
         f_c = block_factor(m['glast'])
-        # ---- 1. the entering state of every chunk ---------------------------------------------------------------------
-        S_all = torch.empty(B, H, NT, K, V, dtype=f32, device=dev)
-        S = torch.zeros(B, H, K, V, dtype=f32, device=dev) if h0 is None else h0.detach().to(f32)
-        for c in range(NT):
-            S_all[:, :, c] = S
-            vn = m['TmB'][:, :, c] @ (m['vc'][:, :, c] - m['w'][:, :, c] @ S) if delta else m['vc'][:, :, c]
-            S_up = m['dec'][:, :, c, None, None] * S + m['kd'][:, :, c].transpose(-1, -2) @ vn
-            if last_l[c]:
-                back = S_all[:, :, first_l[c]] * f_c[:, :, c, None, None]
-                S = torch.where(keep_c[:, :, c, None, None], S_up, back)
-            else:
-                S = S_up
+        # ---- 1. the entering state of every chunk: the forward kernel run once more, storing them ------------------------
+        from . import _capi
+        from ._mixed_common import linear_chunk_fwd
+        flags = (_capi.DECAY_NON_LINEAR if decay else 0) | (_capi.QK_L2NORM if l2norm else 0) | (_capi.INTRA_CHUNK if intra else 0)
+        bf16 = torch.bfloat16
+        ty = types.detach()
+        ty = (ty if ty.dtype in (bf16, f32) else ty.float()).contiguous()
+        _, _, st = linear_chunk_fwd(kind, q.detach().to(bf16).contiguous(), k.detach().to(bf16).contiguous(),
+                                    v.detach().to(bf16).contiguous(), g.detach().to(f32).contiguous(),
+                                    beta.detach().to(bf16).contiguous() if delta else None,
+                                    None if h0 is None else h0.detach().to(f32).contiguous(), ty, scale, block, flags,
+                                    False, None, chunk_states=True)
+        S_all = st.view(B, NT, H, V, K).permute(0, 2, 1, 4, 3).to(f32)                                     # [B,H,NT,K,V]
+        del st
         # ---- 2. the gradient of the state behind every chunk ----------------------------------------------------------
         dSp = torch.empty(B, H, NT, K, V, dtype=f32, device=dev)
         dS = torch.zeros(B, H, K, V, dtype=f32, device=dev) if dht is None else dht.detach().to(f32)

@@ -52,9 +52,11 @@ def _wants_grad(*tensors) -> bool:
 
 
 def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block: int, flags: int,
-                     output_final_state: bool, seqs: Optional[PackedSeqs], block_start_state: bool = False):
+                     output_final_state: bool, seqs: Optional[PackedSeqs], block_start_state: bool = False,
+                     chunk_states: bool = False):
     """Launch the chunked linear branch ('gdn' or 'mamba'); returns (o, final_state or None), or with
-    block_start_state (o, final_state, state entering the last block, sum of g over the last block)."""
+    block_start_state (o, final_state, state entering the last block, sum of g over the last block), or with chunk_states
+    (o, final_state, the state entering every chunk as bf16 [total_chunks, H, V, K])."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     TN, HN = types.shape[1], types.shape[2]
@@ -67,12 +69,13 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
     ht = torch.empty(n, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
     hs = torch.empty(n, H, K, V, dtype=torch.float32, device=dev) if block_start_state else None
     gs = torch.empty(n, H, dtype=torch.float32, device=dev) if block_start_state else None
+    sc = torch.empty(total_chunks, H, V, K, dtype=torch.bfloat16, device=dev) if chunk_states else None
     if h0 is not None:
         if tuple(h0.shape) != (n, H, K, V):
             raise ValueError(f"initial state must have shape {(n, H, K, V)}, got {tuple(h0.shape)}")
         h0 = h0.to(torch.float32).contiguous()
     sp, ns, tot = _seq_args(seqs, total_chunks)
-    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(hs), _capi.ptr(gs), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
+    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(hs), _capi.ptr(gs), _capi.ptr(sc), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
               block, float(scale), flags, _capi.ptr(ws), ws.numel(), _capi.dtype_code(q.dtype), sp, ns, tot,
               _capi.stream_ptr(dev))
     if kind == 'gdn':
@@ -83,6 +86,8 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
         _capi.check(rc, "natsl_mamba_chunk_fwd")
     if block_start_state:
         return o, ht, hs, gs
+    if chunk_states:
+        return o, ht, sc
     return o, ht
 
 

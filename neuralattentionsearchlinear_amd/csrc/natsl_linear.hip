@@ -50,6 +50,7 @@ struct LinearParams {
   float* ht;
   float* hs;      // state entering each sequence's last selector block (optional)
   float* gs;      // sum of g over that block, [N,H] (optional)
+  bf16_t* s_out;  // the state entering every chunk, transposed: [chunk][H][V][K] bf16 (optional; for the backward)
   const void* types;
   int types_dtype;
   const SeqRow* seqs;
@@ -683,6 +684,12 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     bf16x8 SB[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) SB[s] = pack8(S[2 * s], S[2 * s + 1]);
+    if (p.s_out) {
+      // a B operand is eight consecutive K rows of this lane's column: 16 contiguous bytes of S^T [V][K]
+      bf16_t* so = p.s_out + (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 8 * g4;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(so + 32 * s) = SB[s];
+    }
     const float dec_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, dec_v)));
     const float glast_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, glast_v)));
     const float linf_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, linf_v)));
@@ -930,7 +937,7 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
-                      const float* h0, void* o, float* ht, float* hs, float* gs, const void* types, int types_dtype, int B, int T,
+                      const float* h0, void* o, float* ht, float* hs, float* gs, void* chunk_states, const void* types, int types_dtype, int B, int T,
                       int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                       int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream) {
   const char* what = delta ? "natsl_gdn_chunk_fwd" : "natsl_mamba_chunk_fwd";
@@ -945,7 +952,7 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
     return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   LinearParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.g = g; p.beta = (const bf16_t*)beta;
-  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.hs = hs; p.gs = gs; p.types = types; p.types_dtype = types_dtype;
+  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.hs = hs; p.gs = gs; p.s_out = (bf16_t*)chunk_states; p.types = types; p.types_dtype = types_dtype;
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block;
   p.nt = cdiv(T, C);
@@ -982,19 +989,19 @@ extern "C" size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H) {
 
 extern "C" int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
                                    const float* h0, void* o, float* ht, float* h_block_start, float* g_block_sum,
-                                   const void* types, int types_dtype, int B, int T,
+                                   void* chunk_states, const void* types, int types_dtype, int B, int T,
                                    int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
                                    size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                    natsl_stream_t stream) {
-  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, h_block_start, g_block_sum, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
+  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, h_block_start, g_block_sum, chunk_states, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
                     workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }
 
 extern "C" int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const float* h0, void* o,
-                                     float* ht, float* h_block_start, float* g_block_sum, const void* types, int types_dtype, int B, int T, int H, int HN, int K, int V,
+                                     float* ht, float* h_block_start, float* g_block_sum, void* chunk_states, const void* types, int types_dtype, int B, int T, int H, int HN, int K, int V,
                                      int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                                      int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                      natsl_stream_t stream) {
-  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, h_block_start, g_block_sum, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
+  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, h_block_start, g_block_sum, chunk_states, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
                     flags & ~NATSL_QK_L2NORM, workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }
