@@ -37,6 +37,11 @@ CACHE_WORKLOADS = {
 BACKWARD_WORKLOADS = {
     "softmax_bwd_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
 }
+# backward of the Gated DeltaNet branch at the headline shape (training); not the headline metric
+LINEAR_BACKWARD_WORKLOADS = {
+    "gdn_bwd_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
+    "gdn_bwd_B8_T4096_H6_K128_V256_p25": dict(B=8, T=4096, H=6, K=128, V=256, p_attn=0.25, block=64),
+}
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 
@@ -312,12 +317,51 @@ def bench_softmax_bwd(args):
                       note="whole step: delta, dq and dk/dv kernels"))))
 
 
+def bench_linear_bwd(args):
+    """Backward of the Gated DeltaNet branch: dq, dk, dv, dg, dbeta and the selector's gradient from (q, k, v, g, beta, do):
+    the forward once more (storing every chunk's state and v_new), the reverse scan, the per-chunk gradient kernel.
+    HBM-bound by design: the compulsory bytes are the six inputs and five outputs once."""
+    import torch
+    from neuralattentionsearchlinear_amd import _capi, nats_util
+    from neuralattentionsearchlinear_amd._linear_bwd import linear_chunk_backward_hip
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    w = LINEAR_BACKWARD_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    host, d = make_inputs(w, torch, dev)
+    ty, nb = nats_util.hard_select(d["logits"], force_last_block=True)
+    do = torch.randn(d["v"].shape, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).bfloat16()
+
+    def step():
+        return linear_chunk_backward_hip('gdn', d["q"], d["k"], d["v"], d["g"], d["beta"], None, ty, w["K"] ** -0.5, w["block"], True, True,
+                                         True, do, None, False)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    n_tok = w["B"] * w["T"] * w["H"]
+    nbytes = n_tok * (2 * (4 * w["K"] + 3 * w["V"]) + 4 * 2 + 2 * 2)     # q, k, dq, dk; v, do, dv; g, dg (f32); beta, dbeta
+    print(json.dumps(dict(
+        metric="GDN-branch backward tokens/sec bf16", value=w["B"] * w["T"] / (ms * 1e-3), unit="tokens/s",
+        n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w),
+        roofline=dict(bound="hbm", kernel="linear_prep+linear_scan+linear_bwd_scan+linear_bwd_chunk", achieved=nbytes / (ms * 1e-3) / 1e9,
+                      peak=PEAK_HBM_GBS, unit="GB/s", frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, traffic=None, algorithmic_bytes=nbytes,
+                      note="whole step incl. the forward re-run and the host-side glue"))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS))
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS) + sorted(LINEAR_BACKWARD_WORKLOADS))
     ap.add_argument("--prewarm-ms", type=float, default=300.0,
                     help="milliseconds of untimed load before the warm-up steps, to let the GPU clocks settle (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -341,6 +385,8 @@ def main():
         return bench_kv_compact(args)
     if args.workload in BACKWARD_WORKLOADS:
         return bench_softmax_bwd(args)
+    if args.workload in LINEAR_BACKWARD_WORKLOADS:
+        return bench_linear_bwd(args)
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn

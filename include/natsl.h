@@ -145,11 +145,13 @@ size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H);
  * chunk_states (optional, for a backward): the state ENTERING every 64-token chunk, transposed and rounded as the kernel
  * uses it, bf16 [total_chunks][H][V][K] (total_chunks as for natsl_linear_workspace_bytes; the reference keeps the same
  * per-chunk states as `h`, src/nats/ops/common/chunk_delta_h.py:681-683); NULL = not stored.
+ * chunk_v_new (optional, for a backward): the delta rule's corrected values v_new of every token, bf16 [B*T][H][V] (the
+ * reference's `v_new`, chunk_delta_h.py:684); NULL = not stored.
  * Replaces l2norm_fwd + chunk_gated_delta_rule_nats_fwd
  * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:119-164, src/nats/ops/gated_delta_rule/chunk.py:22-167). */
 int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
                         const float* h0, void* o, float* ht, float* h_block_start, float* g_block_sum,
-                        void* chunk_states, const void* types, int types_dtype, int B,
+                        void* chunk_states, void* chunk_v_new, const void* types, int types_dtype, int B,
                         int T, int H, int HN, int K, int V, int TN, int block, float scale, int flags,
                         void* workspace, size_t workspace_bytes, int dtype, const natsl_seq_row* seqs,
                         int n_seqs, int total_units, natsl_stream_t stream);
@@ -164,6 +166,29 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
                           int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
                           size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs,
                           int total_units, natsl_stream_t stream);
+
+/* Backward of the two chunked linear branches (delta_rule != 0: Gated DeltaNet, else Mamba2-style SSD), regular batches
+ * (packed input: one call per sequence).  Call the forward entry first with chunk_states and (delta rule) chunk_v_new and
+ * keep its workspace: this entry reads the triangular solves from it.  Inputs as for the forward, plus
+ *   v_new [B*T][H][V] (Mamba: v itself), d_o [B*T][H][V] bf16, dht [B][H][K][V] f32 or NULL,
+ *   g_block_sums [B][TN][H] f32 = sum of g over every selector block.
+ * Outputs: dq, dk [B*T][H][K], dv [B*T][H][V] bf16; dg, dbeta (delta rule) [B*T][H] f32; dh0 [B][H][K][V] f32 or NULL;
+ *   d_gate [chunks][H] f32 = derivative with respect to a gate on every chunk's state update (the selector's
+ *   straight-through gradient for the linear operator, src/nats/ops/common/chunk_o.py:438-443, :487-492, before the sum over
+ *   a block's chunks and a selector head's heads);
+ *   d_rollback [chunks][H] f32 = what the decay of a rolled-back block adds to dg of each of its tokens (non-zero behind
+ *   the last chunk of blocks that are not typed linear, NATSL_DECAY_NON_LINEAR only);
+ *   d_chunk_states: scratch, bf16 [chunks][H][V][K] (the gradient of the state behind every chunk);
+ *   dbeta_parts: scratch, f32 [B*T][H][V/16] (delta rule only); state_dot_parts: scratch, f32 [chunks][H][V/16].
+ * K in {64, 128, 192}, V a multiple of 64.
+ * Replaces chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart
+ * (src/nats/ops/mamba/chunk.py:112-260). */
+int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void* k, const void* v_new, const float* g, const void* beta,
+                           const void* d_o, const float* dht, const void* chunk_states, const void* types, int types_dtype,
+                           const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
+                           float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
+                           int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
+                           natsl_stream_t stream);
 
 /* Layer tail: y = (rms(x1)*w1*xw[...,0] + rms(x2)*w2*xw[...,1]) * gate*sigmoid(gate) with
  * rms(x) = x*rsqrt(mean(x^2)+eps); x1, x2, gate, y [rows, D] and x_weights [rows, 2] in `dtype`,

@@ -8,7 +8,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libnatsl.so")
-SOURCES = ["natsl_route.hip", "natsl_softmax.hip", "natsl_softmax_bwd.hip", "natsl_linear.hip", "natsl_norm_gate.hip", "natsl_conv.hip", "natsl_decode.hip", "natsl_cache.hip", "natsl_probe.hip"]
+SOURCES = ["natsl_route.hip", "natsl_softmax.hip", "natsl_softmax_bwd.hip", "natsl_linear.hip", "natsl_linear_bwd.hip", "natsl_norm_gate.hip", "natsl_conv.hip", "natsl_decode.hip", "natsl_cache.hip", "natsl_probe.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
     # keep the compiler from forming packed-fp32 VALU ops

@@ -1,7 +1,8 @@
 """Backward of the linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for training.
 
-NOT HIP kernels yet except for the states: fp32 torch operations on the GPU, organised so that nothing but one short loop
-over the chunks is sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
+linear_chunk_backward runs the HIP kernels of csrc/natsl_linear_bwd.hip; linear_chunk_backward_torch is the same computation
+as fp32 torch operations on the GPU (for the shapes the kernels are not built for, and as the plain statement of the method),
+organised so that nothing but one short loop over the chunks is sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
 to the forward that was actually computed, up to its bf16 rounding.  It replaces chunk_gated_delta_rule_nats_bwd
 (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart (src/nats/ops/mamba/chunk.py:112-260) in function.
 
@@ -112,7 +113,84 @@ def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, de
 def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
                           dnats_for_invalid_blocks):
     """Gradients of the chunked linear branch: -> (dq, dk, dv, dg fp32, dbeta or None, dh0 or None, dnats fp32 [B,NB,HN]).
-    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None."""
+    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None.  The HIP kernels (natsl_linear_chunk_bwd) where they are built
+    (K in 64/128/192, V a multiple of 64), else the torch formulation below."""
+    if q.shape[-1] in (64, 128, 192) and v.shape[-1] % 64 == 0:
+        return linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
+                                         dnats_for_invalid_blocks)
+    return linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
+                                       dnats_for_invalid_blocks)
+
+
+def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
+                              dnats_for_invalid_blocks):
+    """The backward as kernels: the forward once more (storing every chunk's entering state and v_new), then the reverse
+    scan and the per-chunk gradients (csrc/natsl_linear_bwd.hip)."""
+    from . import _capi
+    from ._mixed_common import linear_chunk_fwd
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    NB, HN = types.shape[1], types.shape[2]
+    NT = -(-T // C)
+    per = block // C
+    dev = q.device
+    f32, bf16 = torch.float32, torch.bfloat16
+    delta = kind == 'gdn'
+    flags = (_capi.DECAY_NON_LINEAR if decay else 0) | (_capi.QK_L2NORM if l2norm else 0) | (_capi.INTRA_CHUNK if intra else 0)
+    with torch.no_grad():
+        ty = types.detach()
+        ty = (ty if ty.dtype in (bf16, f32) else ty.float()).contiguous()
+        qb, kb, vb = (t.detach().to(bf16).contiguous() for t in (q, k, v))
+        gf = g.detach().to(f32).contiguous()
+        bb = beta.detach().to(bf16).contiguous() if delta else None
+        h0f = None if h0 is None else h0.detach().to(f32).contiguous()
+        _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, None,
+                                                   chunk_states=True)
+        pad = NB * block - T
+        gp = torch.cat([gf, gf.new_zeros(B, pad, H)], 1) if pad else gf
+        gsum = gp.view(B, NB, block, H).sum(2).contiguous()
+        d_states = torch.empty_like(states)
+        dq, dk, dv = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
+        dg = torch.empty(B, T, H, dtype=f32, device=dev)
+        dbeta = torch.empty(B, T, H, dtype=f32, device=dev) if delta else None
+        dbeta_parts = torch.empty(B, T, H, V // 16, dtype=f32, device=dev) if delta else None
+        sdot_parts = torch.empty(B, NT, H, V // 16, dtype=f32, device=dev)
+        dh0 = torch.empty(B, H, K, V, dtype=f32, device=dev) if h0 is not None else None
+        gate = torch.empty(B, NT, H, dtype=f32, device=dev)
+        rb = torch.empty(B, NT, H, dtype=f32, device=dev)
+        dof = do.detach().to(bf16).contiguous()
+        dhtf = None if dht is None else dht.detach().to(f32).contiguous()
+        P = _capi.ptr
+        rc = _capi.lib().natsl_linear_chunk_bwd(
+            1 if delta else 0, P(qb), P(kb), P(v_new), P(gf), P(bb), P(dof), P(dhtf), P(states), P(ty), _capi.dtype_code(ty.dtype),
+            P(gsum), P(ws), P(d_states), P(dbeta_parts), P(sdot_parts), P(dq), P(dk), P(dv), P(dg), P(dbeta), P(dh0), P(gate), P(rb), B, T, H, HN, K, V, NB, block,
+            float(scale), flags, _capi.dtype_code(bf16), _capi.stream_ptr(dev))
+        _capi.check(rc, "natsl_linear_chunk_bwd")
+        cpad = NB * per - NT
+
+        def per_block(x):                                    # [B,NT,H] -> [B,NB,per,H]
+            x = torch.cat([x, x.new_zeros(B, cpad, H)], 1) if cpad else x
+            return x.view(B, NB, per, H)
+
+        if decay:
+            # the decay of a rolled-back block acts on every token of the block
+            dg += per_block(rb).sum(2).repeat_interleave(block, dim=1)[:, :T]
+        lin = (torch.round(ty[..., 1].float()) == 1).repeat_interleave(H // HN, dim=2)                      # [B,NB,H]
+        gb = per_block(gate)
+        dn = torch.where(lin, gb.sum(2), torch.zeros_like(gb[:, :, 0]))
+        if dnats_for_invalid_blocks:
+            # the (zero-valued) gate on the update a block that is not typed linear would have made: its last chunk's
+            last_idx = torch.full((NB,), per - 1, device=dev)
+            last_idx[-1] = (NT - 1) % per
+            g_last = gb.gather(2, last_idx.view(1, NB, 1, 1).expand(B, NB, 1, H)).squeeze(2)
+            dn = dn + torch.where(lin, torch.zeros_like(g_last), g_last)
+        dn = dn.view(B, NB, HN, H // HN).sum(3)
+    return (dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), dg, None if dbeta is None else dbeta.to(beta.dtype), dh0, dn)
+
+
+def linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
+                                dnats_for_invalid_blocks):
+    """The same gradients with torch operations (every shape)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     HN, NB = types.shape[2], types.shape[1]
@@ -151,11 +229,11 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
         bf16 = torch.bfloat16
         ty = types.detach()
         ty = (ty if ty.dtype in (bf16, f32) else ty.float()).contiguous()
-        _, _, st = linear_chunk_fwd(kind, q.detach().to(bf16).contiguous(), k.detach().to(bf16).contiguous(),
-                                    v.detach().to(bf16).contiguous(), g.detach().to(f32).contiguous(),
-                                    beta.detach().to(bf16).contiguous() if delta else None,
-                                    None if h0 is None else h0.detach().to(f32).contiguous(), ty, scale, block, flags,
-                                    False, None, chunk_states=True)
+        st = linear_chunk_fwd(kind, q.detach().to(bf16).contiguous(), k.detach().to(bf16).contiguous(),
+                              v.detach().to(bf16).contiguous(), g.detach().to(f32).contiguous(),
+                              beta.detach().to(bf16).contiguous() if delta else None,
+                              None if h0 is None else h0.detach().to(f32).contiguous(), ty, scale, block, flags,
+                              False, None, chunk_states=True)[2]
         S_all = st.view(B, NT, H, V, K).permute(0, 2, 1, 4, 3).to(f32)                                     # [B,H,NT,K,V]
         del st
         # ---- 2. the gradient of the state behind every chunk ----------------------------------------------------------

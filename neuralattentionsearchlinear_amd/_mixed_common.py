@@ -56,7 +56,8 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
                      chunk_states: bool = False):
     """Launch the chunked linear branch ('gdn' or 'mamba'); returns (o, final_state or None), or with
     block_start_state (o, final_state, state entering the last block, sum of g over the last block), or with chunk_states
-    (o, final_state, the state entering every chunk as bf16 [total_chunks, H, V, K])."""
+    (o, final_state, the state entering every chunk as bf16 [total_chunks, H, V, K], v_new [B, T, H, V] (for 'mamba': v),
+    the workspace)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     TN, HN = types.shape[1], types.shape[2]
@@ -75,7 +76,9 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
             raise ValueError(f"initial state must have shape {(n, H, K, V)}, got {tuple(h0.shape)}")
         h0 = h0.to(torch.float32).contiguous()
     sp, ns, tot = _seq_args(seqs, total_chunks)
-    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(hs), _capi.ptr(gs), _capi.ptr(sc), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
+    vn = torch.empty_like(v) if chunk_states and kind == 'gdn' else None
+    common = (_capi.ptr(h0), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(hs), _capi.ptr(gs), _capi.ptr(sc),
+              *((_capi.ptr(vn),) if kind == 'gdn' else ()), _capi.ptr(types), _capi.dtype_code(types.dtype), B, T, H, HN, K, V, TN,
               block, float(scale), flags, _capi.ptr(ws), ws.numel(), _capi.dtype_code(q.dtype), sp, ns, tot,
               _capi.stream_ptr(dev))
     if kind == 'gdn':
@@ -87,7 +90,7 @@ def linear_chunk_fwd(kind: str, q, k, v, g, beta, h0, types, scale: float, block
     if block_start_state:
         return o, ht, hs, gs
     if chunk_states:
-        return o, ht, sc
+        return o, ht, sc, (vn if kind == 'gdn' else v), ws
     return o, ht
 
 

@@ -40,6 +40,16 @@ NATSL_DEVICE unsigned pack_bf16x2(float lo, float hi) {
 
 NATSL_DEVICE bf16_t f32_to_bf16(float f) { return (bf16_t)(pack_bf16x2(f, 0.f) & 0xffffu); }
 
+// 8 fp32 -> one bf16x8 operand: slots 0..3 from a, 4..7 from b
+NATSL_DEVICE bf16x8 pack8(const f32x4 a, const f32x4 b) {
+  u32x4 w;
+  w[0] = pack_bf16x2(a[0], a[1]);
+  w[1] = pack_bf16x2(a[2], a[3]);
+  w[2] = pack_bf16x2(b[0], b[1]);
+  w[3] = pack_bf16x2(b[2], b[3]);
+  return __builtin_bit_cast(bf16x8, w);
+}
+
 NATSL_DEVICE f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }

@@ -51,6 +51,7 @@ struct LinearParams {
   float* hs;      // state entering each sequence's last selector block (optional)
   float* gs;      // sum of g over that block, [N,H] (optional)
   bf16_t* s_out;  // the state entering every chunk, transposed: [chunk][H][V][K] bf16 (optional; for the backward)
+  bf16_t* vn_out; // v_new of every token, [tokens][H][V] bf16 (optional, delta rule only; for the backward)
   const void* types;
   int types_dtype;
   const SeqRow* seqs;
@@ -390,16 +391,6 @@ __global__ __launch_bounds__(256) void mamba_scale_kernel(const LinearParams p) 
 // =============================================================================================
 // scan
 // =============================================================================================
-// 8 fp32 -> one bf16x8 operand: slots 0..3 from a, 4..7 from b
-NATSL_DEVICE bf16x8 pack8(const f32x4 a, const f32x4 b) {
-  u32x4 w;
-  w[0] = pack_bf16x2(a[0], a[1]);
-  w[1] = pack_bf16x2(a[2], a[3]);
-  w[2] = pack_bf16x2(b[0], b[1]);
-  w[3] = pack_bf16x2(b[2], b[3]);
-  return __builtin_bit_cast(bf16x8, w);
-}
-
 // one DMA instruction: lane l copies 16 bytes from base + voff to LDS byte address lds + 16 l
 NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned lds) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
@@ -771,6 +762,15 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     }
     // (3) state update / roll-back (the next step waits for it: before the output)
     const bf16x8 VB[2] = {pack8(VN[0], VN[1]), pack8(VN[2], VN[3])};
+    if (DELTA && p.vn_out) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int tok = 16 * t + 4 * g4 + r;
+          if (tok < nvalid) p.vn_out[((size_t)(bos + c * C + tok) * p.H + h) * p.V + col] = f32_to_bf16(VN[t][r]);
+        }
+    }
     if (keep) {
       f32x4 W[4];
 #pragma unroll
@@ -937,7 +937,7 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
-                      const float* h0, void* o, float* ht, float* hs, float* gs, void* chunk_states, const void* types, int types_dtype, int B, int T,
+                      const float* h0, void* o, float* ht, float* hs, float* gs, void* chunk_states, void* chunk_v_new, const void* types, int types_dtype, int B, int T,
                       int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                       int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream) {
   const char* what = delta ? "natsl_gdn_chunk_fwd" : "natsl_mamba_chunk_fwd";
@@ -952,7 +952,7 @@ static int linear_fwd(bool delta, const void* q, const void* k, const void* v, c
     return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   LinearParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.g = g; p.beta = (const bf16_t*)beta;
-  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.hs = hs; p.gs = gs; p.s_out = (bf16_t*)chunk_states; p.types = types; p.types_dtype = types_dtype;
+  p.h0 = h0; p.o = (bf16_t*)o; p.ht = ht; p.hs = hs; p.gs = gs; p.s_out = (bf16_t*)chunk_states; p.vn_out = (bf16_t*)chunk_v_new; p.types = types; p.types_dtype = types_dtype;
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block;
   p.nt = cdiv(T, C);
@@ -989,11 +989,11 @@ extern "C" size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H) {
 
 extern "C" int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
                                    const float* h0, void* o, float* ht, float* h_block_start, float* g_block_sum,
-                                   void* chunk_states, const void* types, int types_dtype, int B, int T,
+                                   void* chunk_states, void* chunk_v_new, const void* types, int types_dtype, int B, int T,
                                    int H, int HN, int K, int V, int TN, int block, float scale, int flags, void* workspace,
                                    size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                    natsl_stream_t stream) {
-  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, h_block_start, g_block_sum, chunk_states, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
+  return linear_fwd(true, q, k, v, g, beta, h0, o, ht, h_block_start, g_block_sum, chunk_states, chunk_v_new, types, types_dtype, B, T, H, HN, K, V, TN, block, scale, flags,
                     workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }
 
@@ -1002,6 +1002,6 @@ extern "C" int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v
                                      int TN, int block, float scale, int flags, void* workspace, size_t workspace_bytes,
                                      int dtype, const natsl_seq_row* seqs, int n_seqs, int total_units,
                                      natsl_stream_t stream) {
-  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, h_block_start, g_block_sum, chunk_states, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
+  return linear_fwd(false, q, k, v, g, nullptr, h0, o, ht, h_block_start, g_block_sum, chunk_states, nullptr, types, types_dtype, B, T, H, HN, K, V, TN, block, scale,
                     flags & ~NATSL_QK_L2NORM, workspace, workspace_bytes, dtype, seqs, n_seqs, total_units, stream);
 }

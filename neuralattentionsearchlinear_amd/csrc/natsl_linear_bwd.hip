@@ -1,0 +1,816 @@
+// Backward of the chunked linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for gfx950.
+// In function it replaces chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332: dh/dv reverse
+// scan chunk_delta_h.py:327+, dq/dk/dw/dg chunk_o.py:217+, the WY backward wy_fast.py) and the Mamba counterpart
+// (src/nats/ops/mamba/chunk.py:112-260).
+//
+// Per 64-token chunk with entering state S (notation of the forward, natsl_linear.hip; q^, k^ = normalised rows):
+//     gamma = cumsum g,  G = gamma_last,  L_ij = e^{gamma_i - gamma_j}
+//     W = e^{gamma} k^,  Q~ = scale e^{gamma} q^,  K~ = e^{G - gamma} k^,  P = scale tril(q^ k^^T . L)
+//     v_new = (1/beta + stril(k^ k^^T . L))^-1 (v - W S) = TmB (v - W S)
+//     o = Q~ S + P v_new,   S' = e^G S + K~^T v_new
+// Two kernels, run after a forward pass that stored S of every chunk and v_new of every token:
+//
+//   linear_bwd_scan_kernel   walks the chunks of one (sequence, head) BACKWARDS; a wave owns 16 columns of the state
+//                            gradient for all K rows (fp32 accumulators), as the forward scan does for the state:
+//                              dv_new = P^T dO + K~ dS',   dX = TmB^T dv_new   (= dv; Mamba: dX = dv_new)
+//                              dS = e^G dS' + Q~^T dO - W^T dX
+//                            At the end of a block that is not typed linear the forward rolled the state back to the one
+//                            that entered the block (times f = e^{sum g} when decay is on): there dS' leaves the chain
+//                            and f dS' is added to dS at the block's first chunk.  Stores dS' of every chunk (bf16) and dX.
+//
+//   linear_bwd_chunk_kernel  one workgroup per (chunk, head), fully parallel: everything else.  With
+//                              N = dO v_new^T, M = dX v_new^T (64x64), Gm = scale tril(N . L), Hm = -stril(M . L):
+//                              dq^ = Gm k^ + scale e^{gamma} (dO S^T)
+//                              dk^ = Gm^T q^ + (Hm + Hm^T) k^ - e^{gamma} (dX S^T) + e^{G-gamma} (v_new dS'^T)
+//                              dbeta_i = M_ii / beta_i^2
+//                              dgamma_i = <dq^_i, q^_i> - <dk^_i, k^_i> + 2 sum_j Hm_ij (k^_i . k^_j) - 2 <e^{gamma_i} (dX S^T)_i, k^_i>
+//                              dG = <e^{G-gamma} (v_new dS'^T), k^> + e^G <dS', S>;   dg_t = sum_{i >= t} dgamma_i + dG
+//                            followed by the backward of the row normalisation.  <e^{G-gamma}(v_new dS'^T), k^> is also the
+//                            derivative with respect to a gate on the chunk's state update: the selector's straight-through
+//                            gradient for the linear operator (src/nats/ops/common/chunk_o.py:438-443, :487-492).
+//
+// Both kernels rebuild q^, k^ and the decay vectors from q, k, g; of the forward's workspace only TmB is read.
+#include "natsl_device.h"
+#include "natsl_host.h"
+
+namespace natsl {
+
+struct LinBwdParams {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* vn;       // v_new [tokens][H][V] (Mamba: v)
+  const bf16_t* d_o;      // [tokens][H][V]
+  const float* g;
+  const bf16_t* beta;
+  const bf16_t* s_all;    // state entering every chunk, [chunk][H][V][K]
+  bf16_t* ds_all;         // gradient of the state behind every chunk, same layout (written by the scan)
+  bf16_t* dv;             // dX [tokens][H][V] (written by the scan)
+  const float* dht;       // [B][H][K][V] or null
+  float* dh0;             // [B][H][K][V] or null
+  const float* gsum_blk;  // sum of g over every selector block, [B][TN][H]
+  const bf16_t* ws_tm;    // TmB of every chunk-head in the forward scan's operand order
+  const void* types;
+  int types_dtype;
+  bf16_t* dq;
+  bf16_t* dk;
+  float* dg;              // [tokens][H]
+  float* dbeta;           // [tokens][H]
+  float* dbeta_parts;     // [tokens][H][V / 16]: <dX, v_new> over each wave's 16 columns (scan -> per-chunk kernel)
+  float* sdot_parts;      // [chunk][H][V / 16]: <dS', S> over each wave's 16 columns, dS' still in fp32 (scan -> per-chunk kernel)
+  float* gate;            // [chunk][H]: derivative with respect to a gate on the chunk's state update
+  float* rb;              // [chunk][H]: f <dS', S_blockstart> behind a rolled-back block's last chunk (the decay's share of dg)
+  int B, T, H, HN, V, TN, block, nt;
+  float scale;
+  int flags;
+};
+
+constexpr int CB = 64;          // tokens per chunk
+constexpr int TP = CB + 8;      // row pitch (elements) of the 64-wide bf16 tiles
+
+NATSL_DEVICE bool lin_type_b(const void* types, int dtype, size_t i) {
+  float x = dtype == NATSL_F32 ? reinterpret_cast<const float*>(types)[i]
+                               : bf16_to_f32(reinterpret_cast<const bf16_t*>(types)[i]);
+  return rintf(x) == 1.0f;
+}
+
+NATSL_DEVICE void unpack8f(const u32x4 w, float* f) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = __uint_as_float(w[j] << 16);
+    f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+  }
+}
+
+// two 8-byte halves -> one operand: slots 0..3 from lo, 4..7 from hi
+NATSL_DEVICE bf16x8 join_u2(const u32x2 lo, const u32x2 hi) {
+  u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+  return __builtin_bit_cast(bf16x8, w);
+}
+
+// What rounding 8 fp32 to a bf16 operand leaves behind, as a second operand: a product with {pack8(a, b), pack8_rest(a, b)}
+// carries the fp32 values to about 16 bits.
+NATSL_DEVICE bf16x8 pack8_rest(const f32x4 a, const f32x4 b) {
+  f32x4 ra, rb;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    ra[r] = a[r] - __uint_as_float(__float_as_uint(a[r]) & 0xffff0000u);
+    rb[r] = b[r] - __uint_as_float(__float_as_uint(b[r]) & 0xffff0000u);
+  }
+  return pack8(ra, rb);
+}
+// (the first operand then has to be the TRUNCATED value, not the rounded one)
+NATSL_DEVICE bf16x8 pack8_trunc(const f32x4 a, const f32x4 b) {
+  u32x4 w;
+  w[0] = (__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u);
+  w[1] = (__float_as_uint(a[2]) >> 16) | (__float_as_uint(a[3]) & 0xffff0000u);
+  w[2] = (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u);
+  w[3] = (__float_as_uint(b[2]) >> 16) | (__float_as_uint(b[3]) & 0xffff0000u);
+  return __builtin_bit_cast(bf16x8, w);
+}
+
+// The chunk's scalars, by wave 0: gamma (inclusive cumsum of g), e^gamma, e^{G - gamma} (Mamba: exponent clamped at 0), beta.
+template <bool DELTA>
+NATSL_DEVICE void stage_scalars(const LinBwdParams& p, const int lane, const size_t row0, const int nvalid, const int h,
+                                float* gam, float* eg, float* ek, float* bet) {
+  const bool ok = lane < nvalid;
+  const size_t gi = (row0 + lane) * p.H + h;
+  float x = ok ? p.g[gi] : 0.f;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const float y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  const float gl = __shfl(x, 63);
+  float dk = gl - x;
+  if (!DELTA) dk = fminf(dk, 0.f);
+  gam[lane] = x;
+  eg[lane] = __expf(x);
+  ek[lane] = __expf(dk);
+  if (DELTA) bet[lane] = ok ? bf16_to_f32(p.beta[gi]) : 0.f;
+}
+
+// q^, k^ of the chunk into LDS, row-major [64][DK + 8] and transposed [DK][TP]; rows past the end are zero.
+template <int DK>
+NATSL_DEVICE void stage_qk(const LinBwdParams& p, const int tid, const size_t row0, const int nvalid, const int h, const bool l2,
+                           bf16_t* Qn, bf16_t* Kn, bf16_t* QT, bf16_t* KT, float* rq, float* rk) {
+  constexpr int KP = DK + 8, KL = DK / 32;
+  const int row = tid >> 2, sub = tid & 3;
+  const bool ok = row < nvalid;
+  const size_t off = ((row0 + row) * p.H + h) * DK;
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  u32x4 a[KL], b[KL];
+  float sq = 0.f, sk = 0.f;
+#pragma unroll
+  for (int i = 0; i < KL; ++i) {
+    a[i] = ok ? *reinterpret_cast<const u32x4*>(p.q + off + (sub + 4 * i) * 8) : z;
+    b[i] = ok ? *reinterpret_cast<const u32x4*>(p.k + off + (sub + 4 * i) * 8) : z;
+    float fa[8], fb[8];
+    unpack8f(a[i], fa);
+    unpack8f(b[i], fb);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sq += fa[e] * fa[e]; sk += fb[e] * fb[e]; }
+  }
+  sq += __shfl_xor(sq, 1); sq += __shfl_xor(sq, 2);
+  sk += __shfl_xor(sk, 1); sk += __shfl_xor(sk, 2);
+  const float fq = l2 ? rsqrtf(sq + 1e-6f) : 1.f, fk = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
+  if (sub == 0) { rq[row] = fq; rk[row] = fk; }
+#pragma unroll
+  for (int i = 0; i < KL; ++i) {
+    const int seg = sub + 4 * i;
+    float fa[8], fb[8];
+    unpack8f(a[i], fa);
+    unpack8f(b[i], fb);
+    u32x4 wa, wb;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wa[j] = pack_bf16x2(fa[2 * j] * fq, fa[2 * j + 1] * fq);
+      wb[j] = pack_bf16x2(fb[2 * j] * fk, fb[2 * j + 1] * fk);
+    }
+    *reinterpret_cast<u32x4*>(Qn + row * KP + seg * 8) = wa;
+    *reinterpret_cast<u32x4*>(Kn + row * KP + seg * 8) = wb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      QT[(seg * 8 + e) * TP + row] = (bf16_t)((wa[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+      KT[(seg * 8 + e) * TP + row] = (bf16_t)((wb[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+    }
+  }
+}
+
+// 64 rows x 64 columns of a token-major [tokens][H][V] tensor into LDS [64][TP]; rows past the end are zero.
+NATSL_DEVICE void stage_tokens64(const bf16_t* src, const int tid, const size_t row0, const int nvalid, const int H, const int V,
+                                 const int h, const int vcol0, bf16_t* dst) {
+  const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int pc = tid + 256 * it, row = pc >> 3, seg = pc & 7;
+    const u32x4 w = row < nvalid ? *reinterpret_cast<const u32x4*>(src + ((row0 + row) * H + h) * V + vcol0 + seg * 8) : z;
+    *reinterpret_cast<u32x4*>(dst + row * TP + seg * 8) = w;
+  }
+}
+
+// =============================================================================================
+// reverse scan
+// =============================================================================================
+template <int DK>
+struct BwdScanLds {
+  static constexpr int KP = DK + 8;
+  static constexpr int QN = 0, KN = QN + CB * KP, QT = KN + CB * KP, KT = QT + DK * TP, DO = KT + DK * TP, TT = DO + CB * TP;
+  static constexpr int VN = TT + CB * TP;
+  static constexpr int ELEMS = VN + CB * TP;
+  static constexpr int FL = ELEMS * 2;            // byte offset of the float area
+  static constexpr int TOTAL = FL + 7 * CB * 4;
+};
+
+template <int DK, bool DELTA>
+__global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams p) {
+  using L = BwdScanLds<DK>;
+  constexpr int KP = L::KP, KT16 = DK / 16, KS = DK / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* const sm = reinterpret_cast<bf16_t*>(smem);
+  bf16_t* const Qn = sm + L::QN;
+  bf16_t* const Kn = sm + L::KN;
+  bf16_t* const QT = sm + L::QT;
+  bf16_t* const KT = sm + L::KT;
+  bf16_t* const DOs = sm + L::DO;
+  bf16_t* const TT = sm + L::TT;
+  bf16_t* const VNs = sm + L::VN;
+  float* const fl = reinterpret_cast<float*>(smem + L::FL);
+  float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *sqv = fl + 6 * CB;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
+  const int nsplit = p.V / 64;
+  const int chain = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
+  const int n = chain / p.H, h = chain % p.H;
+  const int bos = n * p.T, len = p.T, chunk_off = n * p.nt;
+  const int NT = p.nt;
+  const int vcol0 = split * 64;
+  const int col = vcol0 + 16 * wave + x16;
+  const int per = p.block / CB;
+  const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0, intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
+  const bool l2 = DELTA && (p.flags & NATSL_QK_L2NORM) != 0;
+  const int hn = h / (p.H / p.HN);
+
+  // TmB^T: the part above the stored operands stays zero
+  if (DELTA)
+    for (int i = tid; i < CB * TP; i += 256) TT[i] = 0;
+
+  f32x4 dS[KT16], pend[KT16];
+#pragma unroll
+  for (int m = 0; m < KT16; ++m)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      dS[m][r] = p.dht ? p.dht[((size_t)chain * DK + 16 * m + 4 * g4 + r) * p.V + col] : 0.f;
+      pend[m][r] = 0.f;
+    }
+
+  for (int c = NT - 1; c >= 0; --c) {
+    const int t0 = c * CB, nvalid = min(CB, len - t0);
+    const size_t row0 = (size_t)bos + t0;
+    __syncthreads();   // every wave is done with the previous chunk's tiles
+    if (wave == 0) stage_scalars<DELTA>(p, lane, row0, nvalid, h, gam, eg, ek, bet);
+    stage_qk<DK>(p, tid, row0, nvalid, h, l2, Qn, Kn, QT, KT, rq, rk);
+    stage_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, vcol0, DOs);
+    if (DELTA) {
+      stage_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, vcol0, VNs);
+      // TmB^T [j][i] from the six stored operands: operand (t, s) at 2t + s, scan-lane (x, g) at (16 g + x) * 8, slot e stands
+      // for column 32 s + 16 (e / 4) + 4 g + e % 4 of row 16 t + x
+      const bf16_t* tm = p.ws_tm + ((size_t)(chunk_off + c) * p.H + h) * (CB * CB);
+      for (int pc = tid; pc < 6 * 64; pc += 256) {
+        const int oi = pc >> 6, ln = pc & 63, o = oi < 2 ? 2 * oi : oi + 2, t = o >> 1, s = o & 1, x = ln & 15, gg = ln >> 4;
+        const u32x4 w = *reinterpret_cast<const u32x4*>(tm + o * 512 + ln * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = 32 * s + 16 * (e >> 2) + 4 * gg + (e & 3);
+          TT[j * TP + 16 * t + x] = (bf16_t)((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < CB) sqv[tid] = p.scale * eg[tid];
+    // (sqv is read below only after the state-gradient products; the barrier in between is the one after Y2)
+
+    // ---- dS' of this chunk goes out as it arrived; a rolled-back block's leaves the chain here --------------------------
+    {
+      const size_t so = (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 4 * g4;
+      bf16_t* dso = p.ds_all + so;
+      const bf16_t* sin = p.s_all + so;
+      float sd = 0.f;
+#pragma unroll
+      for (int m = 0; m < KT16; ++m) {
+        u32x2 w = {pack_bf16x2(dS[m][0], dS[m][1]), pack_bf16x2(dS[m][2], dS[m][3])};
+        *reinterpret_cast<u32x2*>(dso + 16 * m) = w;
+        const u32x2 sw = *reinterpret_cast<const u32x2*>(sin + 16 * m);
+        sd += dS[m][0] * __uint_as_float(sw[0] << 16) + dS[m][1] * __uint_as_float(sw[0] & 0xffff0000u) +
+              dS[m][2] * __uint_as_float(sw[1] << 16) + dS[m][3] * __uint_as_float(sw[1] & 0xffff0000u);
+      }
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) sd += __shfl_xor(sd, d);
+      if (lane == 0) p.sdot_parts[((size_t)(chunk_off + c) * p.H + h) * (p.V / 16) + 4 * split + wave] = sd;
+    }
+    const int blk = t0 / p.block;
+    const bool last = ((c + 1) % per == 0) || (c == NT - 1);
+    if (last) {
+      const bool lin = lin_type_b(p.types, p.types_dtype, ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1);
+      const float f = lin ? 0.f : (decay ? __expf(p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h]) : 1.f);
+#pragma unroll
+      for (int m = 0; m < KT16; ++m)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          pend[m][r] = dS[m][r] * f;
+          if (!lin) dS[m][r] = 0.f;
+        }
+    }
+    const float dec = __expf(gam[CB - 1]);
+
+    // ---- Y1 = K~ dS' ----------------------------------------------------------------------------------------------------
+    f32x4 DV[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) DV[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    {
+      bf16x8 DSB[KS], DSR[KS];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        DSB[s] = pack8_trunc(dS[2 * s], dS[2 * s + 1]);
+        DSR[s] = pack8_rest(dS[2 * s], dS[2 * s + 1]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const bf16_t* kr = Kn + (16 * t + x16) * KP + 32 * s + 4 * g4;
+          const bf16x8 a = join_u2(*reinterpret_cast<const u32x2*>(kr), *reinterpret_cast<const u32x2*>(kr + 16));
+          DV[t] = mfma16(a, DSR[s], DV[t]);
+          DV[t] = mfma16(a, DSB[s], DV[t]);
+        }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const f32x4 e4 = *reinterpret_cast<const f32x4*>(ek + 16 * t + 4 * g4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) DV[t][r] *= e4[r];
+      }
+    }
+    // ---- dO in accumulator layout (lane = column, registers = tokens 16 t + 4 g + r) ------------------------------------
+    f32x4 DOc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) DOc[t][r] = bf16_to_f32(DOs[(16 * t + 4 * g4 + r) * TP + 16 * wave + x16]);
+    // ---- Y2 = P^T dO: P^T's operands are formed here; Z = q^ k^^T leaves lane (x, g) with key 16 tj + x against queries
+    //      16 ti + 4 g + r, the four slots this lane holds of operand (tj, ti / 2), half ti % 2 ------------------------------
+    if (intra) {
+      const bf16x8 DOB[2] = {pack8(DOc[0], DOc[1]), pack8(DOc[2], DOc[3])};
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        const float gj = gam[16 * tj + x16];
+        f32x4 Z[4];
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) {
+          Z[ti] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          if (ti >= tj) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+              const bf16x8 a = *reinterpret_cast<const bf16x8*>(Qn + (16 * ti + x16) * KP + 32 * s + 8 * g4);
+              const bf16x8 b = *reinterpret_cast<const bf16x8*>(Kn + (16 * tj + x16) * KP + 32 * s + 8 * g4);
+              Z[ti] = mfma16(a, b, Z[ti]);
+            }
+            const f32x4 gi = *reinterpret_cast<const f32x4*>(gam + 16 * ti + 4 * g4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const bool vis = ti > tj || 4 * g4 + r >= x16;
+              Z[ti][r] = vis ? Z[ti][r] * p.scale * __expf(gi[r] - gj) : 0.f;
+            }
+          }
+        }
+        if (tj < 2) DV[tj] = mfma16(pack8(Z[0], Z[1]), DOB[0], DV[tj]);
+        DV[tj] = mfma16(pack8(Z[2], Z[3]), DOB[1], DV[tj]);
+      }
+    }
+    // ---- dX = TmB^T dv_new ----------------------------------------------------------------------------------------------
+    f32x4 DX[4];
+    if (DELTA) {
+      const bf16x8 DVB[2] = {pack8_trunc(DV[0], DV[1]), pack8_trunc(DV[2], DV[3])};
+      const bf16x8 DVR[2] = {pack8_rest(DV[0], DV[1]), pack8_rest(DV[2], DV[3])};
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        DX[tj] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          if (2 * s2 + 1 >= tj) {
+            const bf16_t* tr = TT + (16 * tj + x16) * TP + 32 * s2 + 4 * g4;
+            const bf16x8 a = join_u2(*reinterpret_cast<const u32x2*>(tr), *reinterpret_cast<const u32x2*>(tr + 16));
+            DX[tj] = mfma16(a, DVR[s2], DX[tj]);
+            DX[tj] = mfma16(a, DVB[s2], DX[tj]);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) DX[t] = DV[t];
+    }
+    // dv = dX; for dbeta_i = <dX_i, v_new_i> / beta_i^2, this wave's 16 columns of the inner product (dX still in fp32)
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int tok = 16 * t + 4 * g4 + r;
+        if (tok < nvalid) p.dv[((row0 + tok) * p.H + h) * p.V + col] = f32_to_bf16(DX[t][r]);
+        if (DELTA) {
+          float pb = DX[t][r] * bf16_to_f32(VNs[tok * TP + 16 * wave + x16]);
+#pragma unroll
+          for (int d = 1; d < 16; d <<= 1) pb += __shfl_xor(pb, d);
+          if (x16 == 0 && tok < nvalid) p.dbeta_parts[((row0 + tok) * p.H + h) * (p.V / 16) + 4 * split + wave] = pb;
+        }
+      }
+    __syncthreads();   // sqv
+    // ---- dS = e^G dS' + Q~^T dO - W^T dX --------------------------------------------------------------------------------
+    {
+      f32x4 A1[4], A2[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(sqv + 16 * t + 4 * g4);
+        const f32x4 e4 = *reinterpret_cast<const f32x4*>(eg + 16 * t + 4 * g4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          A1[t][r] = DOc[t][r] * s4[r];
+          A2[t][r] = -DX[t][r] * e4[r];
+        }
+      }
+      const bf16x8 B1[2] = {pack8(A1[0], A1[1]), pack8(A1[2], A1[3])};
+      const bf16x8 B2[2] = {pack8(A2[0], A2[1]), pack8(A2[2], A2[3])};
+#pragma unroll
+      for (int m = 0; m < KT16; ++m) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dS[m][r] *= dec;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const bf16_t* qr = QT + (16 * m + x16) * TP + 32 * s2 + 4 * g4;
+          dS[m] = mfma16(join_u2(*reinterpret_cast<const u32x2*>(qr), *reinterpret_cast<const u32x2*>(qr + 16)), B1[s2], dS[m]);
+          if (DELTA) {
+            const bf16_t* kr = KT + (16 * m + x16) * TP + 32 * s2 + 4 * g4;
+            dS[m] = mfma16(join_u2(*reinterpret_cast<const u32x2*>(kr), *reinterpret_cast<const u32x2*>(kr + 16)), B2[s2], dS[m]);
+          }
+        }
+      }
+    }
+    if (c % per == 0) {
+#pragma unroll
+      for (int m = 0; m < KT16; ++m)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          dS[m][r] += pend[m][r];
+          pend[m][r] = 0.f;
+        }
+    }
+  }
+  if (p.dh0) {
+#pragma unroll
+    for (int m = 0; m < KT16; ++m)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p.dh0[((size_t)chain * DK + 16 * m + 4 * g4 + r) * p.V + col] = dS[m][r];
+  }
+}
+
+// =============================================================================================
+// per-chunk gradients
+// =============================================================================================
+template <int DK>
+struct BwdChunkLds {
+  static constexpr int KP = DK + 8;
+  // phase 1 (the products that contract over V, one 64-column slice at a time)
+  static constexpr int DO = 0, DX = DO + CB * TP, VN = DX + CB * TP, ST = VN + CB * TP, DST = ST + DK * TP, P1 = DST + DK * TP;
+  // phase 2 (the products that contract over tokens)
+  static constexpr int QN = 0, KN = QN + CB * KP, QT = KN + CB * KP, KT = QT + DK * TP, GN = KT + DK * TP, GT = GN + CB * TP,
+                       HS = GT + CB * TP, P2 = HS + CB * TP;
+  static constexpr int ELEMS = P1 > P2 ? P1 : P2;
+  static constexpr int FL = ELEMS * 2;
+  static constexpr int TOTAL = FL + (7 * CB + 8) * 4;
+};
+
+template <int DK, bool DELTA>
+__global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParams p) {
+  using L = BwdChunkLds<DK>;
+  constexpr int KP = L::KP, KT16 = DK / 16, KS = DK / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* const sm = reinterpret_cast<bf16_t*>(smem);
+  float* const fl = reinterpret_cast<float*>(smem + L::FL);
+  float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *dgam = fl + 6 * CB;
+  float* red = fl + 7 * CB;   // [0] <dS', S>, [1] sum of the gate terms, [2] <dS', S_blockstart>
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
+  const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
+  const int n = gc / p.nt, c = gc - n * p.nt;
+  const int t0 = c * CB, nvalid = min(CB, p.T - t0);
+  const size_t row0 = (size_t)n * p.T + t0;
+  const int per = p.block / CB;
+  const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0, intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
+  const bool l2 = DELTA && (p.flags & NATSL_QK_L2NORM) != 0;
+  const int hn = h / (p.H / p.HN);
+  const int blk = t0 / p.block;
+  const bool last = ((c + 1) % per == 0) || (c == p.nt - 1);
+  const bool lin = lin_type_b(p.types, p.types_dtype, ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1);
+  const bool rolled = last && !lin;
+  const bool want_rb = rolled && decay;
+  const int c_first = (c / per) * per;
+
+  if (wave == 0) stage_scalars<DELTA>(p, lane, row0, nvalid, h, gam, eg, ek, bet);
+  if (tid < 8) red[tid] = 0.f;
+
+  // ---- phase 1 -------------------------------------------------------------------------------------------------------
+  bf16_t* const DOs = sm + L::DO;
+  bf16_t* const DXs = sm + L::DX;
+  bf16_t* const VNs = sm + L::VN;
+  bf16_t* const ST = sm + L::ST;
+  bf16_t* const DST = sm + L::DST;
+  f32x4 Nm[4], Mm[4], DQ2[KT16], DW[KT16], DK3[KT16];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) { Nm[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; Mm[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+  for (int m = 0; m < KT16; ++m) {
+    DQ2[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; DW[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; DK3[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  float srb = 0.f;
+  const size_t unit = (size_t)gc * p.H + h;
+  const bf16_t* s_src = p.s_all + unit * p.V * DK;
+  const bf16_t* ds_src = p.ds_all + unit * p.V * DK;
+  const bf16_t* sf_src = p.s_all + ((size_t)(n * p.nt + c_first) * p.H + h) * p.V * DK;
+  for (int vs = 0; vs < p.V / 64; ++vs) {
+    __syncthreads();
+    stage_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, 64 * vs, DOs);
+    stage_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, 64 * vs, VNs);
+    if (DELTA) stage_tokens64(p.dv, tid, row0, nvalid, p.H, p.V, h, 64 * vs, DXs);
+    // the state and its gradient, [V][K] in memory, as [K][64 columns] in LDS
+    for (int pc = tid; pc < 64 * (DK / 8); pc += 256) {
+      const int v = pc & 63, seg = pc >> 6;
+      const size_t off = (size_t)(64 * vs + v) * DK + seg * 8;
+      const u32x4 ws = *reinterpret_cast<const u32x4*>(s_src + off);
+      const u32x4 wd = *reinterpret_cast<const u32x4*>(ds_src + off);
+      float fs[8], fd[8];
+      unpack8f(ws, fs);
+      unpack8f(wd, fd);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ST[(seg * 8 + e) * TP + v] = (bf16_t)((ws[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        DST[(seg * 8 + e) * TP + v] = (bf16_t)((wd[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+      }
+      if (want_rb) {
+        float ff[8];
+        unpack8f(*reinterpret_cast<const u32x4*>(sf_src + off), ff);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) srb += ff[e] * fd[e];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const bf16x8 a_do = *reinterpret_cast<const bf16x8*>(DOs + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+      const bf16x8 a_vn = *reinterpret_cast<const bf16x8*>(VNs + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+      bf16x8 a_dx = a_vn;
+      if (DELTA) a_dx = *reinterpret_cast<const bf16x8*>(DXs + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(VNs + (16 * tj + x16) * TP + 32 * s + 8 * g4);
+        Nm[tj] = mfma16(a_do, b, Nm[tj]);
+        if (DELTA) Mm[tj] = mfma16(a_dx, b, Mm[tj]);
+      }
+#pragma unroll
+      for (int m = 0; m < KT16; ++m) {
+        const bf16x8 bs = *reinterpret_cast<const bf16x8*>(ST + (16 * m + x16) * TP + 32 * s + 8 * g4);
+        const bf16x8 bd = *reinterpret_cast<const bf16x8*>(DST + (16 * m + x16) * TP + 32 * s + 8 * g4);
+        DQ2[m] = mfma16(a_do, bs, DQ2[m]);
+        if (DELTA) DW[m] = mfma16(a_dx, bs, DW[m]);
+        DK3[m] = mfma16(a_vn, bd, DK3[m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) srb += __shfl_xor(srb, d);
+  if (lane == 0) atomicAdd(&red[2], srb);
+  if (tid == 64) {
+    // <dS', S>: the scan's partial sums, in a fixed order
+    const float* pp = p.sdot_parts + unit * (p.V / 16);
+    float sum = 0.f;
+    for (int i = 0; i < p.V / 16; ++i) sum += pp[i];
+    red[0] = sum;
+  }
+
+  // ---- phase 2 -------------------------------------------------------------------------------------------------------
+  bf16_t* const Qn = sm + L::QN;
+  bf16_t* const Kn = sm + L::KN;
+  bf16_t* const QT = sm + L::QT;
+  bf16_t* const KT = sm + L::KT;
+  bf16_t* const Gn = sm + L::GN;
+  bf16_t* const GT = sm + L::GT;
+  bf16_t* const Hs = sm + L::HS;
+  __syncthreads();   // phase 1's tiles are dead
+  stage_qk<DK>(p, tid, row0, nvalid, h, l2, Qn, Kn, QT, KT, rq, rk);
+  if (DELTA)
+    for (int i = tid; i < CB * TP; i += 256) Hs[i] = 0;
+  __syncthreads();
+
+  // this lane's rows i = 16 wave + 4 g + r; its column in tile tj is 16 tj + x
+  const f32x4 gi4 = *reinterpret_cast<const f32x4*>(gam + 16 * wave + 4 * g4);
+  f32x4 rsH = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int tj = 0; tj < 4; ++tj) {
+    const int j = 16 * tj + x16;
+    const float gj = gam[j];
+    f32x4 KK = {0.f, 0.f, 0.f, 0.f};
+    if (DELTA) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(Kn + (16 * wave + x16) * KP + 32 * s + 8 * g4);
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(Kn + (16 * tj + x16) * KP + 32 * s + 8 * g4);
+        KK = mfma16(a, b, KK);
+      }
+    }
+    u32x2 gw;
+    float gv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = 16 * wave + 4 * g4 + r;
+      const float Lij = i >= j ? __expf(gi4[r] - gj) : 0.f;
+      gv[r] = intra ? p.scale * Nm[tj][r] * Lij : 0.f;
+      Gn[i * TP + j] = f32_to_bf16(gv[r]);
+      if (DELTA) {
+        if (i > j) {
+          const float hv = -Mm[tj][r] * Lij;
+          rsH[r] += hv * KK[r];
+          const bf16_t hb = f32_to_bf16(hv);
+          Hs[i * TP + j] = hb;
+          Hs[j * TP + i] = hb;
+        }
+      }
+    }
+    gw[0] = pack_bf16x2(gv[0], gv[1]);
+    gw[1] = pack_bf16x2(gv[2], gv[3]);
+    *reinterpret_cast<u32x2*>(GT + j * TP + 16 * wave + 4 * g4) = gw;
+  }
+  if (DELTA) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1) rsH[r] += __shfl_xor(rsH[r], d);
+  }
+  __syncthreads();
+
+  // dq^, dk^ of this wave's 16 tokens: lane = K column 16 m + x, registers = tokens 16 wave + 4 g + r
+  const f32x4 eg4 = *reinterpret_cast<const f32x4*>(eg + 16 * wave + 4 * g4);
+  const f32x4 ek4 = *reinterpret_cast<const f32x4*>(ek + 16 * wave + 4 * g4);
+  const float nr = rolled ? 0.f : 1.f;
+  f32x4 a_i = {0.f, 0.f, 0.f, 0.f}, b_i = {0.f, 0.f, 0.f, 0.f}, t2_i = {0.f, 0.f, 0.f, 0.f}, t3_i = {0.f, 0.f, 0.f, 0.f};
+  bf16x8 ga[2], gta[2], ha[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    ga[s] = *reinterpret_cast<const bf16x8*>(Gn + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+    gta[s] = *reinterpret_cast<const bf16x8*>(GT + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+    ha[s] = gta[s];
+    if (DELTA) ha[s] = *reinterpret_cast<const bf16x8*>(Hs + (16 * wave + x16) * TP + 32 * s + 8 * g4);
+  }
+  f32x4 DQ[KT16], DKg[KT16];
+#pragma unroll
+  for (int m = 0; m < KT16; ++m) {
+    float qv[4], kv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      qv[r] = bf16_to_f32(Qn[(16 * wave + 4 * g4 + r) * KP + 16 * m + x16]);
+      kv[r] = bf16_to_f32(Kn[(16 * wave + 4 * g4 + r) * KP + 16 * m + x16]);
+    }
+    f32x4 dq, dk;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float w2 = DELTA ? eg4[r] * DW[m][r] : 0.f, w3 = ek4[r] * DK3[m][r];
+      dq[r] = p.scale * eg4[r] * DQ2[m][r];
+      dk[r] = nr * w3 - w2;
+      t2_i[r] += w2 * kv[r];
+      t3_i[r] += w3 * kv[r];
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const bf16x8 bk = *reinterpret_cast<const bf16x8*>(KT + (16 * m + x16) * TP + 32 * s + 8 * g4);
+      const bf16x8 bq = *reinterpret_cast<const bf16x8*>(QT + (16 * m + x16) * TP + 32 * s + 8 * g4);
+      dq = mfma16(ga[s], bk, dq);
+      dk = mfma16(gta[s], bq, dk);
+      if (DELTA) dk = mfma16(ha[s], bk, dk);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      a_i[r] += dq[r] * qv[r];
+      b_i[r] += dk[r] * kv[r];
+    }
+    DQ[m] = dq;
+    DKg[m] = dk;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+      a_i[r] += __shfl_xor(a_i[r], d);
+      b_i[r] += __shfl_xor(b_i[r], d);
+      t2_i[r] += __shfl_xor(t2_i[r], d);
+      t3_i[r] += __shfl_xor(t3_i[r], d);
+    }
+  if (x16 == 0) {
+    float t3s = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      dgam[16 * wave + 4 * g4 + r] = a_i[r] - b_i[r] + 2.f * rsH[r] - 2.f * t2_i[r];
+      t3s += t3_i[r];
+    }
+    atomicAdd(&red[1], t3s);
+  }
+  __syncthreads();   // every wave is done with q^, k^ and the weight tiles; dgam and red are complete
+
+  // ---- the row normalisation's backward, then out through LDS (rows of KP elements in the space of q^, k^ tiles) --------
+  {
+    const f32x4 rq4 = *reinterpret_cast<const f32x4*>(rq + 16 * wave + 4 * g4);
+    const f32x4 rk4 = *reinterpret_cast<const f32x4*>(rk + 16 * wave + 4 * g4);
+#pragma unroll
+    for (int m = 0; m < KT16; ++m)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * wave + 4 * g4 + r, kc = 16 * m + x16;
+        float dq = DQ[m][r], dk = DKg[m][r];
+        if (l2) {
+          const float qv = bf16_to_f32(Qn[i * KP + kc]), kv = bf16_to_f32(Kn[i * KP + kc]);
+          dq = rq4[r] * (dq - qv * a_i[r]);
+          dk = rk4[r] * (dk - kv * b_i[r]);
+        }
+        // (each element is read and then overwritten by the same lane)
+        Qn[i * KP + kc] = f32_to_bf16(dq);
+        Kn[i * KP + kc] = f32_to_bf16(dk);
+      }
+  }
+  if (DELTA && wave == 1 && lane < nvalid) {
+    const float* pp = p.dbeta_parts + ((row0 + lane) * p.H + h) * (p.V / 16);
+    float sum = 0.f;
+    for (int i = 0; i < p.V / 16; ++i) sum += pp[i];
+    p.dbeta[(row0 + lane) * p.H + h] = sum / (bet[lane] * bet[lane]);
+  }
+  if (wave == 0) {
+    // dg_t = sum_{i >= t} dgamma_i + dG
+    const float dG = nr * (red[1] + __expf(gam[CB - 1]) * red[0]);
+    float x = dgam[lane];
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float y = __shfl_down(x, d);
+      if (lane + d < 64) x += y;
+    }
+    if (lane < nvalid) p.dg[(row0 + lane) * p.H + h] = x + dG;
+    if (lane == 0) {
+      p.gate[unit] = red[1];
+      p.rb[unit] = want_rb ? __expf(p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h]) * red[2] : 0.f;
+    }
+  }
+  __syncthreads();
+  for (int pc = tid; pc < CB * (DK / 8); pc += 256) {
+    const int row = pc / (DK / 8), seg = pc % (DK / 8);
+    if (row < nvalid) {
+      const size_t off = ((row0 + row) * p.H + h) * DK + seg * 8;
+      *reinterpret_cast<u32x4*>(p.dq + off) = *reinterpret_cast<const u32x4*>(Qn + row * KP + seg * 8);
+      *reinterpret_cast<u32x4*>(p.dk + off) = *reinterpret_cast<const u32x4*>(Kn + row * KP + seg * 8);
+    }
+  }
+}
+
+template <int DK, bool DELTA>
+static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* what) {
+  {
+    using L = BwdScanLds<DK>;
+    auto kern = linear_bwd_scan_kernel<DK, DELTA>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
+    if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.B * p.H * (p.V / 64))), dim3(256), L::TOTAL, stream, p);
+    const int rc = check_launch(what);
+    if (rc != NATSL_OK) return rc;
+  }
+  {
+    using L = BwdChunkLds<DK>;
+    auto kern = linear_bwd_chunk_kernel<DK, DELTA>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
+    if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.B * p.nt * p.H)), dim3(256), L::TOTAL, stream, p);
+    return check_launch(what);
+  }
+}
+
+}  // namespace natsl
+
+using namespace natsl;
+
+extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void* k, const void* v_new, const float* g, const void* beta,
+                                      const void* d_o, const float* dht, const void* chunk_states, const void* types, int types_dtype,
+                                      const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
+                                      float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
+                                      int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
+                                      natsl_stream_t stream) {
+  const char* what = "natsl_linear_chunk_bwd";
+  if (!q || !k || !v_new || !g || !d_o || !chunk_states || !types || !g_block_sums || !d_chunk_states || !dq || !dk || !dv || !dg ||
+      !d_gate || !d_rollback || !state_dot_parts || (delta_rule && (!beta || !dbeta || !dbeta_parts || !workspace)))
+    return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
+  if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
+  if (B <= 0 || T <= 0 || H <= 0 || HN <= 0 || TN <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
+  if (H % HN) return fail(NATSL_ERR_INVALID, "%s: H=%d must be a multiple of HN=%d", what, H, HN);
+  if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
+  if (V % 64 || V <= 0) return fail(NATSL_ERR_UNSUPPORTED, "%s: V=%d must be a multiple of 64", what, V);
+  if (TN != cdiv(T, block)) return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d", what, TN, T, block);
+  LinBwdParams p;
+  p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.vn = (const bf16_t*)v_new; p.d_o = (const bf16_t*)d_o; p.g = g;
+  p.beta = (const bf16_t*)beta; p.s_all = (const bf16_t*)chunk_states; p.ds_all = (bf16_t*)d_chunk_states; p.dv = (bf16_t*)dv;
+  p.dht = dht; p.dh0 = dh0; p.gsum_blk = g_block_sums; p.ws_tm = (const bf16_t*)workspace; p.types = types; p.types_dtype = types_dtype;
+  p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dg = dg; p.dbeta = dbeta; p.dbeta_parts = dbeta_parts; p.sdot_parts = state_dot_parts; p.gate = d_gate; p.rb = d_rollback;
+  p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block; p.nt = cdiv(T, CB);
+  p.scale = scale; p.flags = flags;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (delta_rule) {
+    if (K == 128) return launch_bwd<128, true>(p, s, what);
+    if (K == 64) return launch_bwd<64, true>(p, s, what);
+    if (K == 192) return launch_bwd<192, true>(p, s, what);
+  } else {
+    p.flags &= ~NATSL_QK_L2NORM;
+    if (K == 128) return launch_bwd<128, false>(p, s, what);
+    if (K == 64) return launch_bwd<64, false>(p, s, what);
+    if (K == 192) return launch_bwd<192, false>(p, s, what);
+  }
+  return fail(NATSL_ERR_UNSUPPORTED, "%s: key dim K=%d not built (supported: 64, 128, 192)", what, K);
+}

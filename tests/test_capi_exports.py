@@ -45,7 +45,7 @@ def test_argument_validation_needs_no_gpu():
     p = ctypes.c_void_p(256)
     rc = L.natsl_softmax_sparse_fwd(p, p, p, p, p, p, 1, p, p, 1, 256, 4, 4, 4, 96, 96, 4, 64, 0.1, 1, 1, None, 0, 0, None)
     assert rc == -2 and b"head dims" in L.natsl_last_error()
-    rc = L.natsl_gdn_chunk_fwd(p, p, p, p, p, None, p, None, None, None, None, p, 1, 1, 256, 4, 4, 128, 128, 4, 64, 0.1, 7, p, 16, 1,
+    rc = L.natsl_gdn_chunk_fwd(p, p, p, p, p, None, p, None, None, None, None, None, p, 1, 1, 256, 4, 4, 128, 128, 4, 64, 0.1, 7, p, 16, 1,
                                None, 0, 0, None)
     assert rc == -3 and b"workspace" in L.natsl_last_error()
     # the softmax backward's 32-bit row offsets: T * HQ * max(K, V) * 2 bytes must stay below 2^32 -- refused on the host,

@@ -1,0 +1,88 @@
+"""GPU parity: the backward kernels of the two linear branches (natsl_linear_chunk_bwd: reverse scan + per-chunk gradients)
+against autograd through the fp64 chunked oracle (oracle.linear_branch.linear_branch_bwd), and the torch formulation of the
+same method against the same oracle.
+
+Tolerance: rel-L2 5e-3 and max-abs 2e-2 of the reference's largest magnitude for dq, dk, dv, dh0; rel-L2 1e-2 for the
+per-token scalars dg and dbeta and for the selector's gate gradient (sums of large terms of both signs over bf16-rounded
+intermediates)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import linear_branch as LB
+from tests._util import make_gates, make_qkv, make_types, max_abs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+CASES = [
+    # kind, B, T, H, HN, K, V, block, decay, intra, h0, dht, invalid
+    ('gdn', 2, 512, 4, 2, 128, 128, 64, True, True, True, True, False),
+    ('gdn', 1, 300, 4, 2, 64, 64, 128, True, True, False, True, True),      # ragged last chunk, incomplete last block
+    ('gdn', 1, 640, 2, 1, 192, 384, 256, True, True, True, False, True),    # the 760M geometry
+    ('gdn', 1, 512, 6, 6, 128, 256, 64, False, True, True, True, False),    # the 340M geometry, no decay on rolled-back blocks
+    ('gdn', 1, 256, 2, 2, 128, 64, 64, True, False, True, True, True),      # no intra-chunk term
+    ('mamba', 2, 512, 4, 2, 128, 64, 64, True, True, True, True, True),
+    ('mamba', 1, 330, 4, 4, 64, 128, 128, False, True, False, True, False),
+]
+
+
+def _inputs(kind, B, T, H, HN, K, V, block, seed):
+    q, k, v = make_qkv(B, T, H, K, V, seed)
+    if kind == 'mamba':
+        q, k = F.normalize(q.float(), dim=-1).bfloat16(), F.normalize(k.float(), dim=-1).bfloat16()
+    g, beta = make_gates(B, T, H, seed + 1)
+    ty = make_types(B, -(-T // block), HN, 0.4, seed + 2, torch.bfloat16)
+    gen = torch.Generator().manual_seed(seed + 3)
+    init = torch.randn(B, H, K, V, generator=gen) * 0.3
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.3      # the scale of the states themselves
+    return q, k, v, g, beta, ty, init, do, dht
+
+
+def _check(out, ref, kind, h0):
+    names = ['dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0']
+    for name, got in zip(names, out[:6]):
+        if name == 'dbeta' and kind != 'gdn':
+            assert got is None
+            continue
+        if name == 'dh0' and not h0:
+            assert got is None
+            continue
+        want = ref[name]
+        tol = 1e-2 if name in ('dg', 'dbeta') else 5e-3
+        rl, ma, top = rel_l2(got.float().cpu(), want), max_abs(got.float().cpu(), want), float(want.abs().max())
+        assert rl <= tol and ma <= 2e-2 * max(top, 1.0), f"{name}: rel-L2 {rl:.3e}, max-abs {ma:.3e} (largest reference value {top:.3e})"
+    dn, want = out[6].double().cpu(), ref['dnats']
+    assert rel_l2(dn, want) <= 1e-2 and float((dn - want).abs().max()) <= 2e-2 * max(float(want.abs().max()), 1.0), \
+        f"dnats: rel-L2 {rel_l2(dn, want):.3e}"
+
+
+@pytest.mark.parametrize("which", ['hip', 'torch'])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"{c[0]}-T{c[2]}-K{c[5]}-V{c[6]}-b{c[7]}")
+def test_linear_branch_backward(case, which):
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    kind, B, T, H, HN, K, V, block, decay, intra, h0, dht_on, invalid = case
+    q, k, v, g, beta, ty, init, do, dht = _inputs(kind, B, T, H, HN, K, V, block, 100 + K + V)
+    scale = K ** -0.5 if kind == 'gdn' else 1.0
+    l2 = kind == 'gdn'
+    ref = LB.linear_branch_bwd(kind, q, k, v, g, beta if kind == 'gdn' else None, ty[..., 1], scale, do, dht if dht_on else None,
+                               init if h0 else None, block, decay, l2, intra, invalid)
+    d = lambda t: t.to(DEV)
+    fn = B_.linear_chunk_backward_hip if which == 'hip' else B_.linear_chunk_backward_torch
+    out = fn(kind, d(q), d(k), d(v), d(g), d(beta) if kind == 'gdn' else None, d(init) if h0 else None, d(ty), scale, block, decay,
+             l2, intra, d(do), d(dht) if dht_on else None, invalid)
+    torch.cuda.synchronize()
+    _check(out, ref, kind, h0)
+
+
+def test_backward_entry_rejects_what_is_not_built():
+    """Argument errors come back as codes from the host, before any launch."""
+    import ctypes
+    from neuralattentionsearchlinear_amd import _capi
+    L = _capi.lib()
+    p = ctypes.c_void_p(256)
+    args = lambda K, V, block: (1, p, p, p, p, p, p, None, p, p, 1, p, p, p, p, p, p, p, p, p, p, None, p, p, 1, 256, 4, 4, K, V, 256 // block, block,
+                                0.1, 7, 1, None)
+    assert L.natsl_linear_chunk_bwd(*args(96, 64, 64)) == -2 and b"K=96" in L.natsl_last_error()
+    assert L.natsl_linear_chunk_bwd(*args(128, 48, 64)) == -2 and b"V=48" in L.natsl_last_error()
