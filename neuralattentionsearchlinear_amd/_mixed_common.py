@@ -193,7 +193,7 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
 class _MixedFunction(torch.autograd.Function):
     """The mixed operator with its backward (src/nats/ops/mixed_ops/mixed_attn_gdn.py:193-283,
     src/nats/ops/mixed_ops/mixed_attn_mamba.py:194-292): the softmax branch's gradients come from the HIP backward
-    (natsl_softmax_sparse_bwd), the linear branch's from the differentiable chunked forward in _linear_bwd.py; the
+    (natsl_softmax_sparse_bwd), the linear branch's from natsl_linear_chunk_bwd behind _linear_bwd.linear_chunk_backward; the
     selector's straight-through gradient is returned for nats_block_types, column 0 = softmax op, column 1 = linear op."""
 
     @staticmethod

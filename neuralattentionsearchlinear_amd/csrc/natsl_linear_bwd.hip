@@ -30,6 +30,9 @@
 //                            gradient for the linear operator (src/nats/ops/common/chunk_o.py:438-443, :487-492).
 //
 // Both kernels rebuild q^, k^ and the decay vectors from q, k, g; of the forward's workspace only TmB is read.
+// Tiles sit in LDS row-major as they lie in memory; an operand that needs the other orientation (k^T, q^T, S, dS', TmB^T) is
+// fetched with the transposing read ds_read_b64_tr_b16 (within 16 lanes, lane i names four consecutive elements R_i and
+// receives element i % 4 of R_{i/4}, R_{4+i/4}, R_{8+i/4}, R_{12+i/4}): two such reads are the eight contraction slots of a lane.
 #include "natsl_device.h"
 #include "natsl_host.h"
 
@@ -108,45 +111,44 @@ NATSL_DEVICE bf16x8 pack8_trunc(const f32x4 a, const f32x4 b) {
   return __builtin_bit_cast(bf16x8, w);
 }
 
-// The chunk's scalars, by wave 0: gamma (inclusive cumsum of g), e^gamma, e^{G - gamma} (Mamba: exponent clamped at 0), beta.
-template <bool DELTA>
-NATSL_DEVICE void stage_scalars(const LinBwdParams& p, const int lane, const size_t row0, const int nvalid, const int h,
-                                float* gam, float* eg, float* ek, float* bet) {
-  const bool ok = lane < nvalid;
-  const size_t gi = (row0 + lane) * p.H + h;
-  float x = ok ? p.g[gi] : 0.f;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const float y = __shfl_up(x, d);
-    if (lane >= d) x += y;
-  }
-  const float gl = __shfl(x, 63);
-  float dk = gl - x;
-  if (!DELTA) dk = fminf(dk, 0.f);
-  gam[lane] = x;
-  eg[lane] = __expf(x);
-  ek[lane] = __expf(dk);
-  if (DELTA) bet[lane] = ok ? bf16_to_f32(p.beta[gi]) : 0.f;
+// {M[rowA + j][c0 + x] : j < 4} and {M[rowB + j][c0 + x] : j < 4} for lane x of a 16-lane group, M row-major in LDS with
+// `pitch` elements per row: the transposed operand of a 16x16x32 matrix instruction (x = the operand's row or column,
+// rowA.. and rowB.. = the lane group's eight contraction slots).
+NATSL_DEVICE bf16x8 tr_operand(const bf16_t* base, const int pitch, const int rowA, const int rowB, const int c0, const int x16) {
+  const int off = (x16 >> 2) * pitch + c0 + 4 * (x16 & 3);
+  return join4(lds_tr4(base + rowA * pitch + off), lds_tr4(base + rowB * pitch + off));
 }
 
-// q^, k^ of the chunk into LDS, row-major [64][DK + 8] and transposed [DK][TP]; rows past the end are zero.
+// q^, k^ rows of a chunk: what a thread fetches (row tid / 4, 16-byte pieces tid % 4 + 4 i) and, normalised, puts into LDS
 template <int DK>
-NATSL_DEVICE void stage_qk(const LinBwdParams& p, const int tid, const size_t row0, const int nvalid, const int h, const bool l2,
-                           bf16_t* Qn, bf16_t* Kn, bf16_t* QT, bf16_t* KT, float* rq, float* rk) {
-  constexpr int KP = DK + 8, KL = DK / 32;
+struct QkRegs {
+  u32x4 a[DK / 32], b[DK / 32];
+};
+
+template <int DK>
+NATSL_DEVICE void load_qk(const LinBwdParams& p, const int tid, const size_t row0, const int nvalid, const int h, QkRegs<DK>& r) {
   const int row = tid >> 2, sub = tid & 3;
   const bool ok = row < nvalid;
   const size_t off = ((row0 + row) * p.H + h) * DK;
   const u32x4 z = {0u, 0u, 0u, 0u};
-  u32x4 a[KL], b[KL];
+#pragma unroll
+  for (int i = 0; i < DK / 32; ++i) {
+    r.a[i] = ok ? *reinterpret_cast<const u32x4*>(p.q + off + (sub + 4 * i) * 8) : z;
+    r.b[i] = ok ? *reinterpret_cast<const u32x4*>(p.k + off + (sub + 4 * i) * 8) : z;
+  }
+}
+
+// rows past the end of the sequence arrive as zeros
+template <int DK>
+NATSL_DEVICE void store_qk(const QkRegs<DK>& r, const int tid, const bool l2, bf16_t* Qn, bf16_t* Kn, float* rq, float* rk) {
+  constexpr int KP = DK + 8, KL = DK / 32;
+  const int row = tid >> 2, sub = tid & 3;
   float sq = 0.f, sk = 0.f;
 #pragma unroll
   for (int i = 0; i < KL; ++i) {
-    a[i] = ok ? *reinterpret_cast<const u32x4*>(p.q + off + (sub + 4 * i) * 8) : z;
-    b[i] = ok ? *reinterpret_cast<const u32x4*>(p.k + off + (sub + 4 * i) * 8) : z;
     float fa[8], fb[8];
-    unpack8f(a[i], fa);
-    unpack8f(b[i], fb);
+    unpack8f(r.a[i], fa);
+    unpack8f(r.b[i], fb);
 #pragma unroll
     for (int e = 0; e < 8; ++e) { sq += fa[e] * fa[e]; sk += fb[e] * fb[e]; }
   }
@@ -158,8 +160,8 @@ NATSL_DEVICE void stage_qk(const LinBwdParams& p, const int tid, const size_t ro
   for (int i = 0; i < KL; ++i) {
     const int seg = sub + 4 * i;
     float fa[8], fb[8];
-    unpack8f(a[i], fa);
-    unpack8f(b[i], fb);
+    unpack8f(r.a[i], fa);
+    unpack8f(r.b[i], fb);
     u32x4 wa, wb;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -168,24 +170,46 @@ NATSL_DEVICE void stage_qk(const LinBwdParams& p, const int tid, const size_t ro
     }
     *reinterpret_cast<u32x4*>(Qn + row * KP + seg * 8) = wa;
     *reinterpret_cast<u32x4*>(Kn + row * KP + seg * 8) = wb;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      QT[(seg * 8 + e) * TP + row] = (bf16_t)((wa[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-      KT[(seg * 8 + e) * TP + row] = (bf16_t)((wb[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-    }
   }
 }
 
-// 64 rows x 64 columns of a token-major [tokens][H][V] tensor into LDS [64][TP]; rows past the end are zero.
-NATSL_DEVICE void stage_tokens64(const bf16_t* src, const int tid, const size_t row0, const int nvalid, const int H, const int V,
-                                 const int h, const int vcol0, bf16_t* dst) {
+// 64 rows x 64 columns of a token-major [tokens][H][V] tensor: a thread's two 16-byte pieces (rows past the end: zeros)
+NATSL_DEVICE void load_tokens64(const bf16_t* src, const int tid, const size_t row0, const int nvalid, const int H, const int V,
+                                const int h, const int vcol0, u32x4* w) {
   const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int pc = tid + 256 * it, row = pc >> 3, seg = pc & 7;
-    const u32x4 w = row < nvalid ? *reinterpret_cast<const u32x4*>(src + ((row0 + row) * H + h) * V + vcol0 + seg * 8) : z;
-    *reinterpret_cast<u32x4*>(dst + row * TP + seg * 8) = w;
+    w[it] = row < nvalid ? *reinterpret_cast<const u32x4*>(src + ((row0 + row) * H + h) * V + vcol0 + seg * 8) : z;
   }
+}
+NATSL_DEVICE void store_tokens64(const u32x4* w, const int tid, bf16_t* dst) {
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int pc = tid + 256 * it, row = pc >> 3, seg = pc & 7;
+    *reinterpret_cast<u32x4*>(dst + row * TP + seg * 8) = w[it];
+  }
+}
+
+// The chunk's scalars from g (and beta) of the wave's lanes = tokens: gamma (inclusive cumsum of g), e^gamma, e^{G - gamma}
+// (Mamba: exponent clamped at 0), scale e^gamma, beta.  Tokens past the end carry g = 0, beta = 0.
+template <bool DELTA>
+NATSL_DEVICE void store_scalars(const int lane, float x, const float b, const float scale, float* gam, float* eg, float* ek, float* sqv,
+                                float* bet) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const float y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  const float gl = __shfl(x, 63);
+  float dk = gl - x;
+  if (!DELTA) dk = fminf(dk, 0.f);
+  const float e = __expf(x);
+  gam[lane] = x;
+  eg[lane] = e;
+  ek[lane] = __expf(dk);
+  sqv[lane] = scale * e;
+  if (DELTA) bet[lane] = b;
 }
 
 // =============================================================================================
@@ -194,9 +218,9 @@ NATSL_DEVICE void stage_tokens64(const bf16_t* src, const int tid, const size_t 
 template <int DK>
 struct BwdScanLds {
   static constexpr int KP = DK + 8;
-  static constexpr int QN = 0, KN = QN + CB * KP, QT = KN + CB * KP, KT = QT + DK * TP, DO = KT + DK * TP, TT = DO + CB * TP;
-  static constexpr int VN = TT + CB * TP;
-  static constexpr int ELEMS = VN + CB * TP;
+  // q^, k^ [64][KP]; dO (later dX) and v_new [64][TP]; TmB as stored (eight 1 KiB operands); P^T as six 1 KiB operands
+  static constexpr int QN = 0, KN = QN + CB * KP, DO = KN + CB * KP, VN = DO + CB * TP, TM = VN + CB * TP, PT = TM + 8 * 512;
+  static constexpr int ELEMS = PT + 6 * 512;
   static constexpr int FL = ELEMS * 2;            // byte offset of the float area
   static constexpr int TOTAL = FL + 7 * CB * 4;
 };
@@ -209,11 +233,10 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
   bf16_t* const sm = reinterpret_cast<bf16_t*>(smem);
   bf16_t* const Qn = sm + L::QN;
   bf16_t* const Kn = sm + L::KN;
-  bf16_t* const QT = sm + L::QT;
-  bf16_t* const KT = sm + L::KT;
   bf16_t* const DOs = sm + L::DO;
-  bf16_t* const TT = sm + L::TT;
   bf16_t* const VNs = sm + L::VN;
+  bf16_t* const TmS = sm + L::TM;
+  bf16_t* const PTs = sm + L::PT;
   float* const fl = reinterpret_cast<float*>(smem + L::FL);
   float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *sqv = fl + 6 * CB;
 
@@ -230,10 +253,6 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
   const bool l2 = DELTA && (p.flags & NATSL_QK_L2NORM) != 0;
   const int hn = h / (p.H / p.HN);
 
-  // TmB^T: the part above the stored operands stays zero
-  if (DELTA)
-    for (int i = tid; i < CB * TP; i += 256) TT[i] = 0;
-
   f32x4 dS[KT16], pend[KT16];
 #pragma unroll
   for (int m = 0; m < KT16; ++m)
@@ -243,43 +262,78 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
       pend[m][r] = 0.f;
     }
 
+  // ---- what a thread fetches for a chunk; requested one chunk ahead, under the state-gradient update of the chunk before ----
+  QkRegs<DK> qk;
+  u32x4 do_r[2], vn_r[2], tm_r[2];
+  u32x2 s_r[KT16];      // the chunk's entering state, this lane's column: for <dS', S>
+  // (scalars are fetched raw and interpreted when the chunk's turn comes: anything computed from them here would make
+  // the wave wait for all of the requests)
+  float g_r = 0.f, gs_r = 0.f;
+  unsigned beta_r = 0u, ty_r = 0u;
+  auto fetch = [&](const int cc) __attribute__((always_inline)) {
+    const int t0 = cc * CB, nvalid = min(CB, len - t0);
+    const size_t row0 = (size_t)bos + t0;
+    load_qk<DK>(p, tid, row0, nvalid, h, qk);
+    load_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, vcol0, do_r);
+    if (DELTA) {
+      load_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, vcol0, vn_r);
+      // TmB: a straight copy of the six stored operands (operand (t, s) at 2 t + s; 0, 2, 4..7 exist)
+      const bf16_t* tm = p.ws_tm + ((size_t)(chunk_off + cc) * p.H + h) * (CB * CB);
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+        const int pc = tid + 256 * it;
+        if (pc < 6 * 64) {
+          const int oi = pc >> 6, o = oi < 2 ? 2 * oi : oi + 2;
+          tm_r[it] = *reinterpret_cast<const u32x4*>(tm + o * 512 + (pc & 63) * 8);
+        }
+      }
+    }
+    const size_t so = (((size_t)(chunk_off + cc) * p.H + h) * p.V + col) * DK + 4 * g4;
+#pragma unroll
+    for (int m = 0; m < KT16; ++m) s_r[m] = *reinterpret_cast<const u32x2*>(p.s_all + so + 16 * m);
+    if (wave == 0) {
+      const size_t gi = (row0 + min(lane, nvalid - 1)) * p.H + h;
+      g_r = p.g[gi];
+      if (DELTA) beta_r = p.beta[gi];
+    }
+    const int blk = t0 / p.block;
+    const size_t ti = ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1;
+    if (p.types_dtype == NATSL_F32) ty_r = reinterpret_cast<const unsigned*>(p.types)[ti];
+    else ty_r = reinterpret_cast<const bf16_t*>(p.types)[ti];
+    gs_r = p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h];
+  };
+  fetch(NT - 1);
+
   for (int c = NT - 1; c >= 0; --c) {
     const int t0 = c * CB, nvalid = min(CB, len - t0);
     const size_t row0 = (size_t)bos + t0;
     __syncthreads();   // every wave is done with the previous chunk's tiles
-    if (wave == 0) stage_scalars<DELTA>(p, lane, row0, nvalid, h, gam, eg, ek, bet);
-    stage_qk<DK>(p, tid, row0, nvalid, h, l2, Qn, Kn, QT, KT, rq, rk);
-    stage_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, vcol0, DOs);
+    if (wave == 0)
+      store_scalars<DELTA>(lane, lane < nvalid ? g_r : 0.f, lane < nvalid ? bf16_to_f32((bf16_t)beta_r) : 0.f, p.scale, gam, eg, ek, sqv, bet);
+    store_qk<DK>(qk, tid, l2, Qn, Kn, rq, rk);
+    store_tokens64(do_r, tid, DOs);
     if (DELTA) {
-      stage_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, vcol0, VNs);
-      // TmB^T [j][i] from the six stored operands: operand (t, s) at 2t + s, scan-lane (x, g) at (16 g + x) * 8, slot e stands
-      // for column 32 s + 16 (e / 4) + 4 g + e % 4 of row 16 t + x
-      const bf16_t* tm = p.ws_tm + ((size_t)(chunk_off + c) * p.H + h) * (CB * CB);
-      for (int pc = tid; pc < 6 * 64; pc += 256) {
-        const int oi = pc >> 6, ln = pc & 63, o = oi < 2 ? 2 * oi : oi + 2, t = o >> 1, s = o & 1, x = ln & 15, gg = ln >> 4;
-        const u32x4 w = *reinterpret_cast<const u32x4*>(tm + o * 512 + ln * 8);
+      store_tokens64(vn_r, tid, VNs);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int j = 32 * s + 16 * (e >> 2) + 4 * gg + (e & 3);
-          TT[j * TP + 16 * t + x] = (bf16_t)((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+      for (int it = 0; it < 2; ++it) {
+        const int pc = tid + 256 * it;
+        if (pc < 6 * 64) {
+          const int oi = pc >> 6, o = oi < 2 ? 2 * oi : oi + 2;
+          *reinterpret_cast<u32x4*>(TmS + o * 512 + (pc & 63) * 8) = tm_r[it];
         }
       }
     }
-    __syncthreads();
-    if (tid < CB) sqv[tid] = p.scale * eg[tid];
-    // (sqv is read below only after the state-gradient products; the barrier in between is the one after Y2)
-
-    // ---- dS' of this chunk goes out as it arrived; a rolled-back block's leaves the chain here --------------------------
+    const bool lin = rintf(__uint_as_float(p.types_dtype == NATSL_F32 ? ty_r : ty_r << 16)) == 1.0f;
+    const float f_blk = decay ? __expf(gs_r) : 1.f;
+    float sd = 0.f;
     {
-      const size_t so = (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 4 * g4;
-      bf16_t* dso = p.ds_all + so;
-      const bf16_t* sin = p.s_all + so;
-      float sd = 0.f;
+      // dS' of this chunk goes out as it arrived, and <dS', S> with it
+      bf16_t* dso = p.ds_all + (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 4 * g4;
 #pragma unroll
       for (int m = 0; m < KT16; ++m) {
         u32x2 w = {pack_bf16x2(dS[m][0], dS[m][1]), pack_bf16x2(dS[m][2], dS[m][3])};
         *reinterpret_cast<u32x2*>(dso + 16 * m) = w;
-        const u32x2 sw = *reinterpret_cast<const u32x2*>(sin + 16 * m);
+        const u32x2 sw = s_r[m];
         sd += dS[m][0] * __uint_as_float(sw[0] << 16) + dS[m][1] * __uint_as_float(sw[0] & 0xffff0000u) +
               dS[m][2] * __uint_as_float(sw[1] << 16) + dS[m][3] * __uint_as_float(sw[1] & 0xffff0000u);
       }
@@ -287,11 +341,45 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
       for (int d = 1; d < 64; d <<= 1) sd += __shfl_xor(sd, d);
       if (lane == 0) p.sdot_parts[((size_t)(chunk_off + c) * p.H + h) * (p.V / 16) + 4 * split + wave] = sd;
     }
-    const int blk = t0 / p.block;
+    __syncthreads();   // the tiles are there
+
+    // ---- P^T as operands, once per workgroup: Z = q^ k^^T leaves lane (x, g) with key 16 tj + x against queries
+    //      16 ti + 4 g + r, the four slots this lane holds of operand (tj, ti / 2), half ti % 2.  Operand (tj, s2) at index
+    //      tj < 2 ? 2 tj + s2 : 2 + tj; waves 0..3 form {(0,0), (1,0)}, {(0,1), (3,1)}, {(1,1)}, {(2,1)}: 3, 3, 2, 2 tiles. ----
+    if (intra) {
+      auto make_operand = [&](const int tj, const int s2) __attribute__((always_inline)) {
+        const float gj = gam[16 * tj + x16];
+        f32x4 Z[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const int ti = 2 * s2 + hf;
+          Z[hf] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          if (ti >= tj) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+              const bf16x8 a = *reinterpret_cast<const bf16x8*>(Qn + (16 * ti + x16) * KP + 32 * s + 8 * g4);
+              const bf16x8 b = *reinterpret_cast<const bf16x8*>(Kn + (16 * tj + x16) * KP + 32 * s + 8 * g4);
+              Z[hf] = mfma16(a, b, Z[hf]);
+            }
+            const f32x4 gi = *reinterpret_cast<const f32x4*>(gam + 16 * ti + 4 * g4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const bool vis = ti > tj || 4 * g4 + r >= x16;
+              Z[hf][r] = vis ? Z[hf][r] * p.scale * __expf(gi[r] - gj) : 0.f;
+            }
+          }
+        }
+        *reinterpret_cast<bf16x8*>(PTs + (tj < 2 ? 2 * tj + s2 : 2 + tj) * 512 + lane * 8) = pack8(Z[0], Z[1]);
+      };
+      if (wave == 0) { make_operand(0, 0); make_operand(1, 0); }
+      else if (wave == 1) { make_operand(0, 1); make_operand(3, 1); }
+      else if (wave == 2) make_operand(1, 1);
+      else make_operand(2, 1);
+    }
+    // ---- a rolled-back block's dS' leaves the chain here ---------------------------------------------------------------
     const bool last = ((c + 1) % per == 0) || (c == NT - 1);
     if (last) {
-      const bool lin = lin_type_b(p.types, p.types_dtype, ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1);
-      const float f = lin ? 0.f : (decay ? __expf(p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h]) : 1.f);
+      const float f = lin ? 0.f : f_blk;
 #pragma unroll
       for (int m = 0; m < KT16; ++m)
 #pragma unroll
@@ -302,7 +390,7 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
     }
     const float dec = __expf(gam[CB - 1]);
 
-    // ---- Y1 = K~ dS' ----------------------------------------------------------------------------------------------------
+    // ---- Y1 = K~ dS' (the state gradient as two operands: truncated value and remainder) --------------------------------
     f32x4 DV[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) DV[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -335,37 +423,20 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) DOc[t][r] = bf16_to_f32(DOs[(16 * t + 4 * g4 + r) * TP + 16 * wave + x16]);
-    // ---- Y2 = P^T dO: P^T's operands are formed here; Z = q^ k^^T leaves lane (x, g) with key 16 tj + x against queries
-    //      16 ti + 4 g + r, the four slots this lane holds of operand (tj, ti / 2), half ti % 2 ------------------------------
+    __syncthreads();   // P^T
+    // ---- Y2 = P^T dO ----------------------------------------------------------------------------------------------------
     if (intra) {
       const bf16x8 DOB[2] = {pack8(DOc[0], DOc[1]), pack8(DOc[2], DOc[3])};
 #pragma unroll
-      for (int tj = 0; tj < 4; ++tj) {
-        const float gj = gam[16 * tj + x16];
-        f32x4 Z[4];
+      for (int tj = 0; tj < 4; ++tj)
 #pragma unroll
-        for (int ti = 0; ti < 4; ++ti) {
-          Z[ti] = (f32x4){0.f, 0.f, 0.f, 0.f};
-          if (ti >= tj) {
-#pragma unroll
-            for (int s = 0; s < KS; ++s) {
-              const bf16x8 a = *reinterpret_cast<const bf16x8*>(Qn + (16 * ti + x16) * KP + 32 * s + 8 * g4);
-              const bf16x8 b = *reinterpret_cast<const bf16x8*>(Kn + (16 * tj + x16) * KP + 32 * s + 8 * g4);
-              Z[ti] = mfma16(a, b, Z[ti]);
-            }
-            const f32x4 gi = *reinterpret_cast<const f32x4*>(gam + 16 * ti + 4 * g4);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const bool vis = ti > tj || 4 * g4 + r >= x16;
-              Z[ti][r] = vis ? Z[ti][r] * p.scale * __expf(gi[r] - gj) : 0.f;
-            }
-          }
-        }
-        if (tj < 2) DV[tj] = mfma16(pack8(Z[0], Z[1]), DOB[0], DV[tj]);
-        DV[tj] = mfma16(pack8(Z[2], Z[3]), DOB[1], DV[tj]);
-      }
+        for (int s2 = 0; s2 < 2; ++s2)
+          if (tj < 2 || s2 == 1)
+            DV[tj] = mfma16(*reinterpret_cast<const bf16x8*>(PTs + (tj < 2 ? 2 * tj + s2 : 2 + tj) * 512 + lane * 8), DOB[s2], DV[tj]);
     }
-    // ---- dX = TmB^T dv_new ----------------------------------------------------------------------------------------------
+    // ---- dX = TmB^T dv_new (dv_new as two operands).  Element (row i, column cc) of TmB sits in stored operand
+    //      (i / 16, cc / 32), lane slot 16 ((cc % 16) / 4) + i % 16, element 4 ((cc % 32) / 16) + cc % 4: four consecutive
+    //      columns are contiguous, so the transposing read applies with "rows" = lane slots ------------------------------
     f32x4 DX[4];
     if (DELTA) {
       const bf16x8 DVB[2] = {pack8_trunc(DV[0], DV[1]), pack8_trunc(DV[2], DV[3])};
@@ -376,8 +447,11 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           if (2 * s2 + 1 >= tj) {
-            const bf16_t* tr = TT + (16 * tj + x16) * TP + 32 * s2 + 4 * g4;
-            const bf16x8 a = join_u2(*reinterpret_cast<const u32x2*>(tr), *reinterpret_cast<const u32x2*>(tr + 16));
+            // rows i = 32 s2 + 16 hf + 4 g + j of column 16 tj + x: lane l names slot 16 (l % 4) + 4 g + l / 4 of operand
+            // (2 s2 + hf, tj / 2), elements 4 (tj % 2) ..
+            const int slot = 16 * (x16 & 3) + 4 * g4 + (x16 >> 2);
+            const bf16_t* lo = TmS + (2 * (2 * s2) + (tj >> 1)) * 512 + slot * 8 + 4 * (tj & 1);
+            const bf16x8 a = join4(lds_tr4(lo), lds_tr4(lo + 2 * 512));
             DX[tj] = mfma16(a, DVR[s2], DX[tj]);
             DX[tj] = mfma16(a, DVB[s2], DX[tj]);
           }
@@ -387,22 +461,42 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
 #pragma unroll
       for (int t = 0; t < 4; ++t) DX[t] = DV[t];
     }
-    // dv = dX; for dbeta_i = <dX_i, v_new_i> / beta_i^2, this wave's 16 columns of the inner product (dX still in fp32)
+    // dv = dX, through this wave's 16 columns of the dO tile (read above, by this wave only) so that it leaves in whole rows
+    {
+      float pb[16];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int tok = 16 * t + 4 * g4 + r;
-        if (tok < nvalid) p.dv[((row0 + tok) * p.H + h) * p.V + col] = f32_to_bf16(DX[t][r]);
-        if (DELTA) {
-          float pb = DX[t][r] * bf16_to_f32(VNs[tok * TP + 16 * wave + x16]);
-#pragma unroll
-          for (int d = 1; d < 16; d <<= 1) pb += __shfl_xor(pb, d);
-          if (x16 == 0 && tok < nvalid) p.dbeta_parts[((row0 + tok) * p.H + h) * (p.V / 16) + 4 * split + wave] = pb;
+        for (int r = 0; r < 4; ++r) {
+          const int tok = 16 * t + 4 * g4 + r;
+          DOs[tok * TP + 16 * wave + x16] = f32_to_bf16(DX[t][r]);
+          if (DELTA) pb[4 * t + r] = DX[t][r] * bf16_to_f32(VNs[tok * TP + 16 * wave + x16]);
         }
+      if (DELTA) {
+        // for dbeta_i = <dX_i, v_new_i> / beta_i^2: this wave's 16 columns of the inner product (dX still in fp32).  Sixteen
+        // sums over sixteen lanes as a butterfly: in every step a lane hands half of its values to its partner and adds
+        // the partner's other half to the rest; lane x ends up with sum number x.
+#pragma unroll
+        for (int d = 8; d >= 1; d >>= 1) {
+          const bool up = (x16 & d) != 0;
+#pragma unroll
+          for (int i = 0; i < d; ++i) {
+            const float send = up ? pb[i] : pb[i + d], keep = up ? pb[i + d] : pb[i];
+            pb[i] = keep + __shfl_xor(send, d);
+          }
+        }
+        const int tok = 16 * (x16 >> 2) + 4 * g4 + (x16 & 3);
+        if (tok < nvalid) p.dbeta_parts[((row0 + tok) * p.H + h) * (p.V / 16) + 4 * split + wave] = pb[0];
       }
-    __syncthreads();   // sqv
-    // ---- dS = e^G dS' + Q~^T dO - W^T dX --------------------------------------------------------------------------------
+    }
+    __syncthreads();   // the dX tile
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int pc = tid + 256 * it, row = pc >> 3, seg = pc & 7;
+      if (row < nvalid)
+        *reinterpret_cast<u32x4*>(p.dv + ((row0 + row) * p.H + h) * p.V + vcol0 + seg * 8) = *reinterpret_cast<const u32x4*>(DOs + row * TP + seg * 8);
+    }
+    // ---- dS = e^G dS' + Q~^T dO - W^T dX, with the next chunk's requests in flight ------------------------------------------
     {
       f32x4 A1[4], A2[4];
 #pragma unroll
@@ -417,18 +511,16 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
       }
       const bf16x8 B1[2] = {pack8(A1[0], A1[1]), pack8(A1[2], A1[3])};
       const bf16x8 B2[2] = {pack8(A2[0], A2[1]), pack8(A2[2], A2[3])};
+      if (c > 0) fetch(c - 1);
 #pragma unroll
       for (int m = 0; m < KT16; ++m) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) dS[m][r] *= dec;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          const bf16_t* qr = QT + (16 * m + x16) * TP + 32 * s2 + 4 * g4;
-          dS[m] = mfma16(join_u2(*reinterpret_cast<const u32x2*>(qr), *reinterpret_cast<const u32x2*>(qr + 16)), B1[s2], dS[m]);
-          if (DELTA) {
-            const bf16_t* kr = KT + (16 * m + x16) * TP + 32 * s2 + 4 * g4;
-            dS[m] = mfma16(join_u2(*reinterpret_cast<const u32x2*>(kr), *reinterpret_cast<const u32x2*>(kr + 16)), B2[s2], dS[m]);
-          }
+          // rows = K index 16 m + x, slots = tokens 32 s2 + 4 g + j and 32 s2 + 16 + 4 g + j
+          dS[m] = mfma16(tr_operand(Qn, KP, 32 * s2 + 4 * g4, 32 * s2 + 16 + 4 * g4, 16 * m, x16), B1[s2], dS[m]);
+          if (DELTA) dS[m] = mfma16(tr_operand(Kn, KP, 32 * s2 + 4 * g4, 32 * s2 + 16 + 4 * g4, 16 * m, x16), B2[s2], dS[m]);
         }
       }
     }
@@ -456,25 +548,25 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
 template <int DK>
 struct BwdChunkLds {
   static constexpr int KP = DK + 8;
-  // phase 1 (the products that contract over V, one 64-column slice at a time)
-  static constexpr int DO = 0, DX = DO + CB * TP, VN = DX + CB * TP, ST = VN + CB * TP, DST = ST + DK * TP, P1 = DST + DK * TP;
-  // phase 2 (the products that contract over tokens)
-  static constexpr int QN = 0, KN = QN + CB * KP, QT = KN + CB * KP, KT = QT + DK * TP, GN = KT + DK * TP, GT = GN + CB * TP,
-                       HS = GT + CB * TP, P2 = HS + CB * TP;
+  // phase 1 (the products that contract over V, one 64-column slice at a time): dO, dX, v_new [64][TP]; S, dS' [64 columns][KP]
+  static constexpr int DO = 0, DX = DO + CB * TP, VN = DX + CB * TP, SN = VN + CB * TP, DSN = SN + CB * KP, P1 = DSN + CB * KP;
+  // phase 2 (the products that contract over tokens): q^, k^ [64][KP]; the weight tiles Gm, Gm^T, Hm + Hm^T [64][TP]
+  static constexpr int QN = 0, KN = QN + CB * KP, GN = KN + CB * KP, GT = GN + CB * TP, HS = GT + CB * TP, P2 = HS + CB * TP;
   static constexpr int ELEMS = P1 > P2 ? P1 : P2;
   static constexpr int FL = ELEMS * 2;
-  static constexpr int TOTAL = FL + (7 * CB + 8) * 4;
+  static constexpr int TOTAL = FL + (8 * CB + 8) * 4;
 };
 
 template <int DK, bool DELTA>
-__global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParams p) {
+__global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kernel(const LinBwdParams p) {
   using L = BwdChunkLds<DK>;
   constexpr int KP = L::KP, KT16 = DK / 16, KS = DK / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* const sm = reinterpret_cast<bf16_t*>(smem);
   float* const fl = reinterpret_cast<float*>(smem + L::FL);
-  float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *dgam = fl + 6 * CB;
-  float* red = fl + 7 * CB;   // [0] <dS', S>, [1] sum of the gate terms, [2] <dS', S_blockstart>
+  float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *dgam = fl + 6 * CB,
+        *sqv = fl + 7 * CB;
+  float* red = fl + 8 * CB;   // [0] <dS', S>, [1] sum of the gate terms, [2] <dS', S_blockstart>
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
   const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
@@ -492,15 +584,22 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
   const bool want_rb = rolled && decay;
   const int c_first = (c / per) * per;
 
-  if (wave == 0) stage_scalars<DELTA>(p, lane, row0, nvalid, h, gam, eg, ek, bet);
+  if (wave == 0) {
+    const bool ok = lane < nvalid;
+    const size_t gi = (row0 + lane) * p.H + h;
+    store_scalars<DELTA>(lane, ok ? p.g[gi] : 0.f, DELTA && ok ? bf16_to_f32(p.beta[gi]) : 0.f, p.scale, gam, eg, ek, sqv, bet);
+  }
   if (tid < 8) red[tid] = 0.f;
+  // q^, k^ are requested now and put into LDS when phase 1 is done with it
+  QkRegs<DK> qk;
+  load_qk<DK>(p, tid, row0, nvalid, h, qk);
 
   // ---- phase 1 -------------------------------------------------------------------------------------------------------
   bf16_t* const DOs = sm + L::DO;
   bf16_t* const DXs = sm + L::DX;
   bf16_t* const VNs = sm + L::VN;
-  bf16_t* const ST = sm + L::ST;
-  bf16_t* const DST = sm + L::DST;
+  bf16_t* const Sn = sm + L::SN;
+  bf16_t* const DSn = sm + L::DSN;
   f32x4 Nm[4], Mm[4], DQ2[KT16], DW[KT16], DK3[KT16];
 #pragma unroll
   for (int t = 0; t < 4; ++t) { Nm[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; Mm[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
@@ -514,27 +613,26 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
   const bf16_t* ds_src = p.ds_all + unit * p.V * DK;
   const bf16_t* sf_src = p.s_all + ((size_t)(n * p.nt + c_first) * p.H + h) * p.V * DK;
   for (int vs = 0; vs < p.V / 64; ++vs) {
-    __syncthreads();
-    stage_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, 64 * vs, DOs);
-    stage_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, 64 * vs, VNs);
-    if (DELTA) stage_tokens64(p.dv, tid, row0, nvalid, p.H, p.V, h, 64 * vs, DXs);
-    // the state and its gradient, [V][K] in memory, as [K][64 columns] in LDS
+    u32x4 w_do[2], w_vn[2], w_dx[2];
+    load_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, 64 * vs, w_do);
+    load_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, 64 * vs, w_vn);
+    if (DELTA) load_tokens64(p.dv, tid, row0, nvalid, p.H, p.V, h, 64 * vs, w_dx);
+    __syncthreads();   // the previous slice's tiles are dead
+    store_tokens64(w_do, tid, DOs);
+    store_tokens64(w_vn, tid, VNs);
+    if (DELTA) store_tokens64(w_dx, tid, DXs);
+    // the state and its gradient as they lie in memory: [64 columns][K]
     for (int pc = tid; pc < 64 * (DK / 8); pc += 256) {
-      const int v = pc & 63, seg = pc >> 6;
+      const int v = pc / (DK / 8), seg = pc % (DK / 8);
       const size_t off = (size_t)(64 * vs + v) * DK + seg * 8;
       const u32x4 ws = *reinterpret_cast<const u32x4*>(s_src + off);
       const u32x4 wd = *reinterpret_cast<const u32x4*>(ds_src + off);
-      float fs[8], fd[8];
-      unpack8f(ws, fs);
-      unpack8f(wd, fd);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        ST[(seg * 8 + e) * TP + v] = (bf16_t)((ws[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-        DST[(seg * 8 + e) * TP + v] = (bf16_t)((wd[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-      }
+      *reinterpret_cast<u32x4*>(Sn + v * KP + seg * 8) = ws;
+      *reinterpret_cast<u32x4*>(DSn + v * KP + seg * 8) = wd;
       if (want_rb) {
-        float ff[8];
+        float ff[8], fd[8];
         unpack8f(*reinterpret_cast<const u32x4*>(sf_src + off), ff);
+        unpack8f(wd, fd);
 #pragma unroll
         for (int e = 0; e < 8; ++e) srb += ff[e] * fd[e];
       }
@@ -554,8 +652,9 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
       }
 #pragma unroll
       for (int m = 0; m < KT16; ++m) {
-        const bf16x8 bs = *reinterpret_cast<const bf16x8*>(ST + (16 * m + x16) * TP + 32 * s + 8 * g4);
-        const bf16x8 bd = *reinterpret_cast<const bf16x8*>(DST + (16 * m + x16) * TP + 32 * s + 8 * g4);
+        // columns = K index 16 m + x, slots = state columns 32 s + 8 g + j
+        const bf16x8 bs = tr_operand(Sn, KP, 32 * s + 8 * g4, 32 * s + 8 * g4 + 4, 16 * m, x16);
+        const bf16x8 bd = tr_operand(DSn, KP, 32 * s + 8 * g4, 32 * s + 8 * g4 + 4, 16 * m, x16);
         DQ2[m] = mfma16(a_do, bs, DQ2[m]);
         if (DELTA) DW[m] = mfma16(a_dx, bs, DW[m]);
         DK3[m] = mfma16(a_vn, bd, DK3[m]);
@@ -576,15 +675,13 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
   // ---- phase 2 -------------------------------------------------------------------------------------------------------
   bf16_t* const Qn = sm + L::QN;
   bf16_t* const Kn = sm + L::KN;
-  bf16_t* const QT = sm + L::QT;
-  bf16_t* const KT = sm + L::KT;
   bf16_t* const Gn = sm + L::GN;
   bf16_t* const GT = sm + L::GT;
   bf16_t* const Hs = sm + L::HS;
   __syncthreads();   // phase 1's tiles are dead
-  stage_qk<DK>(p, tid, row0, nvalid, h, l2, Qn, Kn, QT, KT, rq, rk);
+  store_qk<DK>(qk, tid, l2, Qn, Kn, rq, rk);
   if (DELTA)
-    for (int i = tid; i < CB * TP; i += 256) Hs[i] = 0;
+    for (int i = tid; i < CB * TP / 8; i += 256) *reinterpret_cast<u32x4*>(Hs + 8 * i) = (u32x4){0u, 0u, 0u, 0u};
   __syncthreads();
 
   // this lane's rows i = 16 wave + 4 g + r; its column in tile tj is 16 tj + x
@@ -666,8 +763,9 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
     }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const bf16x8 bk = *reinterpret_cast<const bf16x8*>(KT + (16 * m + x16) * TP + 32 * s + 8 * g4);
-      const bf16x8 bq = *reinterpret_cast<const bf16x8*>(QT + (16 * m + x16) * TP + 32 * s + 8 * g4);
+      // columns = K index 16 m + x, slots = tokens 32 s + 8 g + j
+      const bf16x8 bk = tr_operand(Kn, KP, 32 * s + 8 * g4, 32 * s + 8 * g4 + 4, 16 * m, x16);
+      const bf16x8 bq = tr_operand(Qn, KP, 32 * s + 8 * g4, 32 * s + 8 * g4 + 4, 16 * m, x16);
       dq = mfma16(ga[s], bk, dq);
       dk = mfma16(gta[s], bq, dk);
       if (DELTA) dk = mfma16(ha[s], bk, dk);
@@ -700,7 +798,7 @@ __global__ __launch_bounds__(256) void linear_bwd_chunk_kernel(const LinBwdParam
   }
   __syncthreads();   // every wave is done with q^, k^ and the weight tiles; dgam and red are complete
 
-  // ---- the row normalisation's backward, then out through LDS (rows of KP elements in the space of q^, k^ tiles) --------
+  // ---- the row normalisation's backward, then out through LDS (in place of the q^, k^ tiles) ---------------------------
   {
     const f32x4 rq4 = *reinterpret_cast<const f32x4*>(rq + 16 * wave + 4 * g4);
     const f32x4 rk4 = *reinterpret_cast<const f32x4*>(rk + 16 * wave + 4 * g4);
