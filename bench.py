@@ -41,6 +41,7 @@ BACKWARD_WORKLOADS = {
 LINEAR_BACKWARD_WORKLOADS = {
     "gdn_bwd_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
     "gdn_bwd_B8_T4096_H6_K128_V256_p25": dict(B=8, T=4096, H=6, K=128, V=256, p_attn=0.25, block=64),
+    "mamba_bwd_B4_T8192_H32_N128_d64_p25": dict(B=4, T=8192, H=32, K=128, V=64, p_attn=0.25, block=256, kind="mamba"),
 }
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
@@ -334,7 +335,12 @@ def bench_linear_bwd(args):
     ty, nb = nats_util.hard_select(d["logits"], force_last_block=True)
     do = torch.randn(d["v"].shape, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).bfloat16()
 
+    is_mamba = w.get("kind") == "mamba"
+
     def step():
+        if is_mamba:
+            return linear_chunk_backward_hip('mamba', d["q"], d["k"], d["v_l"], d["g"], None, None, ty, 1.0, w["block"], True, False, True, do,
+                                             None, False)
         return linear_chunk_backward_hip('gdn', d["q"], d["k"], d["v"], d["g"], d["beta"], None, ty, w["K"] ** -0.5, w["block"], True, True,
                                          True, do, None, False)
     for _ in range(args.warmup):
@@ -346,12 +352,12 @@ def bench_linear_bwd(args):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     n_tok = w["B"] * w["T"] * w["H"]
-    nbytes = n_tok * (2 * (4 * w["K"] + 3 * w["V"]) + 4 * 2 + 2 * 2)     # q, k, dq, dk; v, do, dv; g, dg (f32); beta, dbeta
+    nbytes = n_tok * (2 * (4 * w["K"] + 3 * w["V"]) + 4 * 2 + (0 if is_mamba else 2 * 2))     # q, k, dq, dk; v, do, dv; g, dg (f32); beta, dbeta
     print(json.dumps(dict(
-        metric="GDN-branch backward tokens/sec bf16", value=w["B"] * w["T"] / (ms * 1e-3), unit="tokens/s",
+        metric=("Mamba2-SSD" if is_mamba else "GDN") + "-branch backward tokens/sec bf16", value=w["B"] * w["T"] / (ms * 1e-3), unit="tokens/s",
         n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak", vs_baseline=None,
         dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w),
-        roofline=dict(bound="hbm", kernel="linear_prep+linear_scan+linear_bwd_scan+linear_bwd_chunk", achieved=nbytes / (ms * 1e-3) / 1e9,
+        roofline=dict(bound="hbm", kernel=("mamba_scale" if is_mamba else "linear_prep") + "+linear_scan+linear_bwd_scan+linear_bwd_chunk", achieved=nbytes / (ms * 1e-3) / 1e9,
                       peak=PEAK_HBM_GBS, unit="GB/s", frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, traffic=None, algorithmic_bytes=nbytes,
                       note="whole step incl. the forward re-run and the host-side glue"))))
 

@@ -167,11 +167,11 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
                           size_t workspace_bytes, int dtype, const natsl_seq_row* seqs, int n_seqs,
                           int total_units, natsl_stream_t stream);
 
-/* Backward of the two chunked linear branches (delta_rule != 0: Gated DeltaNet, else Mamba2-style SSD), regular batches
- * (packed input: one call per sequence).  Call the forward entry first with chunk_states and (delta rule) chunk_v_new and
+/* Backward of the two chunked linear branches (delta_rule != 0: Gated DeltaNet, else Mamba2-style SSD); packed input as for the
+ * forward (B = 1, the sequence table, TN = all blocks; dht, dh0 then hold one state per sequence).  Call the forward entry first with chunk_states and (delta rule) chunk_v_new and
  * keep its workspace: this entry reads the triangular solves from it.  Inputs as for the forward, plus
  *   v_new [B*T][H][V] (Mamba: v itself), d_o [B*T][H][V] bf16, dht [B][H][K][V] f32 or NULL,
- *   g_block_sums [B][TN][H] f32 = sum of g over every selector block.
+ *   g_block_sums [B][TN][H] f32 = sum of g over every selector block (packed: flat over the sequences' blocks).
  * Outputs: dq, dk [B*T][H][K], dv [B*T][H][V] bf16; dg, dbeta (delta rule) [B*T][H] f32; dh0 [B][H][K][V] f32 or NULL;
  *   d_gate [chunks][H] f32 = derivative with respect to a gate on every chunk's state update (the selector's
  *   straight-through gradient for the linear operator, src/nats/ops/common/chunk_o.py:438-443, :487-492, before the sum over
@@ -188,7 +188,7 @@ int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void* k, const v
                            const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
                            float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
                            int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
-                           natsl_stream_t stream);
+                           const natsl_seq_row* seqs, int n_seqs, int total_chunks, natsl_stream_t stream);
 
 /* Layer tail: y = (rms(x1)*w1*xw[...,0] + rms(x2)*w2*xw[...,1]) * gate*sigmoid(gate) with
  * rms(x) = x*rsqrt(mean(x^2)+eps); x1, x2, gate, y [rows, D] and x_weights [rows, 2] in `dtype`,

@@ -111,28 +111,80 @@ def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, de
 
 
 def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                          dnats_for_invalid_blocks):
+                          dnats_for_invalid_blocks, seqs=None):
     """Gradients of the chunked linear branch: -> (dq, dk, dv, dg fp32, dbeta or None, dh0 or None, dnats fp32 [B,NB,HN]).
-    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None.  The HIP kernels (natsl_linear_chunk_bwd) where they are built
-    (K in 64/128/192, V a multiple of 64), else the torch formulation below."""
+    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None; seqs: packed sequences (B = 1) or None.  The HIP kernels
+    (natsl_linear_chunk_bwd) where they are built (K in 64/128/192, V a multiple of 64), else the torch formulation below,
+    one sequence at a time."""
     if q.shape[-1] in (64, 128, 192) and v.shape[-1] % 64 == 0:
         return linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                                         dnats_for_invalid_blocks)
-    return linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                                       dnats_for_invalid_blocks)
+                                         dnats_for_invalid_blocks, seqs)
+    if seqs is None:
+        return linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
+                                           dnats_for_invalid_blocks)
+    parts = []
+    for i in range(seqs.n_seqs):
+        a, b = seqs.cu_seqlens[i], seqs.cu_seqlens[i + 1]
+        na, nb = seqs.cu_seqlens_nats[i], seqs.cu_seqlens_nats[i + 1]
+        parts.append(linear_chunk_backward_torch(
+            kind, q[:, a:b], k[:, a:b], v[:, a:b], g[:, a:b], None if beta is None else beta[:, a:b],
+            None if h0 is None else h0[i:i + 1], types[:, na:nb], scale, block, decay, l2norm, intra, do[:, a:b],
+            None if dht is None else dht[i:i + 1], dnats_for_invalid_blocks))
+    cat = lambda j, dim: None if parts[0][j] is None else torch.cat([p[j] for p in parts], dim)
+    return cat(0, 1), cat(1, 1), cat(2, 1), cat(3, 1), cat(4, 1), cat(5, 0), cat(6, 1)
+
+
+_MAPS = {}
+
+
+def _block_maps(B, T, block, seqs, dev):
+    """Index tensors that tie tokens and chunks to selector blocks, flat over the sequences: for every block the first / one
+    past the last token and chunk, the index of its last chunk, and for every token its block."""
+    key = (B, T, block, None if seqs is None else tuple(seqs.cu_seqlens), str(dev))
+    m = _MAPS.get(key)
+    if m is not None:
+        return m
+    per = block // C
+    bounds = [(i * T, (i + 1) * T) for i in range(B)] if seqs is None else list(zip(seqs.cu_seqlens[:-1], seqs.cu_seqlens[1:]))
+    t0s, t1s, c0s, c1s, toks = [], [], [], [], []
+    coff, boff = 0, 0
+    for a, b in bounds:
+        n = b - a
+        nb, nc = -(-n // block), -(-n // C)
+        j = torch.arange(nb)
+        t0s.append(a + j * block)
+        t1s.append(torch.clamp(a + (j + 1) * block, max=b))
+        c0s.append(coff + j * per)
+        c1s.append(torch.clamp(coff + (j + 1) * per, max=coff + nc))
+        toks.append(boff + torch.arange(n) // block)
+        coff += nc
+        boff += nb
+    m = tuple(torch.cat(x).to(dev) for x in (t0s, t1s, c0s, c1s, toks))
+    if len(_MAPS) > 16:
+        _MAPS.clear()
+    _MAPS[key] = m
+    return m
+
+
+def _range_sums(x, first, end):
+    """Sums of x[first[j]:end[j]] along dim 0 for every j (fp64 running sums: the same result every time)."""
+    xt = x.double().t().contiguous()                      # [H, n]: the running sum along the contiguous dimension
+    cs = torch.cat([xt.new_zeros(xt.shape[0], 1), xt.cumsum(1)], 1)
+    return (cs[:, end] - cs[:, first]).t().float().contiguous()
 
 
 def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                              dnats_for_invalid_blocks):
+                              dnats_for_invalid_blocks, seqs=None):
     """The backward as kernels: the forward once more (storing every chunk's entering state and v_new), then the reverse
     scan and the per-chunk gradients (csrc/natsl_linear_bwd.hip)."""
     from . import _capi
     from ._mixed_common import linear_chunk_fwd
+    from .nats_util import _seq_args
     B, T, H, K = q.shape
     V = v.shape[-1]
     NB, HN = types.shape[1], types.shape[2]
-    NT = -(-T // C)
-    per = block // C
+    N = B if seqs is None else seqs.n_seqs
+    NTtot = B * (-(-T // C)) if seqs is None else seqs.total_chunks
     dev = q.device
     f32, bf16 = torch.float32, torch.bfloat16
     delta = kind == 'gdn'
@@ -144,46 +196,36 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
         gf = g.detach().to(f32).contiguous()
         bb = beta.detach().to(bf16).contiguous() if delta else None
         h0f = None if h0 is None else h0.detach().to(f32).contiguous()
-        _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, None,
+        _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, seqs,
                                                    chunk_states=True)
-        pad = NB * block - T
-        gp = torch.cat([gf, gf.new_zeros(B, pad, H)], 1) if pad else gf
-        gsum = gp.view(B, NB, block, H).sum(2).contiguous()
+        tok0, tok1, ch0, ch1, tok_blk = _block_maps(B, T, block, seqs, dev)
+        gsum = _range_sums(gf.view(B * T, H), tok0, tok1).contiguous()                  # [all blocks, H]
         d_states = torch.empty_like(states)
         dq, dk, dv = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
         dg = torch.empty(B, T, H, dtype=f32, device=dev)
         dbeta = torch.empty(B, T, H, dtype=f32, device=dev) if delta else None
         dbeta_parts = torch.empty(B, T, H, V // 16, dtype=f32, device=dev) if delta else None
-        sdot_parts = torch.empty(B, NT, H, V // 16, dtype=f32, device=dev)
-        dh0 = torch.empty(B, H, K, V, dtype=f32, device=dev) if h0 is not None else None
-        gate = torch.empty(B, NT, H, dtype=f32, device=dev)
-        rb = torch.empty(B, NT, H, dtype=f32, device=dev)
+        sdot_parts = torch.empty(NTtot, H, V // 16, dtype=f32, device=dev)
+        dh0 = torch.empty(N, H, K, V, dtype=f32, device=dev) if h0 is not None else None
+        gate = torch.empty(NTtot, H, dtype=f32, device=dev)
+        rb = torch.empty(NTtot, H, dtype=f32, device=dev)
         dof = do.detach().to(bf16).contiguous()
         dhtf = None if dht is None else dht.detach().to(f32).contiguous()
         P = _capi.ptr
+        sp, ns, tot = _seq_args(seqs, NTtot)
         rc = _capi.lib().natsl_linear_chunk_bwd(
             1 if delta else 0, P(qb), P(kb), P(v_new), P(gf), P(bb), P(dof), P(dhtf), P(states), P(ty), _capi.dtype_code(ty.dtype),
-            P(gsum), P(ws), P(d_states), P(dbeta_parts), P(sdot_parts), P(dq), P(dk), P(dv), P(dg), P(dbeta), P(dh0), P(gate), P(rb), B, T, H, HN, K, V, NB, block,
-            float(scale), flags, _capi.dtype_code(bf16), _capi.stream_ptr(dev))
+            P(gsum), P(ws), P(d_states), P(dbeta_parts), P(sdot_parts), P(dq), P(dk), P(dv), P(dg), P(dbeta), P(dh0), P(gate), P(rb),
+            B, T, H, HN, K, V, NB, block, float(scale), flags, _capi.dtype_code(bf16), sp, ns, tot, _capi.stream_ptr(dev))
         _capi.check(rc, "natsl_linear_chunk_bwd")
-        cpad = NB * per - NT
-
-        def per_block(x):                                    # [B,NT,H] -> [B,NB,per,H]
-            x = torch.cat([x, x.new_zeros(B, cpad, H)], 1) if cpad else x
-            return x.view(B, NB, per, H)
-
         if decay:
-            # the decay of a rolled-back block acts on every token of the block
-            dg += per_block(rb).sum(2).repeat_interleave(block, dim=1)[:, :T]
-        lin = (torch.round(ty[..., 1].float()) == 1).repeat_interleave(H // HN, dim=2)                      # [B,NB,H]
-        gb = per_block(gate)
-        dn = torch.where(lin, gb.sum(2), torch.zeros_like(gb[:, :, 0]))
+            # the decay of a rolled-back block acts on every token of the block (rb is non-zero at such a block's last chunk)
+            dg.view(B * T, H).add_(rb[ch1 - 1][tok_blk])
+        lin = (torch.round(ty[..., 1].float()) == 1).repeat_interleave(H // HN, dim=2).view(-1, H)          # [all blocks, H]
+        dn = torch.where(lin, _range_sums(gate, ch0, ch1), torch.zeros_like(gsum))
         if dnats_for_invalid_blocks:
             # the (zero-valued) gate on the update a block that is not typed linear would have made: its last chunk's
-            last_idx = torch.full((NB,), per - 1, device=dev)
-            last_idx[-1] = (NT - 1) % per
-            g_last = gb.gather(2, last_idx.view(1, NB, 1, 1).expand(B, NB, 1, H)).squeeze(2)
-            dn = dn + torch.where(lin, torch.zeros_like(g_last), g_last)
+            dn = dn + torch.where(lin, torch.zeros_like(gsum), gate[ch1 - 1])
         dn = dn.view(B, NB, HN, H // HN).sum(3)
     return (dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), dg, None if dbeta is None else dbeta.to(beta.dtype), dh0, dn)
 

@@ -238,22 +238,8 @@ class _MixedFunction(torch.autograd.Function):
         if do_lin is None:
             do_lin = torch.zeros(*q_l.shape[:3], v_l.shape[-1], dtype=torch.float32, device=q_l.device)
         lin_args = (cfg['scale_lattn'], cfg['block'], cfg['decay_non_linear'], cfg['qk_l2norm'], cfg['lin_intra'])
-        if seqs is None:
-            dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
-                cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, *lin_args, do_lin, dht, cfg['dnats_invalid_linear'])
-        else:
-            # packed sequences: each sequence is its own chain (own initial state, own blocks)
-            parts = []
-            for i in range(seqs.n_seqs):
-                a, b = seqs.cu_seqlens[i], seqs.cu_seqlens[i + 1]
-                na, nb_ = seqs.cu_seqlens_nats[i], seqs.cu_seqlens_nats[i + 1]
-                parts.append(linear_chunk_backward(
-                    cfg['kind'], q_l[:, a:b], k_l[:, a:b], v_l[:, a:b], g[:, a:b], None if beta is None else beta[:, a:b],
-                    None if h0 is None else h0[i:i + 1], types[:, na:nb_], *lin_args, do_lin[:, a:b],
-                    None if dht is None else dht[i:i + 1], cfg['dnats_invalid_linear']))
-            cat = lambda j, dim: None if parts[0][j] is None else torch.cat([p[j] for p in parts], dim)
-            dq_l, dk_l, dv_l, dg, dbeta, dn_lin = cat(0, 1), cat(1, 1), cat(2, 1), cat(3, 1), cat(4, 1), cat(6, 1)
-            dh0 = cat(5, 0)
+        dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
+            cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, *lin_args, do_lin, dht, cfg['dnats_invalid_linear'], seqs)
         d_types = torch.stack([dn_attn.float(), dn_lin.float()], -1)
         grads = [dq_a, dk_a, dv_a, dq_l, dk_l, dv_l, dh0, dg, dbeta, d_types]
         grads = [None if (t is None or dt is None) else t.to(dt) for t, dt in zip(grads, ctx.in_dtypes)]

@@ -62,6 +62,8 @@ struct LinBwdParams {
   float* sdot_parts;      // [chunk][H][V / 16]: <dS', S> over each wave's 16 columns, dS' still in fp32 (scan -> per-chunk kernel)
   float* gate;            // [chunk][H]: derivative with respect to a gate on the chunk's state update
   float* rb;              // [chunk][H]: f <dS', S_blockstart> behind a rolled-back block's last chunk (the decay's share of dg)
+  const SeqRow* seqs;     // packed sequences (B = 1), or null
+  int n_seqs, total_chunks;
   int B, T, H, HN, V, TN, block, nt;
   float scale;
   int flags;
@@ -244,8 +246,13 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
   const int nsplit = p.V / 64;
   const int chain = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
   const int n = chain / p.H, h = chain % p.H;
-  const int bos = n * p.T, len = p.T, chunk_off = n * p.nt;
-  const int NT = p.nt;
+  int bos, len, chunk_off, blk0;   // first token, length, first chunk and first selector block of the sequence
+  if (p.seqs == nullptr) {
+    bos = n * p.T; len = p.T; chunk_off = n * p.nt; blk0 = n * p.TN;
+  } else {
+    bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; chunk_off = p.seqs[n].chunk_off; blk0 = p.seqs[n].bos_nats;
+  }
+  const int NT = (len + CB - 1) / CB;
   const int vcol0 = split * 64;
   const int col = vcol0 + 16 * wave + x16;
   const int per = p.block / CB;
@@ -297,10 +304,10 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
       if (DELTA) beta_r = p.beta[gi];
     }
     const int blk = t0 / p.block;
-    const size_t ti = ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1;
+    const size_t ti = ((size_t)(blk0 + blk) * p.HN + hn) * 2 + 1;
     if (p.types_dtype == NATSL_F32) ty_r = reinterpret_cast<const unsigned*>(p.types)[ti];
     else ty_r = reinterpret_cast<const bf16_t*>(p.types)[ti];
-    gs_r = p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h];
+    gs_r = p.gsum_blk[((size_t)blk0 + blk) * p.H + h];
   };
   fetch(NT - 1);
 
@@ -554,7 +561,7 @@ struct BwdChunkLds {
   static constexpr int QN = 0, KN = QN + CB * KP, GN = KN + CB * KP, GT = GN + CB * TP, HS = GT + CB * TP, P2 = HS + CB * TP;
   static constexpr int ELEMS = P1 > P2 ? P1 : P2;
   static constexpr int FL = ELEMS * 2;
-  static constexpr int TOTAL = FL + (8 * CB + 8) * 4;
+  static constexpr int TOTAL = FL + (8 * CB + 32) * 4;
 };
 
 template <int DK, bool DELTA>
@@ -566,20 +573,31 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   float* const fl = reinterpret_cast<float*>(smem + L::FL);
   float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *dgam = fl + 6 * CB,
         *sqv = fl + 7 * CB;
-  float* red = fl + 8 * CB;   // [0] <dS', S>, [1] sum of the gate terms, [2] <dS', S_blockstart>
+  // [0] <dS', S>; [4..7] <dS', S_blockstart> per wave; [8..23] the gate terms per (wave, lane group): summed in a fixed order
+  float* red = fl + 8 * CB;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
   const int gc = blockIdx.x / p.H, h = blockIdx.x % p.H;
-  const int n = gc / p.nt, c = gc - n * p.nt;
-  const int t0 = c * CB, nvalid = min(CB, p.T - t0);
-  const size_t row0 = (size_t)n * p.T + t0;
+  int c, bos, len, blk0, chunk_off;
+  if (p.seqs == nullptr) {
+    const int n = gc / p.nt;
+    c = gc - n * p.nt; bos = n * p.T; len = p.T; blk0 = n * p.TN; chunk_off = n * p.nt;
+  } else {
+    int n = 0;
+    for (int i = 1; i < p.n_seqs; ++i)
+      if (p.seqs[i].chunk_off <= gc) n = i;
+    chunk_off = p.seqs[n].chunk_off;
+    c = gc - chunk_off; bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; blk0 = p.seqs[n].bos_nats;
+  }
+  const int t0 = c * CB, nvalid = min(CB, len - t0);
+  const size_t row0 = (size_t)bos + t0;
   const int per = p.block / CB;
   const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0, intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
   const bool l2 = DELTA && (p.flags & NATSL_QK_L2NORM) != 0;
   const int hn = h / (p.H / p.HN);
   const int blk = t0 / p.block;
-  const bool last = ((c + 1) % per == 0) || (c == p.nt - 1);
-  const bool lin = lin_type_b(p.types, p.types_dtype, ((size_t)(n * p.TN + blk) * p.HN + hn) * 2 + 1);
+  const bool last = ((c + 1) % per == 0) || (c == (len + CB - 1) / CB - 1);
+  const bool lin = lin_type_b(p.types, p.types_dtype, ((size_t)(blk0 + blk) * p.HN + hn) * 2 + 1);
   const bool rolled = last && !lin;
   const bool want_rb = rolled && decay;
   const int c_first = (c / per) * per;
@@ -589,7 +607,6 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
     const size_t gi = (row0 + lane) * p.H + h;
     store_scalars<DELTA>(lane, ok ? p.g[gi] : 0.f, DELTA && ok ? bf16_to_f32(p.beta[gi]) : 0.f, p.scale, gam, eg, ek, sqv, bet);
   }
-  if (tid < 8) red[tid] = 0.f;
   // q^, k^ are requested now and put into LDS when phase 1 is done with it
   QkRegs<DK> qk;
   load_qk<DK>(p, tid, row0, nvalid, h, qk);
@@ -611,7 +628,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   const size_t unit = (size_t)gc * p.H + h;
   const bf16_t* s_src = p.s_all + unit * p.V * DK;
   const bf16_t* ds_src = p.ds_all + unit * p.V * DK;
-  const bf16_t* sf_src = p.s_all + ((size_t)(n * p.nt + c_first) * p.H + h) * p.V * DK;
+  const bf16_t* sf_src = p.s_all + ((size_t)(chunk_off + c_first) * p.H + h) * p.V * DK;
   for (int vs = 0; vs < p.V / 64; ++vs) {
     u32x4 w_do[2], w_vn[2], w_dx[2];
     load_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, 64 * vs, w_do);
@@ -663,7 +680,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   }
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) srb += __shfl_xor(srb, d);
-  if (lane == 0) atomicAdd(&red[2], srb);
+  if (lane == 0) red[4 + wave] = srb;
   if (tid == 64) {
     // <dS', S>: the scan's partial sums, in a fixed order
     const float* pp = p.sdot_parts + unit * (p.V / 16);
@@ -794,7 +811,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
       dgam[16 * wave + 4 * g4 + r] = a_i[r] - b_i[r] + 2.f * rsH[r] - 2.f * t2_i[r];
       t3s += t3_i[r];
     }
-    atomicAdd(&red[1], t3s);
+    red[8 + 4 * wave + g4] = t3s;
   }
   __syncthreads();   // every wave is done with q^, k^ and the weight tiles; dgam and red are complete
 
@@ -826,7 +843,9 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   }
   if (wave == 0) {
     // dg_t = sum_{i >= t} dgamma_i + dG
-    const float dG = nr * (red[1] + __expf(gam[CB - 1]) * red[0]);
+    float gate_sum = 0.f;
+    for (int i = 0; i < 16; ++i) gate_sum += red[8 + i];
+    const float dG = nr * (gate_sum + __expf(gam[CB - 1]) * red[0]);
     float x = dgam[lane];
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -835,8 +854,8 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
     }
     if (lane < nvalid) p.dg[(row0 + lane) * p.H + h] = x + dG;
     if (lane == 0) {
-      p.gate[unit] = red[1];
-      p.rb[unit] = want_rb ? __expf(p.gsum_blk[((size_t)n * p.TN + blk) * p.H + h]) * red[2] : 0.f;
+      p.gate[unit] = gate_sum;
+      p.rb[unit] = want_rb ? __expf(p.gsum_blk[((size_t)blk0 + blk) * p.H + h]) * (red[4] + red[5] + red[6] + red[7]) : 0.f;
     }
   }
   __syncthreads();
@@ -857,7 +876,7 @@ static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* wha
     auto kern = linear_bwd_scan_kernel<DK, DELTA>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)(p.B * p.H * (p.V / 64))), dim3(256), L::TOTAL, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((p.seqs ? p.n_seqs : p.B) * p.H * (p.V / 64))), dim3(256), L::TOTAL, stream, p);
     const int rc = check_launch(what);
     if (rc != NATSL_OK) return rc;
   }
@@ -866,7 +885,7 @@ static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* wha
     auto kern = linear_bwd_chunk_kernel<DK, DELTA>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)(p.B * p.nt * p.H)), dim3(256), L::TOTAL, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.total_chunks * p.H)), dim3(256), L::TOTAL, stream, p);
     return check_launch(what);
   }
 }
@@ -880,7 +899,7 @@ extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void*
                                       const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
                                       float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
                                       int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
-                                      natsl_stream_t stream) {
+                                      const natsl_seq_row* seqs, int n_seqs, int total_chunks, natsl_stream_t stream) {
   const char* what = "natsl_linear_chunk_bwd";
   if (!q || !k || !v_new || !g || !d_o || !chunk_states || !types || !g_block_sums || !d_chunk_states || !dq || !dk || !dv || !dg ||
       !d_gate || !d_rollback || !state_dot_parts || (delta_rule && (!beta || !dbeta || !dbeta_parts || !workspace)))
@@ -891,13 +910,15 @@ extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void*
   if (H % HN) return fail(NATSL_ERR_INVALID, "%s: H=%d must be a multiple of HN=%d", what, H, HN);
   if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "%s: block size %d must be a multiple of 64", what, block);
   if (V % 64 || V <= 0) return fail(NATSL_ERR_UNSUPPORTED, "%s: V=%d must be a multiple of 64", what, V);
-  if (TN != cdiv(T, block)) return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d", what, TN, T, block);
+  if (seqs ? (B != 1 || n_seqs <= 0 || total_chunks <= 0) : (TN != cdiv(T, block)))
+    return fail(NATSL_ERR_INVALID, "%s: TN=%d does not match T=%d, block=%d (or bad packed-input arguments)", what, TN, T, block);
   LinBwdParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.vn = (const bf16_t*)v_new; p.d_o = (const bf16_t*)d_o; p.g = g;
   p.beta = (const bf16_t*)beta; p.s_all = (const bf16_t*)chunk_states; p.ds_all = (bf16_t*)d_chunk_states; p.dv = (bf16_t*)dv;
   p.dht = dht; p.dh0 = dh0; p.gsum_blk = g_block_sums; p.ws_tm = (const bf16_t*)workspace; p.types = types; p.types_dtype = types_dtype;
   p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dg = dg; p.dbeta = dbeta; p.dbeta_parts = dbeta_parts; p.sdot_parts = state_dot_parts; p.gate = d_gate; p.rb = d_rollback;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block; p.nt = cdiv(T, CB);
+  p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0; p.total_chunks = seqs ? total_chunks : B * p.nt;
   p.scale = scale; p.flags = flags;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (delta_rule) {

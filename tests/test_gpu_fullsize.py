@@ -33,13 +33,13 @@ def _inputs(B, T, H, K, V, seed):
     return q, k, v, g, beta
 
 
-def _assert_doubles(o2, o1, what):
+def _assert_doubles(o2, o1, what, one_in=1_000_000):
     """o2 == 2*o1 bit for bit, except where an intermediate product falls into the denormal range (flushed by
-    the matrix cores): there the two runs may differ by one rounding.  Allow at most one element in a million,
-    and only by a negligible amount."""
+    the matrix cores): there the two runs may differ by one rounding.  Allow at most one element in a million
+    (`one_in`), and only by a negligible amount."""
     d = (o2.float() - 2 * o1.float()).abs()
     bad = int((d != 0).sum())
-    assert bad <= max(1, o1.numel() // 1_000_000) and float(d.max()) <= 1e-4, f"{what}: {bad} elements differ, max {float(d.max()):.3e}"
+    assert bad <= max(1, o1.numel() // one_in) and float(d.max()) <= 1e-4, f"{what}: {bad} elements differ, max {float(d.max()):.3e}"
 
 
 def _linear(kind, q, k, v, g, beta, h0, types, block, scale, decay=True, seqs=None, final=True):
@@ -309,3 +309,46 @@ def test_c3_packed_sequence_against_token_recurrence():
     o_lin, s = _linear('gdn', q, k, v, g, beta, None, ty, block, scale, seqs=seqs)
     _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o_lin, s, 0, 9, block, scale, t0=cu[3], t1=cu[4], s_index=3, what="c3 packed")
     _gdn_slice_against_token_recurrence(q, k, v, g, beta, ty, o_lin, s, 0, 30, block, scale, t0=cu[1], t1=cu[2], s_index=1, what="c3 packed")
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / (b.norm() + 1e-30))
+
+
+def test_c2_gdn_backward_full_depth(c2):
+    """The linear branch's backward kernels at c2 (128 chunks deep, the drawn mask, decay across attention blocks):
+    (i) two (batch, head) slices against autograd through the fp64 chunked oracle on that slice alone (heads and batch
+    entries are independent chains); (ii) the whole result against the torch formulation of the same method;
+    (iii) the gradients are linear in dO: doubling dO doubles them bit for bit.
+    Tolerances as in tests/test_gpu_linear_bwd.py: rel-L2 5e-3 for dq, dk, dv, 1e-2 for the per-token scalars dg, dbeta."""
+    from oracle import linear_branch as LB
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    w = C2
+    scale = w['K'] ** -0.5
+    do = _randn((w['B'], w['T'], w['H'], w['V']), 300)
+    args = ('gdn', c2['q'], c2['k'], c2['v'], c2['g'], c2['beta'], None, c2['ty'], scale, w['block'], True, True, True)
+    with torch.no_grad():
+        got = B_.linear_chunk_backward_hip(*args, do, None, False)
+        got2 = B_.linear_chunk_backward_hip(*args, do * 2, None, False)
+        ref = B_.linear_chunk_backward_torch(*args, do, None, False)
+    names = ['dq', 'dk', 'dv', 'dg', 'dbeta']
+    for j, name in enumerate(names):
+        assert torch.isfinite(got[j].float()).all(), name
+        # (a gradient passes through many more products than an output: one element in 100 000)
+        _assert_doubles(got2[j], got[j], f"{name}(2 dO) vs 2 {name}(dO)", 100_000)
+        r = _rel(got[j], ref[j])
+        assert r <= (1e-2 if name in ('dg', 'dbeta') else 5e-3), f"{name} against the torch formulation: rel-L2 {r:.3e}"
+    r = _rel(got[6], ref[6])
+    assert r <= 1e-2, f"dnats against the torch formulation: rel-L2 {r:.3e}"
+    for b, h in ((0, 0), (6, 13)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].cpu()
+        o = LB.linear_branch_bwd('gdn', sl(c2['q']), sl(c2['k']), sl(c2['v']), sl(c2['g']), sl(c2['beta']), c2['ty'][b:b + 1, :, h:h + 1, 1].cpu(),
+                                 scale, sl(do), None, None, w['block'], True, True, True, False)
+        errs = {}
+        for j, name in enumerate(names):
+            errs[name] = _rel(got[j][b:b + 1, :, h:h + 1], o[name])
+            assert errs[name] <= (1e-2 if name in ('dg', 'dbeta') else 5e-3), f"{name}[{b},:,{h}] against the fp64 oracle: rel-L2 {errs[name]:.3e}"
+        e_n = _rel(got[6][b:b + 1, :, h:h + 1], o['dnats'])
+        assert e_n <= 1e-2, f"dnats[{b},:,{h}] against the fp64 oracle: rel-L2 {e_n:.3e}"
+        print(f"\nc2 backward slice ({b},{h}): " + "  ".join(f"{n} {e:.2e}" for n, e in errs.items()) + f"  dnats {e_n:.2e}", flush=True)

@@ -83,6 +83,41 @@ def test_backward_entry_rejects_what_is_not_built():
     L = _capi.lib()
     p = ctypes.c_void_p(256)
     args = lambda K, V, block: (1, p, p, p, p, p, p, None, p, p, 1, p, p, p, p, p, p, p, p, p, p, None, p, p, 1, 256, 4, 4, K, V, 256 // block, block,
-                                0.1, 7, 1, None)
+                                0.1, 7, 1, None, 0, 0, None)
     assert L.natsl_linear_chunk_bwd(*args(96, 64, 64)) == -2 and b"K=96" in L.natsl_last_error()
     assert L.natsl_linear_chunk_bwd(*args(128, 48, 64)) == -2 and b"V=48" in L.natsl_last_error()
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+def test_packed_sequences_equal_separate_calls(kind):
+    """One call over packed sequences gives, bit for bit, what one call per sequence gives (own initial state, own
+    final-state gradient, own blocks; ragged lengths)."""
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    from neuralattentionsearchlinear_amd.nats_util import pack_sequences
+    lens, H, HN, K, V, block = [200, 64, 450, 129], 4, 2, 128, 64, 128
+    T = sum(lens)
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    NB = sum(-(-n // block) for n in lens)
+    q, k, v, g, beta, _, _, do, _ = _inputs(kind, 1, T, H, HN, K, V, block, 7)
+    ty = make_types(1, NB, HN, 0.4, 9, torch.bfloat16)
+    gen = torch.Generator().manual_seed(5)
+    init = torch.randn(len(lens), H, K, V, generator=gen) * 0.3
+    dht = torch.randn(len(lens), H, K, V, generator=gen) * 0.3
+    d = lambda t: t.to(DEV)
+    scale = K ** -0.5 if kind == 'gdn' else 1.0
+    seqs = pack_sequences(cu, None, block, DEV)
+    args = lambda sl, nsl, i: (kind, d(q[:, sl]), d(k[:, sl]), d(v[:, sl]), d(g[:, sl]), d(beta[:, sl]) if kind == 'gdn' else None,
+                               d(init[i]), d(ty[:, nsl]), scale, block, True, kind == 'gdn', True, d(do[:, sl]), d(dht[i]), True)
+    whole = B_.linear_chunk_backward_hip(*args(slice(None), slice(None), slice(None)), seqs)
+    nb = 0
+    for i, n in enumerate(lens):
+        nbi = -(-n // block)
+        part = B_.linear_chunk_backward_hip(*args(slice(cu[i], cu[i + 1]), slice(nb, nb + nbi), slice(i, i + 1)))
+        for j, name in enumerate(['dq', 'dk', 'dv', 'dg', 'dbeta']):
+            if part[j] is not None:
+                assert torch.equal(whole[j][:, cu[i]:cu[i + 1]], part[j]), f"{name} of sequence {i}"
+        assert torch.equal(whole[5][i:i + 1], part[5]), f"dh0 of sequence {i}"
+        assert torch.equal(whole[6][:, nb:nb + nbi], part[6]), f"dnats of sequence {i}"
+        nb += nbi
