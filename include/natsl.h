@@ -199,6 +199,16 @@ int natsl_norm_gate_fwd(const void* x1, const void* x2, const void* gate, const 
                         const void* w2, void* y, int64_t rows, int D, int dtype, float eps, int w_dtype,
                         natsl_stream_t stream);
 
+/* Backward of natsl_norm_gate_fwd: dx1, dx2, dgate [rows, D] in `dtype`; dx_weights [rows, 2] f32; dw1, dw2 [D] f32, the two
+ * rows of ONE [2][D] tensor (dw2 == dw1 + D).  The weight gradients are summed over the rows in a fixed order (partial sums
+ * per 128 rows in the workspace, then one reduction): the same bits on every run.
+ * Replaces the backward of FusedMultiInputRMSNormGated (src/nats/modules/fused_norm_gate.py:185-420). */
+size_t natsl_norm_gate_bwd_workspace_bytes(int64_t rows, int D);
+int natsl_norm_gate_bwd(const void* x1, const void* x2, const void* gate, const void* x_weights, const void* w1,
+                        const void* w2, const void* dy, void* dx1, void* dx2, void* dgate, float* dx_weights, float* dw1,
+                        float* dw2, void* workspace, size_t workspace_bytes, int64_t rows, int D, int dtype, float eps,
+                        int w_dtype, natsl_stream_t stream);
+
 /* Layer glue, depthwise causal short convolution with its activation, on the layer's token-major tensors:
  * y[b,t,d] = act(bias[d] + sum_j w[d,j] e[b, t-(W-1)+j, d]) where e is x preceded by the W-1 inputs before it: the last
  * W-1 entries of `state` [B,D,W] (the cache of a previous call, in `state_dtype`), or zeros when state is NULL.

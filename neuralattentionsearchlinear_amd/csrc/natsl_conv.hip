@@ -227,16 +227,37 @@ __global__ __launch_bounds__(256) void short_conv_bwd_kernel(const void* x, cons
   }
 }
 
-// dw[d][j] = sum over run ids of part[id][j][d], dbias[d] = the same of part[id][W][d]; a thread per (j, d)
-__global__ __launch_bounds__(256) void conv_wgrad_reduce_kernel(const float* part, float* dw, float* dbias, const int n_part, const int D,
-                                                                const int W) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= (W + 1) * D) return;
-  const int j = i / D, d = i % D;
+// dw[d][j] = sum over run ids of part[id][j][d], dbias[d] = the same of part[id][W][d].  A workgroup takes 64 adjacent
+// (j, d) columns; its 16 thread rows each add up every 16th run id (eight loads in flight), then the 16 row sums are added
+// in a fixed order: the same bits on every run.
+__global__ __launch_bounds__(1024) void conv_wgrad_reduce_kernel(const float* part, float* dw, float* dbias, const int n_part, const int D,
+                                                                 const int W) {
+  __shared__ float sums[16][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + tx, n_col = (W + 1) * D;
   float acc = 0.f;
-  for (int k = 0; k < n_part; ++k) acc += part[((size_t)k * (W + 1) + j) * D + d];
-  if (j < W) dw[(size_t)d * W + j] = acc;
-  else if (dbias) dbias[d] = acc;
+  if (i < n_col) {
+    const float* src = part + i;
+    int k = ty;
+    for (; k + 7 * 16 < n_part; k += 8 * 16) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(k + 16 * u) * n_col];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; k < n_part; k += 16) acc += src[(size_t)k * n_col];
+  }
+  sums[ty][tx] = acc;
+  __syncthreads();
+  if (ty == 0 && i < n_col) {
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t += sums[r][tx];
+    const int j = i / D, d = i % D;
+    if (j < W) dw[(size_t)d * W + j] = t;
+    else if (dbias) dbias[d] = t;
+  }
 }
 
 // A row is handled by LANES adjacent lanes with PER pieces of 8 elements each (D = 8 LANES PER).
@@ -350,7 +371,7 @@ extern "C" int natsl_short_conv_bwd(const void* x, const void* weight, const voi
 #undef NATSL_CONVB
   int rc = check_launch(what);
   if (rc != NATSL_OK) return rc;
-  hipLaunchKernelGGL(conv_wgrad_reduce_kernel, dim3((unsigned)(((W + 1) * D + 255) / 256)), dim3(256), 0, s, part, dweight, dbias, B * runs, D, W);
+  hipLaunchKernelGGL(conv_wgrad_reduce_kernel, dim3((unsigned)(((W + 1) * D + 63) / 64)), dim3(1024), 0, s, part, dweight, dbias, B * runs, D, W);
   return check_launch(what);
 }
 

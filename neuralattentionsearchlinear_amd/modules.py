@@ -18,6 +18,7 @@ from . import _capi
 
 
 _ROW_NORM_WIDTHS = (32, 64, 96, 128, 192, 256, 384, 512)
+_NORM_GATE_WIDTHS = (32, 64, 96, 128, 192, 256, 384, 512)
 
 
 def _row_norm_torch(x, weight, eps, l2):
@@ -240,9 +241,9 @@ def _norm_gate_fwd(x1, x2, g, x_weights, weight1, weight2, eps):
 
 
 class _NormGate(torch.autograd.Function):
-    """The HIP forward with a backward for training: the gradients are those of the same formula evaluated as fp32 torch
-    operations (elementwise work plus two row reductions; replaces the backward of
-    src/nats/modules/fused_norm_gate.py:185-420 in function)."""
+    """The HIP forward and backward (natsl_norm_gate_fwd / natsl_norm_gate_bwd; the backward replaces that of
+    src/nats/modules/fused_norm_gate.py:185-420 in function).  Widths without a kernel: the gradients of the same formula as
+    fp32 torch operations."""
 
     @staticmethod
     def forward(ctx, x1, x2, g, x_weights, weight1, weight2, eps):
@@ -253,6 +254,28 @@ class _NormGate(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         saved = ctx.saved_tensors
+        x1, x2, g, xw, w1, w2 = saved
+        D = x1.shape[-1]
+        if D in _NORM_GATE_WIDTHS and x1.numel() > 0:
+            # natsl_norm_gate_bwd: one pass over the rows, the weight gradients through per-workgroup partial sums
+            to = lambda t: t.detach().to(torch.bfloat16).contiguous()
+            a, b, gg, xwb, d = to(x1), to(x2.reshape(x1.shape)), to(g.reshape(x1.shape)), to(xw), to(dy.reshape(x1.shape))
+            wa, wb = w1.detach().contiguous(), w2.detach().contiguous()
+            if wa.dtype != wb.dtype or wa.dtype not in (torch.float32, torch.bfloat16):
+                wa, wb = wa.float(), wb.float()
+            rows = a.numel() // D
+            L = _capi.lib()
+            da, db, dg = torch.empty_like(a), torch.empty_like(a), torch.empty_like(a)
+            dxw = torch.empty(rows, 2, dtype=torch.float32, device=a.device)
+            dw = torch.empty(2, D, dtype=torch.float32, device=a.device)
+            ws = torch.empty(L.natsl_norm_gate_bwd_workspace_bytes(rows, D), dtype=torch.uint8, device=a.device)
+            P = _capi.ptr
+            rc = L.natsl_norm_gate_bwd(P(a), P(b), P(gg), P(xwb), P(wa), P(wb), P(d), P(da), P(db), P(dg), P(dxw), P(dw[0]), P(dw[1]),
+                                       P(ws), ws.numel(), rows, D, _capi.BF16, float(ctx.eps), _capi.dtype_code(wa.dtype),
+                                       _capi.stream_ptr(a.device))
+            _capi.check(rc, "natsl_norm_gate_bwd")
+            return (da.to(x1.dtype), db.view(x2.shape).to(x2.dtype), dg.view(g.shape).to(g.dtype), dxw.view(xw.shape).to(xw.dtype),
+                    dw[0].to(w1.dtype), dw[1].to(w2.dtype), None)
         with torch.enable_grad():
             x1, x2, g, xw, w1, w2 = (t.detach().float().requires_grad_(True) for t in saved)
             r1 = x1 * torch.rsqrt((x1 * x1).mean(-1, keepdim=True) + ctx.eps) * w1

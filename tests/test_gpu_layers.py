@@ -31,6 +31,31 @@ def test_norm_gate(D, wdtype):
     assert rel_l2(y.float(), ref) <= 5e-3
 
 
+@pytest.mark.parametrize("D,wdtype", [(32, torch.float32), (128, torch.bfloat16), (256, torch.float32), (384, torch.float32)])
+def test_norm_gate_backward(D, wdtype):
+    """natsl_norm_gate_bwd against fp64 autograd through the oracle's formula on the same (bf16-rounded) inputs; 300 rows are
+    three workgroups' worth, so the weight gradients cross the partial-sum reduction."""
+    from neuralattentionsearchlinear_amd.modules import two_inputs_rms_norm_gated
+    g = torch.Generator().manual_seed(D + 1)
+    shape = (2, 50, 3, D)
+    x1, x2, gate, dy = (torch.randn(shape, generator=g).bfloat16() for _ in range(4))
+    xw = torch.softmax(torch.randn(2, 50, 3, 2, generator=g), -1).bfloat16()
+    w1, w2 = (1 + 0.1 * torch.randn(D, generator=g)).to(wdtype), (1 + 0.1 * torch.randn(D, generator=g)).to(wdtype)
+    leaves = [t.double().requires_grad_(True) for t in (x1, x2, gate, xw, w1, w2)]
+    ref_y = ong.two_input_rmsnorm_gated(*leaves, 1e-5, dtype=torch.float64)
+    ref = torch.autograd.grad(ref_y, leaves, dy.double())
+    dev = [t.to(DEV).requires_grad_(True) for t in (x1, x2, gate, xw, w1, w2)]
+    y = two_inputs_rms_norm_gated(*dev, 1e-5)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    for name, t, r in zip(['dx1', 'dx2', 'dgate', 'dx_weights', 'dw1', 'dw2'], dev, ref):
+        got = t.grad.double().cpu()
+        err = (got - r).abs()
+        # outputs are rounded to the inputs' dtype: one bf16 ulp of the value plus a small absolute term
+        assert bool((err <= 2.0 ** -7 * r.abs() + 2e-3 * float(r.abs().max())).all()), f"{name}: max-abs {float(err.max()):.3e}"
+        assert rel_l2(got, r) <= 5e-3, f"{name}: rel-L2 {rel_l2(got, r):.3e}"
+
+
 # head geometry of the two published model configurations (experiments/configs/natsl_340M.json, natsl_760M.json):
 # linear heads K 128 / V 256 resp. K 192 / V 384, attention view K 64 / V 128 in both
 PUBLISHED = {'340M': dict(hidden_size=1024, head_dim=128, num_heads=6, num_attn_heads=12, norm_eps=1e-6),
