@@ -322,12 +322,14 @@ def linear_branch_bwd(kind, q, k, v, g, beta, lin_types, scale, do, dht=None, h0
         loss = loss + (S * dht.to(dtype)).sum()
     loss.backward()
     lin_c = _expand_types(lin_types, H).repeat_interleave(per, dim=1)[:, :NT]
-    dn = torch.where(lin_c, gate_on.grad, torch.zeros_like(gate_on.grad))
+    # (a leaf nothing of the loss depends on -- one chunk without a final-state gradient -- has no gradient: zero)
+    z_ = lambda t, like: torch.zeros_like(like) if (t is None or t.grad is None) else t.grad
+    dn = torch.where(lin_c, z_(gate_on, gate_on), torch.zeros_like(gate_on))
     if dnats_for_invalid_blocks:
-        dn = dn + torch.where(lin_c, torch.zeros_like(dn), gate_off.grad)
+        dn = dn + torch.where(lin_c, torch.zeros_like(dn), z_(gate_off, gate_off))
     NB = lin_types.shape[1]
     if NB * per != NT:
         dn = torch.cat([dn, dn.new_zeros(B, NB * per - NT, H)], 1)
     dn = dn.view(B, NB, per, HN, H // HN).sum((2, 4))
-    g_ = lambda t: None if t is None else t.grad
+    g_ = lambda t: None if t is None else z_(t, t)
     return dict(dq=g_(qf), dk=g_(kf), dv=g_(vf), dg=g_(gf), dbeta=g_(bf), dh0=g_(hf), dnats=dn)

@@ -121,3 +121,37 @@ def test_packed_sequences_equal_separate_calls(kind):
         assert torch.equal(whole[5][i:i + 1], part[5]), f"dh0 of sequence {i}"
         assert torch.equal(whole[6][:, nb:nb + nbi], part[6]), f"dnats of sequence {i}"
         nb += nbi
+
+
+def _random_case(seed):
+    import random
+    r = random.Random(seed)
+    kind = r.choice(['gdn', 'gdn', 'mamba'])
+    K = r.choice([64, 128, 192])
+    V = r.choice([64, 128]) if K < 192 else 64
+    block = r.choice([64, 128, 256])
+    H = r.choice([1, 2, 4])
+    HN = r.choice([h for h in (1, 2, 4) if H % h == 0])
+    T = r.choice([r.randrange(1, 64), r.randrange(65, 400), 64 * r.randrange(1, 7)])
+    return (kind, r.choice([1, 2]), T, H, HN, K, V, block, r.random() < 0.7, r.random() < 0.85, r.random() < 0.5, r.random() < 0.5,
+            r.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_linear_branch_backward_random_shapes(seed):
+    """Drawn shapes and options (ragged lengths down to a single token, all three key widths, blocks of 1, 2, 4 chunks,
+    selector heads shared by several heads) against the fp64 oracle."""
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    case = _random_case(1000 + seed)
+    kind, B, T, H, HN, K, V, block, decay, intra, h0, dht_on, invalid = case
+    q, k, v, g, beta, ty, init, do, dht = _inputs(kind, B, T, H, HN, K, V, block, 500 + seed)
+    scale = K ** -0.5 if kind == 'gdn' else 1.0
+    l2 = kind == 'gdn'
+    ref = LB.linear_branch_bwd(kind, q, k, v, g, beta if kind == 'gdn' else None, ty[..., 1], scale, do, dht if dht_on else None,
+                               init if h0 else None, block, decay, l2, intra, invalid)
+    d = lambda t: t.to(DEV)
+    print(f"\ncase {case}", flush=True)
+    out = B_.linear_chunk_backward_hip(kind, d(q), d(k), d(v), d(g), d(beta) if kind == 'gdn' else None, d(init) if h0 else None, d(ty),
+                                       scale, block, decay, l2, intra, d(do), d(dht) if dht_on else None, invalid)
+    torch.cuda.synchronize()
+    _check(out, ref, kind, h0)
