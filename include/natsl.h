@@ -179,14 +179,14 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
  *   d_rollback [chunks][H] f32 = what the decay of a rolled-back block adds to dg of each of its tokens (non-zero behind
  *   the last chunk of blocks that are not typed linear, NATSL_DECAY_NON_LINEAR only);
  *   d_chunk_states: scratch, bf16 [chunks][H][V][K] (the gradient of the state behind every chunk);
- *   dbeta_parts: scratch, f32 [B*T][H][V/16] (delta rule only); state_dot_parts: scratch, f32 [chunks][H][V/16].
+ *   dbeta_parts: scratch, f32 [B*T][H][V/16] (delta rule only).
  * K in {64, 128, 192}, V a multiple of 64.
  * Replaces chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart
  * (src/nats/ops/mamba/chunk.py:112-260). */
 int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void* k, const void* v_new, const float* g, const void* beta,
                            const void* d_o, const float* dht, const void* chunk_states, const void* types, int types_dtype,
                            const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
-                           float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
+                           void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
                            int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
                            const natsl_seq_row* seqs, int n_seqs, int total_chunks, natsl_stream_t stream);
 

@@ -205,7 +205,6 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
         dg = torch.empty(B, T, H, dtype=f32, device=dev)
         dbeta = torch.empty(B, T, H, dtype=f32, device=dev) if delta else None
         dbeta_parts = torch.empty(B, T, H, V // 16, dtype=f32, device=dev) if delta else None
-        sdot_parts = torch.empty(NTtot, H, V // 16, dtype=f32, device=dev)
         dh0 = torch.empty(N, H, K, V, dtype=f32, device=dev) if h0 is not None else None
         gate = torch.empty(NTtot, H, dtype=f32, device=dev)
         rb = torch.empty(NTtot, H, dtype=f32, device=dev)
@@ -215,7 +214,7 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
         sp, ns, tot = _seq_args(seqs, NTtot)
         rc = _capi.lib().natsl_linear_chunk_bwd(
             1 if delta else 0, P(qb), P(kb), P(v_new), P(gf), P(bb), P(dof), P(dhtf), P(states), P(ty), _capi.dtype_code(ty.dtype),
-            P(gsum), P(ws), P(d_states), P(dbeta_parts), P(sdot_parts), P(dq), P(dk), P(dv), P(dg), P(dbeta), P(dh0), P(gate), P(rb),
+            P(gsum), P(ws), P(d_states), P(dbeta_parts), P(dq), P(dk), P(dv), P(dg), P(dbeta), P(dh0), P(gate), P(rb),
             B, T, H, HN, K, V, NB, block, float(scale), flags, _capi.dtype_code(bf16), sp, ns, tot, _capi.stream_ptr(dev))
         _capi.check(rc, "natsl_linear_chunk_bwd")
         if decay:

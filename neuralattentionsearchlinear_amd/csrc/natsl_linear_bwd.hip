@@ -59,7 +59,6 @@ struct LinBwdParams {
   float* dg;              // [tokens][H]
   float* dbeta;           // [tokens][H]
   float* dbeta_parts;     // [tokens][H][V / 16]: <dX, v_new> over each wave's 16 columns (scan -> per-chunk kernel)
-  float* sdot_parts;      // [chunk][H][V / 16]: <dS', S> over each wave's 16 columns, dS' still in fp32 (scan -> per-chunk kernel)
   float* gate;            // [chunk][H]: derivative with respect to a gate on the chunk's state update
   float* rb;              // [chunk][H]: f <dS', S_blockstart> behind a rolled-back block's last chunk (the decay's share of dg)
   const SeqRow* seqs;     // packed sequences (B = 1), or null
@@ -272,7 +271,6 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
   // ---- what a thread fetches for a chunk; requested one chunk ahead, under the state-gradient update of the chunk before ----
   QkRegs<DK> qk;
   u32x4 do_r[2], vn_r[2], tm_r[2];
-  u32x2 s_r[KT16];      // the chunk's entering state, this lane's column: for <dS', S>
   // (scalars are fetched raw and interpreted when the chunk's turn comes: anything computed from them here would make
   // the wave wait for all of the requests)
   float g_r = 0.f, gs_r = 0.f;
@@ -295,9 +293,6 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
         }
       }
     }
-    const size_t so = (((size_t)(chunk_off + cc) * p.H + h) * p.V + col) * DK + 4 * g4;
-#pragma unroll
-    for (int m = 0; m < KT16; ++m) s_r[m] = *reinterpret_cast<const u32x2*>(p.s_all + so + 16 * m);
     if (wave == 0) {
       const size_t gi = (row0 + min(lane, nvalid - 1)) * p.H + h;
       g_r = p.g[gi];
@@ -332,21 +327,14 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
     }
     const bool lin = rintf(__uint_as_float(p.types_dtype == NATSL_F32 ? ty_r : ty_r << 16)) == 1.0f;
     const float f_blk = decay ? __expf(gs_r) : 1.f;
-    float sd = 0.f;
     {
-      // dS' of this chunk goes out as it arrived, and <dS', S> with it
+      // dS' of this chunk goes out as it arrived
       bf16_t* dso = p.ds_all + (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 4 * g4;
 #pragma unroll
       for (int m = 0; m < KT16; ++m) {
         u32x2 w = {pack_bf16x2(dS[m][0], dS[m][1]), pack_bf16x2(dS[m][2], dS[m][3])};
         *reinterpret_cast<u32x2*>(dso + 16 * m) = w;
-        const u32x2 sw = s_r[m];
-        sd += dS[m][0] * __uint_as_float(sw[0] << 16) + dS[m][1] * __uint_as_float(sw[0] & 0xffff0000u) +
-              dS[m][2] * __uint_as_float(sw[1] << 16) + dS[m][3] * __uint_as_float(sw[1] & 0xffff0000u);
       }
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) sd += __shfl_xor(sd, d);
-      if (lane == 0) p.sdot_parts[((size_t)(chunk_off + c) * p.H + h) * (p.V / 16) + 4 * split + wave] = sd;
     }
     __syncthreads();   // the tiles are there
 
@@ -397,24 +385,20 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
     }
     const float dec = __expf(gam[CB - 1]);
 
-    // ---- Y1 = K~ dS' (the state gradient as two operands: truncated value and remainder) --------------------------------
+    // ---- Y1 = K~ dS' ----------------------------------------------------------------------------------------------------
     f32x4 DV[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) DV[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     {
-      bf16x8 DSB[KS], DSR[KS];
+      bf16x8 DSB[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        DSB[s] = pack8_trunc(dS[2 * s], dS[2 * s + 1]);
-        DSR[s] = pack8_rest(dS[2 * s], dS[2 * s + 1]);
-      }
+      for (int s = 0; s < KS; ++s) DSB[s] = pack8(dS[2 * s], dS[2 * s + 1]);
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
           const bf16_t* kr = Kn + (16 * t + x16) * KP + 32 * s + 4 * g4;
           const bf16x8 a = join_u2(*reinterpret_cast<const u32x2*>(kr), *reinterpret_cast<const u32x2*>(kr + 16));
-          DV[t] = mfma16(a, DSR[s], DV[t]);
           DV[t] = mfma16(a, DSB[s], DV[t]);
         }
 #pragma unroll
@@ -573,7 +557,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   float* const fl = reinterpret_cast<float*>(smem + L::FL);
   float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *dgam = fl + 6 * CB,
         *sqv = fl + 7 * CB;
-  // [0] <dS', S>; [4..7] <dS', S_blockstart> per wave; [8..23] the gate terms per (wave, lane group): summed in a fixed order
+  // [0..3] <dS', S> and [4..7] <dS', S_blockstart> per wave; [8..23] the gate terms per (wave, lane group): summed in a fixed order
   float* red = fl + 8 * CB;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
@@ -624,7 +608,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   for (int m = 0; m < KT16; ++m) {
     DQ2[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; DW[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; DK3[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
-  float srb = 0.f;
+  float sds = 0.f, srb = 0.f;
   const size_t unit = (size_t)gc * p.H + h;
   const bf16_t* s_src = p.s_all + unit * p.V * DK;
   const bf16_t* ds_src = p.ds_all + unit * p.V * DK;
@@ -646,10 +630,14 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
       const u32x4 wd = *reinterpret_cast<const u32x4*>(ds_src + off);
       *reinterpret_cast<u32x4*>(Sn + v * KP + seg * 8) = ws;
       *reinterpret_cast<u32x4*>(DSn + v * KP + seg * 8) = wd;
+      float fs[8], fd[8];
+      unpack8f(ws, fs);
+      unpack8f(wd, fd);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sds += fs[e] * fd[e];
       if (want_rb) {
-        float ff[8], fd[8];
+        float ff[8];
         unpack8f(*reinterpret_cast<const u32x4*>(sf_src + off), ff);
-        unpack8f(wd, fd);
 #pragma unroll
         for (int e = 0; e < 8; ++e) srb += ff[e] * fd[e];
       }
@@ -679,15 +667,8 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
     }
   }
 #pragma unroll
-  for (int d = 1; d < 64; d <<= 1) srb += __shfl_xor(srb, d);
-  if (lane == 0) red[4 + wave] = srb;
-  if (tid == 64) {
-    // <dS', S>: the scan's partial sums, in a fixed order
-    const float* pp = p.sdot_parts + unit * (p.V / 16);
-    float sum = 0.f;
-    for (int i = 0; i < p.V / 16; ++i) sum += pp[i];
-    red[0] = sum;
-  }
+  for (int d = 1; d < 64; d <<= 1) { sds += __shfl_xor(sds, d); srb += __shfl_xor(srb, d); }
+  if (lane == 0) { red[wave] = sds; red[4 + wave] = srb; }
 
   // ---- phase 2 -------------------------------------------------------------------------------------------------------
   bf16_t* const Qn = sm + L::QN;
@@ -845,7 +826,7 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
     // dg_t = sum_{i >= t} dgamma_i + dG
     float gate_sum = 0.f;
     for (int i = 0; i < 16; ++i) gate_sum += red[8 + i];
-    const float dG = nr * (gate_sum + __expf(gam[CB - 1]) * red[0]);
+    const float dG = nr * (gate_sum + __expf(gam[CB - 1]) * (red[0] + red[1] + red[2] + red[3]));
     float x = dgam[lane];
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -897,12 +878,12 @@ using namespace natsl;
 extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void* k, const void* v_new, const float* g, const void* beta,
                                       const void* d_o, const float* dht, const void* chunk_states, const void* types, int types_dtype,
                                       const float* g_block_sums, const void* workspace, void* d_chunk_states, float* dbeta_parts,
-                                      float* state_dot_parts, void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
+                                      void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0, float* d_gate, float* d_rollback, int B, int T,
                                       int H, int HN, int K, int V, int TN, int block, float scale, int flags, int dtype,
                                       const natsl_seq_row* seqs, int n_seqs, int total_chunks, natsl_stream_t stream) {
   const char* what = "natsl_linear_chunk_bwd";
   if (!q || !k || !v_new || !g || !d_o || !chunk_states || !types || !g_block_sums || !d_chunk_states || !dq || !dk || !dv || !dg ||
-      !d_gate || !d_rollback || !state_dot_parts || (delta_rule && (!beta || !dbeta || !dbeta_parts || !workspace)))
+      !d_gate || !d_rollback || (delta_rule && (!beta || !dbeta || !dbeta_parts || !workspace)))
     return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
   if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
@@ -916,7 +897,7 @@ extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void*
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.vn = (const bf16_t*)v_new; p.d_o = (const bf16_t*)d_o; p.g = g;
   p.beta = (const bf16_t*)beta; p.s_all = (const bf16_t*)chunk_states; p.ds_all = (bf16_t*)d_chunk_states; p.dv = (bf16_t*)dv;
   p.dht = dht; p.dh0 = dh0; p.gsum_blk = g_block_sums; p.ws_tm = (const bf16_t*)workspace; p.types = types; p.types_dtype = types_dtype;
-  p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dg = dg; p.dbeta = dbeta; p.dbeta_parts = dbeta_parts; p.sdot_parts = state_dot_parts; p.gate = d_gate; p.rb = d_rollback;
+  p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dg = dg; p.dbeta = dbeta; p.dbeta_parts = dbeta_parts; p.gate = d_gate; p.rb = d_rollback;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block; p.nt = cdiv(T, CB);
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0; p.total_chunks = seqs ? total_chunks : B * p.nt;
   p.scale = scale; p.flags = flags;
