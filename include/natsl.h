@@ -240,6 +240,15 @@ int natsl_short_conv_bwd(const void* x, const void* weight, const void* bias, co
 int natsl_row_norm_fwd(const void* x, const void* weight, void* y, int64_t rows, int D, float eps, int l2, int dtype,
                        int w_dtype, natsl_stream_t stream);
 
+/* Backward of natsl_row_norm_fwd: dx [rows, D] in `dtype`; dweight [D] f32 when a weight is given (summed over the rows in a
+ * fixed order: partial sums per 128 rows in the workspace, then one reduction; no weight: workspace may be NULL).
+ * Replaces the backward of the reference's RMSNorm / l2norm modules (fla.modules, as used at
+ * src/nats/layers/natsl_attn_gdn.py:275-330). */
+size_t natsl_row_norm_bwd_workspace_bytes(int64_t rows, int D);
+int natsl_row_norm_bwd(const void* x, const void* weight, const void* dy, void* dx, float* dweight, void* workspace,
+                       size_t workspace_bytes, int64_t rows, int D, float eps, int l2, int dtype, int w_dtype,
+                       natsl_stream_t stream);
+
 /* Decode: T tokens that continue the current (incomplete) selector block of N cached sequences, token by
  * token.  Per token: S *= e^g; d = beta (v - S^T k); S += k d^T; o = scale S^T q (k, q L2-normalised with
  * NATSL_QK_L2NORM).  Only the first min(T, block - n_tokens_in_block) tokens are processed.  If they

@@ -45,6 +45,8 @@ _SIGNATURES = {
     "natsl_linear_chunk_bwd": (c_int, [c_int] + [c_void_p] * 9 + [c_int] + [c_void_p] * 12 + [c_int] * 8 + [c_float, c_int, c_int, c_void_p, c_int, c_int, c_void_p]),
     "natsl_norm_gate_bwd_workspace_bytes": (c_size_t, [c_int64, c_int]),
     "natsl_norm_gate_bwd": (c_int, [c_void_p] * 14 + [c_size_t, c_int64, c_int, c_int, c_float, c_int, c_void_p]),
+    "natsl_row_norm_bwd_workspace_bytes": (c_size_t, [c_int64, c_int]),
+    "natsl_row_norm_bwd": (c_int, [c_void_p] * 6 + [c_size_t, c_int64, c_int, c_float, c_int, c_int, c_int, c_void_p]),
     "natsl_short_conv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_void_p]),
     "natsl_short_conv_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

@@ -289,6 +289,96 @@ __global__ __launch_bounds__(256) void row_norm_kernel(const void* x, const void
   }
 }
 
+// Backward of row_norm_kernel: with n = x r (r = rsqrt(mean x^2 + eps), or rsqrt(sum x^2 + eps) for the L2 form) and
+// a = dy w:  dx = r (a - n mean(a n))  (L2: the sum instead of the mean),  dw = sum over rows of dy n.  A workgroup takes ROWS
+// consecutive rows; the lane groups' shares of dw are added in a fixed order through LDS and leave as one partial row per
+// workgroup (part[workgroup][D]), which row_norm_wgrad_reduce_kernel adds up.
+template <int LANES, int PER, bool F32>
+__global__ __launch_bounds__(256) void row_norm_bwd_kernel(const void* x, const void* weight, const void* dy, void* dx, float* part,
+                                                           const long long rows, const int rows_per_wg, const float eps, const int l2,
+                                                           const bool w_f32) {
+  constexpr int D = LANES * PER * 8, G = 256 / LANES;
+  __shared__ float acc_s[G][D];
+  const int grp = threadIdx.x / LANES, seg = threadIdx.x % LANES;
+  float w[PER][8], dw[PER][8];
+#pragma unroll
+  for (int u = 0; u < PER; ++u)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      w[u][j] = weight ? ld1(weight, w_f32, (u * LANES + seg) * 8 + j) : 1.f;
+      dw[u][j] = 0.f;
+    }
+  const long long first = (long long)blockIdx.x * rows_per_wg;
+  for (int it = 0; it * G < rows_per_wg; ++it) {
+    const long long row = first + it * G + grp;
+    if (it * G + grp >= rows_per_wg || row >= rows) continue;   // (a lane group leaves as a whole)
+    float v[PER][8], d[PER][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      load8<F32>(x, (size_t)row * D + (u * LANES + seg) * 8, v[u]);
+      load8<F32>(dy, (size_t)row * D + (u * LANES + seg) * 8, d[u]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += v[u][j] * v[u][j];
+    }
+#pragma unroll
+    for (int dd = 1; dd < LANES; dd <<= 1) ss += __shfl_xor(ss, dd);
+    const float rs = rsqrtf((l2 ? ss : ss / D) + eps);
+    float an = 0.f;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[u][j] *= rs;                       // n
+        dw[u][j] += d[u][j] * v[u][j];
+        d[u][j] *= w[u][j];                  // a
+        an += d[u][j] * v[u][j];
+      }
+#pragma unroll
+    for (int dd = 1; dd < LANES; dd <<= 1) an += __shfl_xor(an, dd);
+    const float m = l2 ? an : an / D;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = rs * (d[u][j] - v[u][j] * m);
+      store8<F32>(dx, (size_t)row * D + (u * LANES + seg) * 8, o);
+    }
+  }
+  if (part == nullptr) return;
+#pragma unroll
+  for (int u = 0; u < PER; ++u)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc_s[grp][(u * LANES + seg) * 8 + j] = dw[u][j];
+  __syncthreads();
+  for (int i = threadIdx.x; i < D; i += 256) {
+    float t = 0.f;
+#pragma unroll
+    for (int q = 0; q < G; ++q) t += acc_s[q][i];
+    part[(size_t)blockIdx.x * D + i] = t;
+  }
+}
+
+// out[c] = sum over k of part[k][c] (64 columns x 16 partial-sum slices per workgroup, fixed order)
+__global__ __launch_bounds__(1024) void row_norm_wgrad_reduce_kernel(const float* part, float* out, const int n_part, const int n_col) {
+  __shared__ float sums[16][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + tx;
+  float acc = 0.f;
+  if (i < n_col)
+    for (int k = ty; k < n_part; k += 16) acc += part[(size_t)k * n_col + i];
+  sums[ty][tx] = acc;
+  __syncthreads();
+  if (ty == 0 && i < n_col) {
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t += sums[r][tx];
+    out[i] = t;
+  }
+}
+
+constexpr int RN_BWD_ROWS = 128;   // rows per workgroup of the row norms' backward
+
 }  // namespace natsl
 
 using namespace natsl;
@@ -406,4 +496,50 @@ extern "C" int natsl_row_norm_fwd(const void* x, const void* weight, void* y, in
     default: return fail(NATSL_ERR_UNSUPPORTED, "%s: row width %d not built (32, 64, 96, 128, 192, 256, 384, 512)", what, D);
   }
 #undef NATSL_RN
+}
+
+extern "C" size_t natsl_row_norm_bwd_workspace_bytes(int64_t rows, int D) {
+  if (rows <= 0 || D <= 0) return 0;
+  return (size_t)((rows + RN_BWD_ROWS - 1) / RN_BWD_ROWS) * (size_t)D * sizeof(float);
+}
+
+extern "C" int natsl_row_norm_bwd(const void* x, const void* weight, const void* dy, void* dx, float* dweight, void* workspace,
+                                  size_t workspace_bytes, int64_t rows, int D, float eps, int l2, int dtype, int w_dtype,
+                                  natsl_stream_t stream) {
+  const char* what = "natsl_row_norm_bwd";
+  if (!x || !dy || !dx || (weight && !dweight)) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: activations must be f32 or bf16", what);
+  if (weight && w_dtype != NATSL_BF16 && w_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: weights must be f32 or bf16", what);
+  if (rows <= 0) return NATSL_OK;
+  float* part = nullptr;
+  if (weight) {
+    const size_t need = natsl_row_norm_bwd_workspace_bytes(rows, D);
+    if (!workspace || workspace_bytes < need) return fail(NATSL_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
+    part = reinterpret_cast<float*>(workspace);
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool f32 = dtype == NATSL_F32;
+  const unsigned wgs = (unsigned)((rows + RN_BWD_ROWS - 1) / RN_BWD_ROWS);
+#define NATSL_RNB(L, P)                                                                                                         \
+  if (f32) hipLaunchKernelGGL((row_norm_bwd_kernel<L, P, true>), dim3(wgs), dim3(256), 0, s, x, weight, dy, dx, part,            \
+                              (long long)rows, RN_BWD_ROWS, eps, l2, w_dtype == NATSL_F32);                                      \
+  else hipLaunchKernelGGL((row_norm_bwd_kernel<L, P, false>), dim3(wgs), dim3(256), 0, s, x, weight, dy, dx, part,               \
+                          (long long)rows, RN_BWD_ROWS, eps, l2, w_dtype == NATSL_F32);                                          \
+  break;
+  switch (D) {
+    case 32: NATSL_RNB(4, 1)
+    case 64: NATSL_RNB(8, 1)
+    case 96: NATSL_RNB(4, 3)
+    case 128: NATSL_RNB(16, 1)
+    case 192: NATSL_RNB(8, 3)
+    case 256: NATSL_RNB(32, 1)
+    case 384: NATSL_RNB(16, 3)
+    case 512: NATSL_RNB(64, 1)
+    default: return fail(NATSL_ERR_UNSUPPORTED, "%s: row width %d not built (32, 64, 96, 128, 192, 256, 384, 512)", what, D);
+  }
+#undef NATSL_RNB
+  int rc = check_launch(what);
+  if (rc != NATSL_OK || !weight) return rc;
+  hipLaunchKernelGGL(row_norm_wgrad_reduce_kernel, dim3((unsigned)((D + 63) / 64)), dim3(1024), 0, s, part, dweight, (int)wgs, D);
+  return check_launch(what);
 }

@@ -46,7 +46,7 @@ def _row_norm_fwd(x, weight, eps, l2):
 
 
 class _RowNorm(torch.autograd.Function):
-    """The HIP forward with the gradients of the same formula evaluated as fp32 torch operations."""
+    """The HIP forward and backward (natsl_row_norm_fwd / natsl_row_norm_bwd)."""
 
     @staticmethod
     def forward(ctx, x, weight, eps, l2):
@@ -57,12 +57,21 @@ class _RowNorm(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, weight = ctx.saved_tensors
-        with torch.enable_grad():
-            xf = x.detach().float().requires_grad_(True)
-            wf = None if weight is None else weight.detach().float().requires_grad_(True)
-            y = _row_norm_torch(xf, wf, ctx.eps, ctx.l2)
-            grads = torch.autograd.grad(y, (xf,) if wf is None else (xf, wf), dy.float())
-        return grads[0].to(x.dtype), (None if wf is None else grads[1].to(weight.dtype)), None, None
+        D = x.shape[-1]
+        xc, dyc = x.detach().contiguous(), dy.detach().to(x.dtype).contiguous()
+        w = None if weight is None else weight.detach().contiguous()
+        if w is not None and w.dtype not in (torch.float32, torch.bfloat16):
+            w = w.float()
+        rows = xc.numel() // D
+        L = _capi.lib()
+        dx = torch.empty_like(xc)
+        dw = None if w is None else torch.empty(D, dtype=torch.float32, device=xc.device)
+        ws = None if w is None else torch.empty(L.natsl_row_norm_bwd_workspace_bytes(rows, D), dtype=torch.uint8, device=xc.device)
+        rc = L.natsl_row_norm_bwd(_capi.ptr(xc), _capi.ptr(w), _capi.ptr(dyc), _capi.ptr(dx), _capi.ptr(dw), _capi.ptr(ws),
+                                  0 if ws is None else ws.numel(), rows, D, float(ctx.eps), int(ctx.l2), _capi.dtype_code(xc.dtype),
+                                  _capi.dtype_code(w.dtype) if w is not None else _capi.F32, _capi.stream_ptr(xc.device))
+        _capi.check(rc, "natsl_row_norm_bwd")
+        return dx, (None if w is None else dw.to(weight.dtype)), None, None
 
 
 def row_norm(x, weight, eps: float, l2: bool):

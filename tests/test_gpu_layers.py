@@ -276,6 +276,23 @@ def test_row_norms(D, dtype):
     tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
     for y, r in ((y1, r1), (y2, r2)):
         assert y.dtype == dtype and bool(((y.float().cpu() - r).abs() <= tol * r.abs() + 1e-6).all())
+    # backward (natsl_row_norm_bwd) against fp64 autograd through the same formulas; 770 rows cross the partial-sum reduction
+    dy1, dy2 = (torch.randn(x.shape, generator=g).to(dtype) for _ in range(2))
     xd = x.to(DEV).requires_grad_(True)
-    (rms(xd).float().sum() + l2(xd).float().pow(2).sum()).backward()
-    assert xd.grad is not None and bool(torch.isfinite(xd.grad).all()) and rms.weight.grad is not None
+    (rms(xd).float() * dy1.to(DEV).float()).sum().backward()
+    g_rms, g_w = xd.grad.clone(), rms.weight.grad.clone()
+    xd.grad = None
+    (l2(xd).float() * dy2.to(DEV).float()).sum().backward()
+    g_l2 = xd.grad.clone()
+    x64, w64 = x.double().requires_grad_(True), rms.weight.detach().double().cpu().requires_grad_(True)
+    ((x64 * torch.rsqrt(x64.pow(2).mean(-1, keepdim=True) + 1e-5) * w64) * dy1.double()).sum().backward()
+    r_rms, r_w = x64.grad.clone(), w64.grad.clone()
+    x64.grad = None
+    ((x64 * torch.rsqrt(x64.pow(2).sum(-1, keepdim=True) + 1e-6)) * dy2.double()).sum().backward()
+    r_l2 = x64.grad.clone()
+    for name, got, ref in (('dx (rms)', g_rms, r_rms), ('dweight', g_w, r_w), ('dx (l2)', g_l2, r_l2)):
+        got = got.double().cpu()
+        err = (got - ref).abs()
+        assert bool((err <= tol * ref.abs() + 2e-3 * float(ref.abs().max()) * (1 if dtype == torch.bfloat16 else 1e-3)).all()), \
+            f"{name}: max-abs {float(err.max()):.3e}"
+        assert rel_l2(got, ref) <= (5e-3 if dtype == torch.bfloat16 else 1e-5), f"{name}: rel-L2 {rel_l2(got, ref):.3e}"
