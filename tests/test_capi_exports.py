@@ -73,3 +73,15 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src.replace("no CPU fallback", ""), f"{f} mentions the oracle"
+
+
+def test_backward_entry_rejects_what_is_not_built():
+    """Argument errors come back as codes from the host, before any launch."""
+    import ctypes
+    from neuralattentionsearchlinear_amd import _capi
+    L = _capi.lib()
+    p = ctypes.c_void_p(256)
+    args = lambda K, V, block: (1, p, p, p, p, p, p, None, p, p, 1, p, p, p, p, p, p, p, p, p, None, p, p, 1, 256, 4, 4, K, V, 256 // block, block,
+                                0.1, 7, 1, None, 0, 0, None)
+    assert L.natsl_linear_chunk_bwd(*args(96, 64, 64)) == -2 and b"K=96" in L.natsl_last_error()
+    assert L.natsl_linear_chunk_bwd(*args(128, 48, 64)) == -2 and b"V=48" in L.natsl_last_error()

@@ -76,18 +76,6 @@ def test_linear_branch_backward(case, which):
     _check(out, ref, kind, h0)
 
 
-def test_backward_entry_rejects_what_is_not_built():
-    """Argument errors come back as codes from the host, before any launch."""
-    import ctypes
-    from neuralattentionsearchlinear_amd import _capi
-    L = _capi.lib()
-    p = ctypes.c_void_p(256)
-    args = lambda K, V, block: (1, p, p, p, p, p, p, None, p, p, 1, p, p, p, p, p, p, p, p, p, None, p, p, 1, 256, 4, 4, K, V, 256 // block, block,
-                                0.1, 7, 1, None, 0, 0, None)
-    assert L.natsl_linear_chunk_bwd(*args(96, 64, 64)) == -2 and b"K=96" in L.natsl_last_error()
-    assert L.natsl_linear_chunk_bwd(*args(128, 48, 64)) == -2 and b"V=48" in L.natsl_last_error()
-
-
 @pytest.mark.parametrize("kind", ['gdn', 'mamba'])
 def test_packed_sequences_equal_separate_calls(kind):
     """One call over packed sequences gives, bit for bit, what one call per sequence gives (own initial state, own
