@@ -4,7 +4,8 @@ same method against the same oracle.
 
 Tolerance: rel-L2 5e-3 and max-abs 2e-2 of the reference's largest magnitude for dq, dk, dv, dh0; rel-L2 1e-2 for the
 per-token scalars dg and dbeta and for the selector's gate gradient (sums of large terms of both signs over bf16-rounded
-intermediates)."""
+intermediates: the kernels round where the reference's do -- h, dh, v_new, dv are kept in the input dtype at
+src/nats/ops/common/chunk_delta_h.py:681, 693, 775, 785)."""
 import pytest
 import torch
 import torch.nn.functional as F
