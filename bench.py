@@ -43,6 +43,12 @@ LINEAR_BACKWARD_WORKLOADS = {
     "gdn_bwd_B8_T4096_H6_K128_V256_p25": dict(B=8, T=4096, H=6, K=128, V=256, p_attn=0.25, block=64),
     "mamba_bwd_B4_T8192_H32_N128_d64_p25": dict(B=4, T=8192, H=32, K=128, V=64, p_attn=0.25, block=256, kind="mamba"),
 }
+# a whole Gated-DeltaNet layer at the published 340M geometry (hidden 1024, 6 heads of 128 / 256, attention view 12 heads of
+# 64 / 128): forward, or forward + backward; not the headline metric
+LAYER_WORKLOADS = {
+    "layer_gdn_340M_B8_T4096_fwd": dict(B=8, T=4096, train=False),
+    "layer_gdn_340M_B8_T4096_train": dict(B=8, T=4096, train=True),
+}
 PEAK_BF16_MFMA_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 
@@ -362,12 +368,51 @@ def bench_linear_bwd(args):
                       note="whole step incl. the forward re-run and the host-side glue"))))
 
 
+def bench_layer(args):
+    """NeuralAttentionSearchLinearAttnGDN (random weights, the selector free to choose) on random hidden states: the
+    projections are torch GEMMs, everything else this package's kernels.  'train' = forward + backward of a scalar loss."""
+    import torch
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd.natsl_attn_gdn import NeuralAttentionSearchLinearAttnGDN
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _capi.lib()
+    w = LAYER_WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    layer = NeuralAttentionSearchLinearAttnGDN(hidden_size=1024, expand_v=2, head_dim=128, num_heads=6, num_attn_heads=12, nats_block_size=64,
+                                               ops_for_incomplete_chunks='all', decay_for_non_gdn_blocks=True, norm_eps=1e-6)
+    layer = layer.to(dev).to(torch.bfloat16)
+    layer.train(w["train"])
+    x = torch.randn(w["B"], w["T"], 1024, device=dev).bfloat16().requires_grad_(w["train"])
+
+    def step():
+        if w["train"]:
+            layer(x)[0].float().pow(2).mean().backward()
+        else:
+            with torch.no_grad():
+                layer(x)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    print(json.dumps(dict(
+        metric="GDN layer (340M geometry) " + ("training step" if w["train"] else "forward") + " tokens/sec bf16", value=w["B"] * w["T"] / (ms * 1e-3),
+        unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak",
+        vs_baseline=None, dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS) + sorted(LINEAR_BACKWARD_WORKLOADS))
+    ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS) + sorted(LINEAR_BACKWARD_WORKLOADS) + sorted(LAYER_WORKLOADS))
     ap.add_argument("--prewarm-ms", type=float, default=300.0,
                     help="milliseconds of untimed load before the warm-up steps, to let the GPU clocks settle (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -393,6 +438,8 @@ def main():
         return bench_softmax_bwd(args)
     if args.workload in LINEAR_BACKWARD_WORKLOADS:
         return bench_linear_bwd(args)
+    if args.workload in LAYER_WORKLOADS:
+        return bench_layer(args)
     import torch
     from neuralattentionsearchlinear_amd import _capi, _mixed_common, nats_util
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn

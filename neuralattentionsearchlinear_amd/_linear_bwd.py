@@ -1,15 +1,18 @@
 """Backward of the linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for training.
 
-linear_chunk_backward runs the HIP kernels of csrc/natsl_linear_bwd.hip; linear_chunk_backward_torch is the same computation
-as fp32 torch operations on the GPU (for the shapes the kernels are not built for, and as the plain statement of the method),
-organised so that nothing but one short loop over the chunks is sequential.  It is the same chunked algorithm the forward kernels implement (csrc/natsl_linear.hip), so the gradients belong
-to the forward that was actually computed, up to its bf16 rounding.  It replaces chunk_gated_delta_rule_nats_bwd
-(src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart (src/nats/ops/mamba/chunk.py:112-260) in function.
+linear_chunk_backward_hip is the product path: the forward once more with its per-chunk state and v_new outputs, then
+natsl_linear_chunk_bwd (csrc/natsl_linear_bwd.hip: a reverse scan over the chunks and a per-chunk gradient kernel), and the
+few lines of host glue around them (block sums of g, the per-block sums of the gate gradients).  It replaces
+chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart
+(src/nats/ops/mamba/chunk.py:112-260) in function.  linear_chunk_backward_torch is the same method as fp32 torch operations
+on the GPU, for the shapes the kernels are not built for (V not a multiple of 64) and as its plain statement; both follow the
+chunked algorithm of the forward kernels (csrc/natsl_linear.hip), so the gradients belong to the forward that was actually
+computed, up to its bf16 rounding.
 
 Per 64-token chunk c with entering state S_c (notation of the forward):
     X = v - W S_c,  v_new = T X,  o = Q~ S_c + P v_new,  S_{c+1} = e^{gamma_last} S_c + gate * K~^T v_new
 (a block that is not typed linear ends in S = f * S_blockstart + gate_off * K~^T v_new instead, f = e^{sum of g over the
-block} or 1).  Three steps:
+block} or 1).  Three steps (the torch formulation; the kernels split the work the same way):
   1. the states S_c of all chunks: the forward kernel run once more with its per-chunk state output (bf16, as the forward
      used them);
   2. the state gradients: the reverse recurrence

@@ -32,6 +32,9 @@
 //                        e^{sum g} when decay is on), which is all the reference's carry logic
 //                        (src/nats/ops/utils/cumsum.py:95-133) amounts to.
 //
+// For a backward the scan can also store the state that enters every chunk (the bf16 B operands it forms anyway, [chunk][H][V][K])
+// and the delta rule's v_new of every token; natsl_linear_bwd.hip reads them, and TmB from the workspace.
+//
 // The Mamba form has no solve: its prep is mamba_scale_kernel (the scale vectors only; q and k are not read), and the
 // scan forms P itself, in registers, from the k and q tiles of the stage.
 #include "natsl_device.h"
