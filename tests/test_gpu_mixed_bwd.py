@@ -175,3 +175,32 @@ def test_layer_training_step(kind, geometry):
         rl_, top = rel_l2(p_.grad.float(), r_), float(r_.abs().max())
         assert rl_ <= 2e-2 and max_abs(p_.grad.float(), r_) <= 5e-2 * max(top, 1e-3), f"{name}: grad rel-L2 {rl_:.3e}"
     assert xd.grad is not None and bool(torch.isfinite(xd.grad).all())
+
+
+def test_config0_backward_fp32_tensors():
+    """The smallest configuration (B1 T256 H2 K=V=64, fp32 tensors) through loss.backward(): gradients come back in fp32,
+    computed on bf16 copies like the forward, and match the oracle on the rounded inputs."""
+    from neuralattentionsearchlinear_amd import nats_util
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    torch.manual_seed(0)
+    B, T, H, D, block = 1, 256, 2, 64, 64
+    q, k, v = (torch.randn(B, T, H, D).bfloat16().float() for _ in range(3))
+    beta = torch.sigmoid(torch.randn(B, T, H)).bfloat16().float()
+    g = -F.softplus(torch.randn(B, T, H))
+    ty = make_types(B, T // block, H, 0.4, 3, torch.float32)
+    do_l, do_a = (torch.randn(B, T, H, D).bfloat16().float() for _ in range(2))
+    rl = LB.linear_branch_bwd('gdn', q, k, v, g, beta, ty[..., 1], D ** -0.5, do_l, None, None, block, True, True, True, False)
+    dq_a, dk_a, dv_a, _, _ = SB.softmax_branch_bwd(q, k, v, ty, do_a, D ** -0.5, block, True, with_magnitude=True)
+    leaf = lambda t: t.to(DEV).requires_grad_(True)
+    qa, ka, va, ql, kl, vl, gd, bd = (leaf(t) for t in (q, k, v, q, k, v, g, beta))
+    nb = ty.to(torch.int32).sum(1).to(DEV)
+    o_l, o_a, _ = nats_mixed_attn_gdn(qa, ka, va, ql, kl, vl, None, gd, bd, ty.to(DEV), nb, nats_block_size=block,
+                                      ops_for_incomplete_chunks='all', decay_for_non_gdn_blocks=True)
+    assert o_l.dtype == torch.float32
+    ((o_l * do_l.to(DEV)).sum() + (o_a * do_a.to(DEV)).sum()).backward()
+    torch.cuda.synchronize()
+    for t in (qa, ka, va, ql, kl, vl, gd, bd):
+        assert t.grad is not None and t.grad.dtype == torch.float32
+    _close(ql.grad, rl['dq'], "dq_lattn"); _close(kl.grad, rl['dk'], "dk_lattn"); _close(vl.grad, rl['dv'], "dv_lattn")
+    _close(gd.grad, rl['dg'], "dg", 1e-2); _close(bd.grad, rl['dbeta'], "dbeta", 1e-2)
+    _close(qa.grad, dq_a, "dq_attn"); _close(ka.grad, dk_a, "dk_attn"); _close(va.grad, dv_a, "dv_attn")
