@@ -40,7 +40,8 @@ BACKWARD_WORKLOADS = {
 # backward of the Gated DeltaNet branch at the headline shape (training); not the headline metric
 LINEAR_BACKWARD_WORKLOADS = {
     "gdn_bwd_B8_T8192_H16_d128_p25": dict(B=8, T=8192, H=16, K=128, V=128, p_attn=0.25, block=64),
-    "gdn_bwd_B8_T4096_H6_K128_V256_p25": dict(B=8, T=4096, H=6, K=128, V=256, p_attn=0.25, block=64),
+    "gdn_bwd_B8_T4096_H6_K128_V256_p25": dict(B=8, T=4096, H=6, K=128, V=256, p_attn=0.25, block=64),     # the 340M geometry
+    "gdn_bwd_B8_T4096_H6_K192_V384_p25": dict(B=8, T=4096, H=6, K=192, V=384, p_attn=0.25, block=64),     # the 760M geometry
     "mamba_bwd_B4_T8192_H32_N128_d64_p25": dict(B=4, T=8192, H=32, K=128, V=64, p_attn=0.25, block=256, kind="mamba"),
 }
 # a whole Gated-DeltaNet layer at the published 340M geometry (hidden 1024, 6 heads of 128 / 256, attention view 12 heads of
