@@ -81,7 +81,7 @@ NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
 // prep
 // =============================================================================================
 template <int DK, bool DELTA>
-__global__ __launch_bounds__(256) void linear_prep_kernel(const LinearParams p) {
+__global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams p) {
   constexpr int KP = DK + 8;   // bf16 row pitch
   constexpr int KL = DK / 32;  // 16-byte loads per thread per tile
   // The 64x64 fp32 matrices of the solve are kept as their ten lower 16x16 blocks, block (i, k) at
