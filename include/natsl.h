@@ -38,7 +38,8 @@ enum natsl_status {
 enum natsl_flags {
   NATSL_DECAY_NON_LINEAR = 1, /* decay_for_non_gdn_blocks / decay_for_non_mamba_blocks */
   NATSL_QK_L2NORM = 2,        /* lattn_use_qk_l2norm_in_kernel */
-  NATSL_INTRA_CHUNK = 4       /* the linear op also scores its own incomplete block ('all', 'gated_delta_net', 'mamba') */
+  NATSL_INTRA_CHUNK = 4,      /* the linear op also scores its own incomplete block ('all', 'gated_delta_net', 'mamba') */
+  NATSL_QUERY_ONLY = 8        /* recurrent entries: outputs from the decayed block-start state, nothing updated ('attn') */
 };
 
 /* One row per packed sequence (cu_seqlens / cu_seqlens_nats of the reference, plus prefix
@@ -258,6 +259,10 @@ int natsl_row_norm_bwd(const void* x, const void* weight, const void* dy, void* 
  * g_cumsum fp32 [N,H] or NULL (0): sum of g over the tokens already in the block; h0 fp32 [N,H,K,V] or NULL
  * (zeros); h_block_start fp32 [N,H,K,V] in/out; ht fp32 [N,H,K,V] or NULL; types [N,1,HN,2] (op 1 = linear);
  * n_tokens_in_block int32 [N] or NULL (then the scalar is used for every sequence).  K in {64, 128, 192}, V % 16 == 0.
+ * With NATSL_QUERY_ONLY (the mode in which the linear operator skips the incomplete block, ops_for_incomplete_chunks = 'attn'):
+ * o_t = scale q_t^T (e^(g_cumsum + g_1 + .. + g_t) h_block_start), no state is read from h0 or written; k, v, beta may be NULL
+ * (the reference's branch without UPDATE_HS_FOR_EACH_ITER, fused_recurrent.py:156-201, as called for one-token steps at
+ * src/nats/ops/mixed_ops/mixed_attn_gdn.py:510-527).
  * Replaces fused_recurrent_gated_delta_rule_nats_fwd, src/nats/ops/gated_delta_rule/fused_recurrent.py:360-470
  * (kernel :28-358) as called with update_hs_for_each_iter=True at
  * src/nats/ops/mixed_ops/mixed_attn_gdn.py:485-503. */

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libnatsl.so")
 
 F32, BF16 = 0, 1
-DECAY_NON_LINEAR, QK_L2NORM, INTRA_CHUNK = 1, 2, 4
+DECAY_NON_LINEAR, QK_L2NORM, INTRA_CHUNK, QUERY_ONLY = 1, 2, 4, 8
 
 _lib = None
 

@@ -105,10 +105,15 @@ class NAtSLayerCache:
             raise NotImplementedError("a mask for several new tokens is built only while they stay inside the current block")
         if self.op_for_incomplete_chunk == 'gated_delta_net':
             raise NotImplementedError("several new tokens per step are not built for ops_for_incomplete_chunks='gated_delta_net'")
-        dev = self.valid_attn_tokens.device
-        B, _, HN = self.valid_attn_tokens.shape
-        past = self.valid_attn_tokens[:, :nmax].repeat_interleave(bs, 1).transpose(1, 2)          # [B, HN, nmax*bs]
-        past = past.unsqueeze(-2).expand(B, HN, n_data, nmax * bs)
+        if self.valid_attn_tokens is None:
+            # an empty cache (a first input shorter than one block): no kept blocks yet, the keys are the new tokens
+            dev, (B, _, HN, _) = nats_block_types.device, nats_block_types.shape
+            past = torch.zeros(B, HN, n_data, 0, dtype=torch.bool, device=dev)
+        else:
+            dev = self.valid_attn_tokens.device
+            B, _, HN = self.valid_attn_tokens.shape
+            past = self.valid_attn_tokens[:, :nmax].repeat_interleave(bs, 1).transpose(1, 2)          # [B, HN, nmax*bs]
+            past = past.unsqueeze(-2).expand(B, HN, n_data, nmax * bs)
         cur = torch.ones(n_data, n_in + n_data, dtype=torch.bool, device=dev).tril_(n_in) if compute_incomplete_chunk \
             else torch.zeros(n_data, n_in + n_data, dtype=torch.bool, device=dev)
         return torch.cat([past, cur.view(1, 1, n_data, -1).expand(B, HN, -1, -1)], dim=-1)

@@ -37,6 +37,7 @@ struct RecurrentParams {
   const void* types; int types_dtype; const int32_t* n_in_block;
   int N, T, H, HN, V, block, dtype;
   float scale; int decay, l2norm, n_in_block_scalar;
+  int query_only;   // outputs from the decayed block-start state, no state update (the 'attn' mode of decode)
 };
 
 // DELTA = false is the Mamba form (src/nats/ops/mamba/fused_recurrent.py:150-178): S += k v^T, no beta, no norms.
@@ -60,6 +61,40 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(const RecurrentParam
   float gcum = p.g_cumsum ? p.g_cumsum[nh] : 0.f;
   const int n_in = p.n_in_block ? p.n_in_block[n] : p.n_in_block_scalar;
   const int n_tok = min(p.T, p.block - n_in);  // fused_recurrent.py:144
+  if (p.query_only) {
+    // The mode in which the linear operator does not run on the incomplete block: a token reads the state that entered
+    // the block, decayed by the block's g up to and including itself (what the chunked forward without its intra-chunk
+    // term gives, and what the reference's UPDATE_HS_FOR_EACH_ITER = False branch gives for a one-token step,
+    // fused_recurrent.py:156-201 as called at mixed_attn_gdn.py:510-527); nothing is written back.
+    const float e0 = __expf(gcum);
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[r] = Scur[r] * e0;
+    for (int t = 0; t < n_tok; ++t) {
+      const size_t tok = (size_t)n * p.T + t;
+      float qq[R];
+      float sq = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        qq[r] = ld_any(p.q, p.dtype, (tok * p.H + h) * DK + kq * R + r);
+        sq += qq[r] * qq[r];
+      }
+      float rq = 1.f;
+      if (DELTA && p.l2norm) {
+        sq += __shfl_xor(sq, 16); sq += __shfl_xor(sq, 32);
+        rq = 1.f / sqrtf(sq + 1e-6f);
+      }
+      const float eg = __expf(p.g[tok * p.H + h]);
+      float hq = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] *= eg;
+        hq += S[r] * qq[r];
+      }
+      hq += __shfl_xor(hq, 16); hq += __shfl_xor(hq, 32);
+      if (kq == 0) st_any(p.o, p.dtype, (tok * p.H + h) * p.V + vc, hq * rq * p.scale);
+    }
+    return;
+  }
 
   for (int t = 0; t < n_tok; ++t) {
     const size_t tok = (size_t)n * p.T + t;
@@ -355,7 +390,9 @@ static int recurrent_fwd(bool delta, const char* what, const void* q, const void
                          const void* types, int types_dtype, const int32_t* n_tokens_in_block, int n_tokens_in_block_scalar,
                          int N, int T, int H, int HN, int K, int V, int block, float scale, int flags, int dtype,
                          natsl_stream_t stream) {
-  if (!q || !k || !v || !g || (delta && !beta) || !h_block_start || !o || !types) return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
+  const bool query_only = (flags & NATSL_QUERY_ONLY) != 0;
+  if (!q || !g || !h_block_start || !o || !types || (!query_only && (!k || !v || (delta && !beta))))
+    return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16 && dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: tensors must be f32 or bf16", what);
   if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
   if (N <= 0 || T <= 0 || H <= 0 || HN <= 0 || block <= 0) return fail(NATSL_ERR_INVALID, "%s: non-positive dimension", what);
@@ -368,7 +405,7 @@ static int recurrent_fwd(bool delta, const char* what, const void* q, const void
   p.q = q; p.k = k; p.v = v; p.g = g; p.g_cumsum = g_cumsum; p.beta = beta; p.h0 = h0; p.hcur = h_block_start; p.o = o; p.ht = ht;
   p.types = types; p.types_dtype = types_dtype; p.n_in_block = n_tokens_in_block; p.n_in_block_scalar = n_tokens_in_block_scalar;
   p.N = N; p.T = T; p.H = H; p.HN = HN; p.V = V; p.block = block; p.dtype = dtype; p.scale = scale;
-  p.decay = (flags & NATSL_DECAY_NON_LINEAR) != 0; p.l2norm = (flags & NATSL_QK_L2NORM) != 0;
+  p.decay = (flags & NATSL_DECAY_NON_LINEAR) != 0; p.l2norm = (flags & NATSL_QK_L2NORM) != 0; p.query_only = query_only ? 1 : 0;
   const dim3 grid(cdiv(V, 64), N * H);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (K == 128 && delta) hipLaunchKernelGGL((gdn_recurrent_kernel<128, true>), grid, dim3(256), 0, s, p);

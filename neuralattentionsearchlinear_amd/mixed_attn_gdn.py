@@ -108,14 +108,20 @@ def nats_mixed_attn_gdn_chunk_inference(
 def fused_recurrent_gated_delta_rule_nats_fwd(q, k, v, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block,
                                               nats_block_size, scale, initial_state, initial_state_in_current_block,
                                               output_final_state=True, use_qk_l2norm_in_kernel=True,
-                                              decay_for_non_gdn_blocks=False):
+                                              decay_for_non_gdn_blocks=False, query_only=False):
     """The gated delta rule token by token on a cached state, for tokens that continue the current selector
     block (src/nats/ops/gated_delta_rule/fused_recurrent.py:360-470 with update_hs_for_each_iter=True).
     -> (o, final_state or None, initial_state_in_current_block); the last is updated in place when the
-    tokens complete the block, as the reference's kernel does."""
+    tokens complete the block, as the reference's kernel does.
+    query_only (the call without update_hs_for_each_iter, for one-token steps): o_t = scale q_t^T (e^(g_cumsum + g_1..t) times
+    initial_state_in_current_block); k, v, beta are not read (may be None) and no state is written."""
     from . import _capi
     N, T, H, K = q.shape
-    V = v.shape[-1]
+    if query_only:
+        if initial_state_in_current_block is None:
+            raise ValueError("query_only needs the state that entered the block")
+        k, v, beta = q, q, q                      # placeholders: the kernel does not read them in this mode
+    V = initial_state_in_current_block.shape[-1] if query_only else v.shape[-1]
     if nats_block_types.shape[1] != 1:
         raise AssertionError("the recurrent form only continues the current selector block: nats_block_types must hold one block")  # :417-419
     HN = nats_block_types.shape[2]
@@ -140,8 +146,9 @@ def fused_recurrent_gated_delta_rule_nats_fwd(q, k, v, g, g_cumsum, beta, nats_b
     else:
         n_ptr, n_scalar = None, int(n_tokens_in_current_block)
     o = torch.empty(N, T, H, V, dtype=q.dtype, device=dev)
-    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
-    flags = (_capi.DECAY_NON_LINEAR if decay_for_non_gdn_blocks else 0) | (_capi.QK_L2NORM if use_qk_l2norm_in_kernel else 0)
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state and not query_only else None
+    flags = (_capi.DECAY_NON_LINEAR if decay_for_non_gdn_blocks else 0) | (_capi.QK_L2NORM if use_qk_l2norm_in_kernel else 0) | \
+            (_capi.QUERY_ONLY if query_only else 0)
     rc = _capi.lib().natsl_gdn_recurrent_fwd(
         _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), _capi.ptr(g_cumsum), _capi.ptr(beta), _capi.ptr(initial_state),
         _capi.ptr(initial_state_in_current_block), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype),
@@ -210,16 +217,24 @@ def nats_mixed_attn_gdn_recurrent(
     of the new queries over the cached keys/values, and the gated delta rule token by token on the cached
     state. -> (o_gated_delta_net, o_attn, final_state, initial_state_in_current_block).
 
-    Built for the modes whose linear operator also runs on the incomplete block ('all', 'gated_delta_net');
-    the reference's 'attn' mode (state advanced in block-sized pieces, :504-589) is not."""
+    'all' / 'gated_delta_net': the linear operator also runs on the incomplete block.  'attn' (:504-589): the new tokens read
+    the state that entered the block (decayed), and the state advances when the block is complete -- here by the same token
+    recurrence over the block's cached k, v, beta, g that the cache hands over with the completing step (the reference does
+    it in parallel form, :529-589: the same state).  Built for a selector block of one 64-token chunk, where it gives what
+    the chunked forward of that mode gives, and for steps that stay inside the block (the layers split longer ones)."""
     if scale_attn is None:
         scale_attn = k_attn.shape[-1] ** -0.5
     if scale_lattn is None:
         scale_lattn = k_lattn.shape[-1] ** -0.5
     strategy = all_incomplete_ops[ops_for_incomplete_chunks]
     if not strategy.gated_delta_net:
-        raise NotImplementedError("the recurrent (decode) operator is built for ops_for_incomplete_chunks 'all' and "
-                                  "'gated_delta_net' only")
+        if nats_block_size != 64:
+            raise NotImplementedError("ops_for_incomplete_chunks='attn' is built for decode with nats_block_size=64 only (with longer "
+                                      "blocks the chunked forward of that mode reads the state at the start of each 64-token chunk)")
+        if torch.is_tensor(n_tokens_in_current_block):
+            raise NotImplementedError("ops_for_incomplete_chunks='attn': n_tokens_in_current_block must be an int")
+        if int(n_tokens_in_current_block) + q_lattn.shape[1] > nats_block_size:
+            raise NotImplementedError("ops_for_incomplete_chunks='attn': a decode step must stay inside the current selector block")
     if cu_seqlens is not None or cu_seqlens_nats is not None:
         raise NotImplementedError("packed sequences are not supported by the recurrent (decode) operator")
     if attn_sw_size is not None or use_g_for_attn:
@@ -229,8 +244,29 @@ def nats_mixed_attn_gdn_recurrent(
         raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
     with torch.no_grad():
         o_attn = masked_attention(q_attn, k_attn, v_attn, attn_msk, scale_attn)
-        o_gdn, final_state, start = fused_recurrent_gated_delta_rule_nats_fwd(
-            q_lattn, k_lattn, v_lattn, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block, nats_block_size,
-            scale_lattn, initial_state_gated_delta, initial_state_gated_delta_chunk_start, output_final_state=True,
-            use_qk_l2norm_in_kernel=lattn_use_qk_l2norm_in_kernel, decay_for_non_gdn_blocks=decay_for_non_gdn_blocks)
+        if strategy.gated_delta_net:
+            o_gdn, final_state, start = fused_recurrent_gated_delta_rule_nats_fwd(
+                q_lattn, k_lattn, v_lattn, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block, nats_block_size,
+                scale_lattn, initial_state_gated_delta, initial_state_gated_delta_chunk_start, output_final_state=True,
+                use_qk_l2norm_in_kernel=lattn_use_qk_l2norm_in_kernel, decay_for_non_gdn_blocks=decay_for_non_gdn_blocks)
+        else:
+            T, n_in = q_lattn.shape[1], int(n_tokens_in_current_block)
+            start = initial_state_gated_delta_chunk_start
+            if start is None:
+                N, _, H, K = q_lattn.shape
+                start = (initial_state_gated_delta.to(torch.float32).clone() if initial_state_gated_delta is not None
+                         else torch.zeros(N, H, K, v_lattn.shape[-1], dtype=torch.float32, device=q_lattn.device))
+            o_gdn, _, _ = fused_recurrent_gated_delta_rule_nats_fwd(
+                q_lattn, None, None, g[:, -T:], g_cumsum, None, nats_block_types, n_in, nats_block_size, scale_lattn, None, start,
+                use_qk_l2norm_in_kernel=lattn_use_qk_l2norm_in_kernel, query_only=True)
+            final_state = start
+            if n_in + T == nats_block_size:
+                # the block is complete: its tokens (handed over by the cache) advance the state, as in the other modes
+                if k_lattn.shape[1] != nats_block_size or g.shape[1] != nats_block_size or beta.shape[1] != nats_block_size:
+                    raise ValueError("ops_for_incomplete_chunks='attn': the step that completes a block needs k, v, g, beta of the "
+                                     f"whole block ({nats_block_size} tokens), got {k_lattn.shape[1]}")
+                _, final_state, start = fused_recurrent_gated_delta_rule_nats_fwd(
+                    k_lattn, k_lattn, v_lattn, g, None, beta, nats_block_types, 0, nats_block_size, scale_lattn, start.clone(), start,
+                    output_final_state=True, use_qk_l2norm_in_kernel=lattn_use_qk_l2norm_in_kernel,
+                    decay_for_non_gdn_blocks=decay_for_non_gdn_blocks)
     return o_gdn, o_attn, final_state, start

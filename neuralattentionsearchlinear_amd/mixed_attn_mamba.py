@@ -99,14 +99,20 @@ def nats_mixed_attn_mamba_chunk_inference(
 
 def fused_recurrent_mamba_nats_fwd(q, k, v, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale,
                                    initial_state, initial_state_in_current_block, output_final_state=True,
-                                   decay_for_non_mamba_blocks=False):
+                                   decay_for_non_mamba_blocks=False, query_only=False):
     """The SSD recurrence token by token on a cached state, for tokens that continue the current selector block
     (src/nats/ops/mamba/fused_recurrent.py with update_hs_for_each_iter=True).
     -> (o, final_state or None, initial_state_in_current_block), the last updated in place when the tokens
-    complete the block."""
+    complete the block.
+    query_only: o_t = scale q_t^T (e^(g_cumsum + g_1..t) times initial_state_in_current_block); k, v are not read (may be
+    None) and no state is written."""
     from . import _capi
     N, T, H, K = q.shape
-    V = v.shape[-1]
+    if query_only:
+        if initial_state_in_current_block is None:
+            raise ValueError("query_only needs the state that entered the block")
+        k, v = q, q                               # placeholders: the kernel does not read them in this mode
+    V = initial_state_in_current_block.shape[-1] if query_only else v.shape[-1]
     if nats_block_types.shape[1] != 1:
         raise AssertionError("the recurrent form only continues the current selector block: nats_block_types must hold one block")
     HN = nats_block_types.shape[2]
@@ -131,8 +137,8 @@ def fused_recurrent_mamba_nats_fwd(q, k, v, g, g_cumsum, nats_block_types, n_tok
     else:
         n_ptr, n_scalar = None, int(n_tokens_in_current_block)
     o = torch.empty(N, T, H, V, dtype=q.dtype, device=dev)
-    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
-    flags = _capi.DECAY_NON_LINEAR if decay_for_non_mamba_blocks else 0
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev) if output_final_state and not query_only else None
+    flags = (_capi.DECAY_NON_LINEAR if decay_for_non_mamba_blocks else 0) | (_capi.QUERY_ONLY if query_only else 0)
     rc = _capi.lib().natsl_mamba_recurrent_fwd(
         _capi.ptr(q), _capi.ptr(k), _capi.ptr(v), _capi.ptr(g), _capi.ptr(g_cumsum), _capi.ptr(initial_state),
         _capi.ptr(initial_state_in_current_block), _capi.ptr(o), _capi.ptr(ht), _capi.ptr(types), _capi.dtype_code(types.dtype),
@@ -163,8 +169,9 @@ def nats_mixed_attn_mamba_recurrent(
 ):
     """Decode step(s) of the Mamba hybrid layer (src/nats/ops/mixed_ops/mixed_attn_mamba.py:460-593).
     -> (o_mamba, o_attn, final_state, initial_state_in_current_block).  As in the reference, scale_lattn
-    defaults to K**-0.5 here.  Built for 'all' and 'mamba' (the linear operator also runs on the incomplete
-    block); the 'attn' mode's block-wise state update (:516-591) is not."""
+    defaults to K**-0.5 here.  'all' / 'mamba': the linear operator also runs on the incomplete block.  'attn' (:516-591): the
+    new tokens read the (decayed) state that entered the block, and the state advances when the block is complete, by the
+    token recurrence over the block's cached k, v, g; built for nats_block_size = 64 and steps that stay inside the block."""
     from .mixed_attn_gdn import masked_attention
     if scale_attn is None:
         scale_attn = k_attn.shape[-1] ** -0.5
@@ -172,7 +179,13 @@ def nats_mixed_attn_mamba_recurrent(
         scale_lattn = k_lattn.shape[-1] ** -0.5
     strategy = all_incomplete_ops[ops_for_incomplete_chunks]
     if not strategy.mamba:
-        raise NotImplementedError("the recurrent (decode) operator is built for ops_for_incomplete_chunks 'all' and 'mamba' only")
+        if nats_block_size != 64:
+            raise NotImplementedError("ops_for_incomplete_chunks='attn' is built for decode with nats_block_size=64 only (with longer "
+                                      "blocks the chunked forward of that mode reads the state at the start of each 64-token chunk)")
+        if torch.is_tensor(n_tokens_in_current_block):
+            raise NotImplementedError("ops_for_incomplete_chunks='attn': n_tokens_in_current_block must be an int")
+        if int(n_tokens_in_current_block) + q_lattn.shape[1] > nats_block_size:
+            raise NotImplementedError("ops_for_incomplete_chunks='attn': a decode step must stay inside the current selector block")
     if cu_seqlens is not None or cu_seqlens_nats is not None:
         raise NotImplementedError("packed sequences are not supported by the recurrent (decode) operator")
     if use_g_for_attn:
@@ -182,8 +195,27 @@ def nats_mixed_attn_mamba_recurrent(
         raise _capi.NatslError("the NAtS-L mixed operator runs on the GPU only (no CPU fallback)")
     with torch.no_grad():
         o_attn = masked_attention(q_attn, k_attn, v_attn, attn_msk, scale_attn)
-        o_mamba, final_state, start = fused_recurrent_mamba_nats_fwd(
-            q_lattn, k_lattn, v_lattn, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale_lattn,
-            initial_state_mamba, initial_state_mamba_chunk_start, output_final_state=True,
-            decay_for_non_mamba_blocks=decay_for_non_mamba_blocks)
+        if strategy.mamba:
+            o_mamba, final_state, start = fused_recurrent_mamba_nats_fwd(
+                q_lattn, k_lattn, v_lattn, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale_lattn,
+                initial_state_mamba, initial_state_mamba_chunk_start, output_final_state=True,
+                decay_for_non_mamba_blocks=decay_for_non_mamba_blocks)
+        else:
+            T, n_in = q_lattn.shape[1], int(n_tokens_in_current_block)
+            start = initial_state_mamba_chunk_start
+            if start is None:
+                N, _, H, K = q_lattn.shape
+                start = (initial_state_mamba.to(torch.float32).clone() if initial_state_mamba is not None
+                         else torch.zeros(N, H, K, v_lattn.shape[-1], dtype=torch.float32, device=q_lattn.device))
+            o_mamba, _, _ = fused_recurrent_mamba_nats_fwd(q_lattn, None, None, g[:, -T:], g_cumsum, nats_block_types, n_in, nats_block_size,
+                                                           scale_lattn, None, start, query_only=True)
+            final_state = start
+            if n_in + T == nats_block_size:
+                # the block is complete: its tokens (handed over by the cache) advance the state, as in the other modes
+                if k_lattn.shape[1] != nats_block_size or g.shape[1] != nats_block_size:
+                    raise ValueError("ops_for_incomplete_chunks='attn': the step that completes a block needs k, v, g of the whole "
+                                     f"block ({nats_block_size} tokens), got {k_lattn.shape[1]}")
+                _, final_state, start = fused_recurrent_mamba_nats_fwd(
+                    k_lattn, k_lattn, v_lattn, g, None, nats_block_types, 0, nats_block_size, scale_lattn, start.clone(), start,
+                    output_final_state=True, decay_for_non_mamba_blocks=decay_for_non_mamba_blocks)
     return o_mamba, o_attn, final_state, start

@@ -3,6 +3,7 @@
 gdn_recurrent   follows src/nats/ops/gated_delta_rule/fused_recurrent.py:28-358 on the path the reference's
                 decode takes (UPDATE_HS_FOR_EACH_ITER, one selector block, src/nats/ops/mixed_ops/
                 mixed_attn_gdn.py:485-503), line by line.
+recurrent_query_only  the decode output of the 'attn' mode (no state update on the incomplete block).
 attn_masked     dense softmax attention under an explicit mask, the scaled_dot_product_attention call at
                 src/nats/ops/mixed_ops/mixed_attn_gdn.py:475-481 with repeat_masks
                 (src/nats/ops/attns/attn_utils.py:3-16).
@@ -59,6 +60,31 @@ def gdn_recurrent(q, k, v, g, g_cumsum, beta, lin_types, n_in_block, h0, h_block
         S = torch.where(is_delta[..., None, None], S, Scur * f[..., None, None])
         Scur = S.clone()
     return o, S, Scur
+
+
+def recurrent_query_only(q, g, g_cumsum, h_block_start, scale, l2norm_qk=True, dtype=torch.float64):
+    """The decode output of the mode in which the linear operator skips the incomplete block (ops_for_incomplete_chunks =
+    'attn'): the kernel's loop without UPDATE_HS_FOR_EACH_ITER (src/nats/ops/gated_delta_rule/fused_recurrent.py:156-201) --
+    per token the state only decays, b_h *= exp(g), and o = b_h^T (scale q^) -- started from the state that entered the
+    block times e^(g_cumsum), which is what the reference's call with g + g_cumsum gives for a one-token step
+    (src/nats/ops/mixed_ops/mixed_attn_gdn.py:510-527).  q [N,T,H,K]; g [N,T,H]; g_cumsum [N,H] or None;
+    h_block_start [N,H,K,V] -> o [N,T,H,V].
+    Pinned in tests/test_oracle_decode.py: fed token by token with the cache's bookkeeping, and the state advanced by
+    gdn_recurrent over a block's tokens once the block is complete, it reproduces the chunked forward without its
+    intra-chunk term (linear_branch.gdn_chunked / mamba_chunked, intra=False) for a selector block of one chunk."""
+    q, g = q.to(dtype), g.to(dtype)
+    N, T, H, K = q.shape
+    S = h_block_start.to(dtype).clone()
+    if g_cumsum is not None:
+        S = S * torch.exp(g_cumsum.to(dtype))[..., None, None]
+    o = torch.zeros(N, T, H, S.shape[-1], dtype=dtype)
+    for t in range(T):
+        qt = q[:, t]
+        if l2norm_qk:
+            qt = qt / torch.sqrt((qt * qt).sum(-1, keepdim=True) + 1e-6)
+        S = S * torch.exp(g[:, t])[..., None, None]
+        o[:, t] = torch.einsum('nhkv,nhk->nhv', S, qt * scale)
+    return o
 
 
 def attn_masked(q, k, v, mask, scale, dtype=torch.float64):

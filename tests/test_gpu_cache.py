@@ -123,14 +123,17 @@ def test_mask_of_the_next_token():
     assert not bool(m[:, :, 0, -1].any()) and bool(m[:, :, 1, -2:].all())
 
 
-@pytest.mark.parametrize("kind,T0,T,geometry", [(k_, a, b, None) for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (64, 130))]
-                         + [('gdn', 200, 270, '760M')])
-def test_layer_generation_matches_whole_forward(kind, T0, T, geometry):
+@pytest.mark.parametrize("kind,T0,T,geometry,ops", [(k_, a, b, None, 'all') for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (64, 130))]
+                         + [('gdn', 200, 270, '760M', 'all'), ('gdn', 30, 140, None, 'all')]
+                         # the mode in which the linear operator skips the incomplete block: its tokens read the state that
+                         # entered the block, and the state advances when the block is complete
+                         + [(k_, a, b, None, 'attn') for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (30, 140))])
+def test_layer_generation_matches_whole_forward(kind, T0, T, geometry, ops):
     """Prefill T0 tokens with a cache, decode up to T token by token (two tokens at a time where the block allows
     it): every output must match the layer's forward over the first T0 tokens resp. the whole sequence at the same
     positions; the selector decisions of the two runs must be identical."""
     from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
-    layer, cfg, w, _ = _layer_case(kind, geometry)
+    layer, cfg, w, _ = _layer_case(kind, geometry, ops)
     layer.layer_idx = 0
     layer = layer.to(DEV).to(torch.bfloat16).eval()
     bs = layer.nats_block_size

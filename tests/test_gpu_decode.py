@@ -175,3 +175,33 @@ def test_mamba_recurrent_against_oracle(K, V, T, n_in, block, decay):
     n_tok = min(T, block - n_in)
     assert_close(o[:, :n_tok].float(), o_ref[:, :n_tok], "o_mamba"); assert_close(o_attn.float(), a_ref, "o_attn")
     assert_close(S, S_ref, "final_state"); assert_close(cur, cur_ref, "block_start_state")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("kind,K,V,T,n_in", [('gdn', 128, 128, 1, 0), ('gdn', 128, 256, 1, 63), ('gdn', 64, 64, 5, 10), ('gdn', 192, 128, 3, 7),
+                                             ('mamba', 128, 64, 1, 33), ('mamba', 64, 128, 4, 60)])
+def test_query_only_outputs_against_oracle(kind, K, V, T, n_in, dtype):
+    """NATSL_QUERY_ONLY (the decode output of ops_for_incomplete_chunks = 'attn'): the decayed block-start state read by the
+    new queries; nothing is written back."""
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import fused_recurrent_gated_delta_rule_nats_fwd
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import fused_recurrent_mamba_nats_fwd
+    N, H, HN, block = 3, 4, 2, 64
+    q, _, _ = make_qkv(N, T, H, K, V, 21, dtype)
+    g, _ = make_gates(N, T, H, 22, dtype)
+    gen = torch.Generator().manual_seed(23)
+    hcur = torch.randn(N, H, K, V, generator=gen) * 0.3
+    gcum = -torch.rand(N, H, generator=gen) * 3
+    ty = make_types(N, 1, HN, 0.5, 24, dtype, force_last=False)
+    scale = K ** -0.5
+    delta = kind == 'gdn'
+    o_ref = D.recurrent_query_only(q.float(), g, gcum, hcur, scale, l2norm_qk=delta)
+    qd, gd, tyd, gcd = _dev(q, g, ty, gcum)
+    hcurd = hcur.to(DEV).clone()
+    if delta:
+        o, S, cur = fused_recurrent_gated_delta_rule_nats_fwd(qd, None, None, gd, gcd, None, tyd, n_in, block, scale, None, hcurd, query_only=True)
+    else:
+        o, S, cur = fused_recurrent_mamba_nats_fwd(qd, None, None, gd, gcd, tyd, n_in, block, scale, None, hcurd, query_only=True)
+    torch.cuda.synchronize()
+    n_tok = min(T, block - n_in)
+    assert_close(o[:, :n_tok].float(), o_ref[:, :n_tok], "o")
+    assert S is None and torch.equal(cur.cpu(), hcur), "query-only must not write a state"

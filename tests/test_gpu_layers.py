@@ -62,19 +62,19 @@ PUBLISHED = {'340M': dict(hidden_size=1024, head_dim=128, num_heads=6, num_attn_
              '760M': dict(hidden_size=1536, head_dim=192, num_heads=6, num_attn_heads=18, norm_eps=1e-6)}
 
 
-def _layer_case(kind, geometry=None):
+def _layer_case(kind, geometry=None, ops='all'):
     torch.manual_seed(0)
     if kind == 'gdn':
         from neuralattentionsearchlinear_amd.natsl_attn_gdn import NeuralAttentionSearchLinearAttnGDN as L
         # the published ratio: attention view = twice as many heads of half the width (K 64 / V 128 vs K 128 / V 256)
         cfg = dict(hidden_size=256, expand_v=2, head_dim=128, num_heads=2, num_attn_heads=4, nats_block_size=64,
-                   ops_for_incomplete_chunks='all', decay_for_non_gdn_blocks=True, norm_eps=1e-5)
+                   ops_for_incomplete_chunks=ops, decay_for_non_gdn_blocks=True, norm_eps=1e-5)
         if geometry is not None:
             cfg.update(PUBLISHED[geometry])
     else:
         from neuralattentionsearchlinear_amd.natsl_attn_mamba2 import NeuralAttentionSearchLinearAttnMamba as L
         cfg = dict(hidden_size=256, expand_v=0.5, head_dim=128, num_heads=4, num_attn_heads=4, nats_block_size=64,
-                   ops_for_incomplete_chunks='all', decay_for_non_mamba_blocks=True, norm_eps=1e-5)
+                   ops_for_incomplete_chunks=ops, decay_for_non_mamba_blocks=True, norm_eps=1e-5)
     layer = L(**cfg)
     with torch.no_grad():
         for n, p_ in layer.named_parameters():

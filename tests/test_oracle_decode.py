@@ -82,3 +82,38 @@ def test_mamba_recurrent_calls_reproduce_token_recurrence():
             gcum = gs if gcum is None else gcum + gs
         t += n
     assert float((torch.cat(outs, 1) - o_ref).abs().max()) < 1e-9 and float((S - S_ref).abs().max()) < 1e-9
+
+
+@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
+def test_attn_mode_decode_reproduces_the_chunked_forward_without_intra_chunk_term(kind):
+    """ops_for_incomplete_chunks = 'attn', selector block = one chunk: every token reads the decayed state that entered its
+    block (recurrent_query_only); when a block is complete the state advances over its tokens (gdn_recurrent /
+    mamba_recurrent, outputs discarded).  Token by token this must give the chunked forward with intra=False."""
+    N, T, H, K, V, block, HN = 2, 200, 2, 16, 8, 64, 1
+    q, k, v = make_qkv(N, T, H, K, V, 13, torch.float32)
+    g, beta = make_gates(N, T, H, 14, torch.float32)
+    ty = make_types(N, -(-T // block), HN, 0.5, 15, force_last=False)
+    delta = kind == 'gdn'
+    scale = K ** -0.5 if delta else 1.0
+    if delta:
+        o_ref, _ = LB.gdn_chunked(q, k, v, g, beta, ty[..., 1], scale, None, block, True, True, torch.float64, False)
+    else:
+        o_ref, _ = LB.mamba_chunked(q, k, v, g, ty[..., 1], scale, None, block, True, torch.float64, False)
+    S = torch.zeros(N, H, K, V, dtype=torch.float64)
+    gcum, outs = None, []
+    for t in range(T):
+        n_in = t % block
+        outs.append(D.recurrent_query_only(q[:, t:t + 1], g[:, t:t + 1], gcum, S, scale, l2norm_qk=delta))
+        gs = g[:, t].double()
+        gcum = gs if gcum is None else gcum + gs
+        if n_in == block - 1:
+            b0 = t + 1 - block
+            blk = ty[:, t // block:t // block + 1, :, 1]
+            if delta:
+                _, S, _ = D.gdn_recurrent(k[:, b0:t + 1], k[:, b0:t + 1], v[:, b0:t + 1], g[:, b0:t + 1], None, beta[:, b0:t + 1], blk, 0, S,
+                                          S, scale, block, True)
+            else:
+                _, S, _ = D.mamba_recurrent(k[:, b0:t + 1], k[:, b0:t + 1], v[:, b0:t + 1], g[:, b0:t + 1], None, blk, 0, S, S, scale, block, True)
+            gcum = None
+    o = torch.cat(outs, 1)
+    assert float((o - o_ref).abs().max()) < 1e-9
