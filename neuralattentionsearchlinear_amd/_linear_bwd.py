@@ -113,15 +113,21 @@ def linear_chunk_forward_torch(kind, q, k, v, g, beta, h0, lin, scale, block, de
     return o, S
 
 
+def hip_backward_is_built(K: int, V: int) -> bool:
+    """The head dims natsl_linear_chunk_bwd is built for."""
+    return K in (64, 128, 192) and V % 64 == 0
+
+
 def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                          dnats_for_invalid_blocks, seqs=None):
+                          dnats_for_invalid_blocks, seqs=None, saved=None):
     """Gradients of the chunked linear branch: -> (dq, dk, dv, dg fp32, dbeta or None, dh0 or None, dnats fp32 [B,NB,HN]).
-    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None; seqs: packed sequences (B = 1) or None.  The HIP kernels
-    (natsl_linear_chunk_bwd) where they are built (K in 64/128/192, V a multiple of 64), else the torch formulation below,
-    one sequence at a time."""
-    if q.shape[-1] in (64, 128, 192) and v.shape[-1] % 64 == 0:
+    types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None; seqs: packed sequences (B = 1) or None; saved: what
+    linear_chunk_fwd(..., chunk_states=True) returned after (o, final_state) on these same inputs, if the caller kept it.  The
+    HIP kernels (natsl_linear_chunk_bwd) where they are built (K in 64/128/192, V a multiple of 64), else the torch formulation
+    below, one sequence at a time."""
+    if hip_backward_is_built(q.shape[-1], v.shape[-1]):
         return linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                                         dnats_for_invalid_blocks, seqs)
+                                         dnats_for_invalid_blocks, seqs, saved)
     if seqs is None:
         return linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
                                            dnats_for_invalid_blocks)
@@ -177,9 +183,9 @@ def _range_sums(x, first, end):
 
 
 def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
-                              dnats_for_invalid_blocks, seqs=None):
-    """The backward as kernels: the forward once more (storing every chunk's entering state and v_new), then the reverse
-    scan and the per-chunk gradients (csrc/natsl_linear_bwd.hip)."""
+                              dnats_for_invalid_blocks, seqs=None, saved=None):
+    """The backward as kernels: the forward once more (storing every chunk's entering state and v_new) unless the caller kept
+    those from its own forward (`saved`), then the reverse scan and the per-chunk gradients (csrc/natsl_linear_bwd.hip)."""
     from . import _capi
     from ._mixed_common import linear_chunk_fwd
     from .nats_util import _seq_args
@@ -199,8 +205,11 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
         gf = g.detach().to(f32).contiguous()
         bb = beta.detach().to(bf16).contiguous() if delta else None
         h0f = None if h0 is None else h0.detach().to(f32).contiguous()
-        _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, seqs,
-                                                   chunk_states=True)
+        if saved is not None:
+            states, v_new, ws = saved
+        else:
+            _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, seqs,
+                                                       chunk_states=True)
         tok0, tok1, ch0, ch1, tok_blk = _block_maps(B, T, block, seqs, dev)
         gsum = _range_sums(gf.view(B * T, H), tok0, tok1).contiguous()                  # [all blocks, H]
         d_states = torch.empty_like(states)

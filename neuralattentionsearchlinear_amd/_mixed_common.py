@@ -23,6 +23,13 @@ TIMING_HOOK = None
 # Both kernels take most of a CU's LDS (127 KiB / 159 KiB), so they never share a CU: when each fills the
 # machine alone, running them side by side gains nothing (measured) and only blurs timings.
 CONCURRENT_BRANCHES = None
+
+# What the differentiable operator keeps from its forward for the linear branch's backward.  True: the state entering every
+# chunk (bf16, K*V per chunk and head), v_new and the prep kernel's workspace (17 KiB per chunk and head) stay in device
+# memory until the backward, which then starts at its reverse scan.  False: only the inputs are kept and the backward runs
+# the forward's two kernels once more, as the reference's backward does
+# (src/nats/ops/gated_delta_rule/chunk.py:170-332 recomputes h).  The gradients are the same bit for bit either way.
+SAVE_CHUNK_STATES = True
 _SCAN_COLUMNS_PER_WG = 16   # state columns of the scan's narrowest workgroup (csrc/natsl_linear.hip)
 
 
@@ -98,9 +105,12 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
                   scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size, attn_sw_size,
                   attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
                   incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
-                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0, return_aux: bool = False):
+                  inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0, return_aux: bool = False,
+                  keep_chunk_states: bool = False):
     """Shared forward of the mixed operators.  With inference=True it also returns the state at the
-    start of the current selector block (4-tuple), as the reference's *_chunk_inference operators do."""
+    start of the current selector block (4-tuple), as the reference's *_chunk_inference operators do.  With return_aux
+    and keep_chunk_states the auxiliary dict also holds what the linear backward would otherwise recompute
+    (`linear_saved`: chunk states, v_new, workspace)."""
     if nats_block_size < CHUNK_SIZE:
         raise AssertionError("nats_block_size must be at least the compute chunk (64)")   # mixed_attn_gdn.py:90
     if nats_block_size % CHUNK_SIZE:
@@ -151,7 +161,8 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
     _mark("linear:start", cur)
     want_start = inference and output_final_state
     res = linear_chunk_fwd(kind, q_lattn, k_lattn, v_lattn, g, beta, initial_state, types, scale_lattn,
-                           nats_block_size, flags, output_final_state, seqs, block_start_state=want_start)
+                           nats_block_size, flags, output_final_state, seqs, block_start_state=want_start,
+                           chunk_states=keep_chunk_states and not want_start)
     o_lin, ht = res[0], res[1]
     _mark("linear:end", cur)
     if side is not cur:
@@ -166,7 +177,8 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
         o_lin, o_attn = o_lin.to(io_dtype), o_attn.to(io_dtype)
     if return_aux:
         aux = dict(q_attn=q_attn, k_attn=k_attn, v_attn=v_attn, q_lattn=q_lattn, k_lattn=k_lattn, v_lattn=v_lattn, beta=beta, g=g,
-                   types=types, lse=_lse, nats_block_indices=r['nats_block_indices'], n_nats_blocks=r['n_nats_blocks'])
+                   types=types, lse=_lse, nats_block_indices=r['nats_block_indices'], n_nats_blocks=r['n_nats_blocks'],
+                   linear_saved=tuple(res[2:5]) if keep_chunk_states and not want_start else None)
         return o_lin, o_attn, ht, aux
     if not inference:
         return o_lin, o_attn, ht
@@ -198,12 +210,15 @@ class _MixedFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, cfg, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types):
+        from ._linear_bwd import hip_backward_is_built
+        keep = bool(SAVE_CHUNK_STATES) and hip_backward_is_built(q_lattn.shape[-1], v_lattn.shape[-1])
         with torch.no_grad():
             o_lin, o_attn, ht, aux = _mixed_forward_impl(
                 cfg['kind'], q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,
                 cfg['scale_attn'], cfg['scale_lattn'], cfg['cu_seqlens'], cfg['cu_seqlens_nats'], cfg['block'], None,
                 cfg['attn_same_block'], cfg['lin_intra'],
-                cfg['output_final_state'], cfg['decay_non_linear'], True, False, cfg['qk_l2norm'], return_aux=True)
+                cfg['output_final_state'], cfg['decay_non_linear'], True, False, cfg['qk_l2norm'], return_aux=True,
+                keep_chunk_states=keep)
         ctx.cfg = cfg
         ctx.in_dtypes = tuple(None if t is None else t.dtype for t in (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
                                                                        initial_state, g, beta, nats_block_types))
@@ -212,6 +227,11 @@ class _MixedFunction(torch.autograd.Function):
                                   'nats_block_indices', 'n_nats_blocks')]
         saved += [o_attn.to(torch.bfloat16), aux['beta'] if aux['beta'] is not None else g.new_zeros(0),
                   initial_state if initial_state is not None else g.new_zeros(0)]
+        ctx.n_linear_saved = 0
+        if aux['linear_saved'] is not None:
+            # (for 'mamba' the second entry is v_lattn itself, saved above already: the same tensor, no second copy)
+            saved += list(aux['linear_saved'])
+            ctx.n_linear_saved = len(aux['linear_saved'])
         ctx.save_for_backward(*saved)
         if ht is None:
             return o_lin, o_attn, None
@@ -222,7 +242,8 @@ class _MixedFunction(torch.autograd.Function):
         from ._linear_bwd import linear_chunk_backward
         from .attns import parallel_attn_nats_bwd
         cfg = ctx.cfg
-        (q_a, k_a, v_a, q_l, k_l, v_l, g, types, lse, idx, nblk, o_attn, beta, h0) = ctx.saved_tensors
+        (q_a, k_a, v_a, q_l, k_l, v_l, g, types, lse, idx, nblk, o_attn, beta, h0) = ctx.saved_tensors[:14]
+        linear_saved = tuple(ctx.saved_tensors[14:]) if ctx.n_linear_saved else None
         beta = beta if beta.numel() else None
         h0 = h0 if ctx.has_h0 else None
         B, NB, HN, _ = types.shape
@@ -239,7 +260,8 @@ class _MixedFunction(torch.autograd.Function):
             do_lin = torch.zeros(*q_l.shape[:3], v_l.shape[-1], dtype=torch.float32, device=q_l.device)
         lin_args = (cfg['scale_lattn'], cfg['block'], cfg['decay_non_linear'], cfg['qk_l2norm'], cfg['lin_intra'])
         dq_l, dk_l, dv_l, dg, dbeta, dh0, dn_lin = linear_chunk_backward(
-            cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, *lin_args, do_lin, dht, cfg['dnats_invalid_linear'], seqs)
+            cfg['kind'], q_l, k_l, v_l, g, beta, h0, types, *lin_args, do_lin, dht, cfg['dnats_invalid_linear'], seqs,
+            saved=linear_saved)
         d_types = torch.stack([dn_attn.float(), dn_lin.float()], -1)
         grads = [dq_a, dk_a, dv_a, dq_l, dk_l, dv_l, dh0, dg, dbeta, d_types]
         grads = [None if (t is None or dt is None) else t.to(dt) for t, dt in zip(grads, ctx.in_dtypes)]

@@ -204,3 +204,52 @@ def test_config0_backward_fp32_tensors():
     _close(ql.grad, rl['dq'], "dq_lattn"); _close(kl.grad, rl['dk'], "dk_lattn"); _close(vl.grad, rl['dv'], "dv_lattn")
     _close(gd.grad, rl['dg'], "dg", 1e-2); _close(bd.grad, rl['dbeta'], "dbeta", 1e-2)
     _close(qa.grad, dq_a, "dq_attn"); _close(ka.grad, dk_a, "dk_attn"); _close(va.grad, dv_a, "dv_attn")
+
+
+@pytest.mark.parametrize("kind,packed", [('gdn', False), ('mamba', False), ('gdn', True)])
+def test_kept_chunk_states_give_the_recomputed_gradients(kind, packed):
+    """_mixed_common.SAVE_CHUNK_STATES: the backward that starts from the forward's kept chunk states, v_new and workspace
+    returns, bit for bit, what the backward that runs the forward's kernels once more returns."""
+    import neuralattentionsearchlinear_amd._mixed_common as MC
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
+    from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
+    B, T, H, HN, K, V, block = (1, 704, 4, 2, 128, 128, 64) if packed else (2, 448, 4, 2, 128, 128, 64)
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = make_qkv(B, T, H, K, V, 21)
+    if kind == 'mamba':
+        q, k = F.normalize(q.float(), dim=-1).bfloat16(), F.normalize(k.float(), dim=-1).bfloat16()
+    g, beta = make_gates(B, T, H, 22)
+    cu = [0, 200, 512, 704] if packed else None
+    nblk = sum(-(-(b - a) // block) for a, b in zip(cu[:-1], cu[1:])) if packed else T // block
+    ty = make_types(B, nblk, HN, 0.4, 23, torch.bfloat16)
+    n = len(cu) - 1 if packed else B
+    init = torch.randn(n, H, K, V, generator=gen) * 0.3
+    do_l, do_a = (torch.randn(B, T, H, V, generator=gen).bfloat16().to(DEV) for _ in range(2))
+    dht = torch.randn(n, H, K, V, generator=gen).to(DEV)
+    kw = dict(cu_seqlens=torch.tensor(cu, dtype=torch.int32, device=DEV)) if packed else {}
+    nb = None if packed else ty.to(torch.int32).sum(1).to(DEV)
+
+    def grads(keep):
+        old, MC.SAVE_CHUNK_STATES = MC.SAVE_CHUNK_STATES, keep
+        try:
+            leaf = lambda t: t.to(DEV).requires_grad_(True)
+            qa, ka, va, ql, kl, vl, gd, bd, hd, tyd = (leaf(t) for t in (q, k, v, q, k, v, g, beta, init, ty))
+            if kind == 'gdn':
+                o_l, o_a, ht = nats_mixed_attn_gdn(qa, ka, va, ql, kl, vl, hd, gd, bd, tyd, nb, nats_block_size=block,
+                                                   ops_for_incomplete_chunks='all', output_final_state_gated_delta=True,
+                                                   decay_for_non_gdn_blocks=True, **kw)
+            else:
+                o_l, o_a, ht = nats_mixed_attn_mamba(qa, ka, va, ql, kl, vl, hd, gd, tyd, nb, scale_lattn=1.0, nats_block_size=block,
+                                                     ops_for_incomplete_chunks='all', output_final_state_mamba=True,
+                                                     decay_for_non_mamba_blocks=True, **kw)
+            ((o_l.float() * do_l.float()).sum() + (o_a.float() * do_a.float()).sum() + (ht * dht).sum()).backward()
+            torch.cuda.synchronize()
+            leaves = [ql, kl, vl, gd, hd] + ([bd] if kind == 'gdn' else [])
+            # (column 1 of the selector's gradient is the linear op's; column 0 comes from the softmax backward's atomic adds)
+            return [o_l.detach(), ht.detach(), tyd.grad[..., 1]] + [t.grad for t in leaves]
+        finally:
+            MC.SAVE_CHUNK_STATES = old
+
+    kept, again = grads(True), grads(False)
+    for i, (a, b) in enumerate(zip(kept, again)):
+        assert torch.equal(a, b), f"tensor {i} differs between the kept and the recomputed chunk states"
