@@ -170,7 +170,8 @@ int natsl_mamba_chunk_fwd(const void* q, const void* k, const void* v, const flo
 
 /* Backward of the two chunked linear branches (delta_rule != 0: Gated DeltaNet, else Mamba2-style SSD); packed input as for the
  * forward (B = 1, the sequence table, TN = all blocks; dht, dh0 then hold one state per sequence).  Call the forward entry first with chunk_states and (delta rule) chunk_v_new and
- * keep its workspace: this entry reads the triangular solves from it.  Inputs as for the forward, plus
+ * keep its workspace (both forms: the reverse scan reads the scale vectors from it and, for the delta rule, the triangular solves
+ * and the intra-chunk matrices).  Inputs as for the forward, plus
  *   v_new [B*T][H][V] (Mamba: v itself), d_o [B*T][H][V] bf16, dht [B][H][K][V] f32 or NULL,
  *   g_block_sums [B][TN][H] f32 = sum of g over every selector block (packed: flat over the sequences' blocks).
  * Outputs: dq, dk [B*T][H][K], dv [B*T][H][V] bf16; dg, dbeta (delta rule) [B*T][H] f32; dh0 [B][H][K][V] f32 or NULL;

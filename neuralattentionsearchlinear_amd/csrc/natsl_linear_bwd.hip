@@ -29,10 +29,12 @@
 //                            derivative with respect to a gate on the chunk's state update: the selector's straight-through
 //                            gradient for the linear operator (src/nats/ops/common/chunk_o.py:438-443, :487-492).
 //
-// Both kernels rebuild q^, k^ and the decay vectors from q, k, g; of the forward's workspace only TmB is read.
-// Tiles sit in LDS row-major as they lie in memory; an operand that needs the other orientation (k^T, q^T, S, dS', TmB^T) is
-// fetched with the transposing read ds_read_b64_tr_b16 (within 16 lanes, lane i names four consecutive elements R_i and
-// receives element i % 4 of R_{i/4}, R_{4+i/4}, R_{8+i/4}, R_{12+i/4}): two such reads are the eight contraction slots of a lane.
+// The reverse scan takes a chunk's inputs as the forward scan does: raw q, k rows, and TmB, P and the scale vectors (which
+// carry the reciprocal row norms) from the forward's workspace, all by LDS-DMA into a two-stage ring.  The per-chunk kernel
+// rebuilds q^, k^ and the decay vectors from q, k, g; its tiles sit in LDS row-major as they lie in memory.  An operand that
+// needs the other orientation (k^T, q^T, S, dS', TmB^T, P^T) is fetched with the transposing read ds_read_b64_tr_b16 (within
+// 16 lanes, lane i names four consecutive elements R_i and receives element i % 4 of R_{i/4}, R_{4+i/4}, R_{8+i/4},
+// R_{12+i/4}): two such reads are the eight contraction slots of a lane.
 #include "natsl_device.h"
 #include "natsl_host.h"
 
@@ -51,7 +53,9 @@ struct LinBwdParams {
   const float* dht;       // [B][H][K][V] or null
   float* dh0;             // [B][H][K][V] or null
   const float* gsum_blk;  // sum of g over every selector block, [B][TN][H]
-  const bf16_t* ws_tm;    // TmB of every chunk-head in the forward scan's operand order
+  const bf16_t* ws_tm;    // the forward's workspace: TmB of every chunk-head in the forward scan's operand order,
+  const bf16_t* ws_p;     // P likewise,
+  const float* ws_sc;     // and the four scale vectors
   const void* types;
   int types_dtype;
   bf16_t* dq;
@@ -216,32 +220,78 @@ NATSL_DEVICE void store_scalars(const int lane, float x, const float b, const fl
 // =============================================================================================
 // reverse scan
 // =============================================================================================
+// one DMA instruction: lane l copies 16 bytes from base + voff to LDS byte address lds + 16 l
+NATSL_DEVICE void dma16(const void* base, const unsigned voff, const unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds) : "memory", "m0");
+}
+
+// Swizzle of the raw k / q tiles (row-major, unpadded rows of DK bf16; the forward scan's): 16-byte segment s of row r sits at
+// s ^ kq_swz(r), so that the row reads (16 lanes = 16 consecutive rows at one segment) and the transposing reads (16 lanes =
+// 4 consecutive rows x 4 segments of an aligned group) both fall on 16 different 16-byte slots of the 256-byte bank period.
+template <int DK>
+NATSL_DEVICE int kq_swz(const int r) {
+  if constexpr (DK == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (r >> 1) & 7;
+}
+// the 64-column dO / v_new tiles (rows of 128 bytes): rows two apart share banks
+NATSL_DEVICE int v_swz(const int r) { return 2 * ((r >> 1) & 1); }
+
+typedef __attribute__((address_space(3))) const bf16x8* lds_b128_t;
+typedef __attribute__((address_space(3))) const f32x4* lds_f4_t;
+typedef __attribute__((address_space(3))) const float* lds_f1_t;
+typedef __attribute__((address_space(3))) s16x4* lds_tr_t;
+typedef __attribute__((address_space(3))) bf16_t* lds_h_t;
+typedef __attribute__((address_space(3))) bf16x8* lds_w128_t;
+
+NATSL_DEVICE s16x4 lds_tr4_at(const unsigned addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr_t>(addr));
+}
+// x of another lane of the row, chosen by a data-parallel-primitive control word (row mirror 0x140, half-row mirror 0x141,
+// quad permutations 0x00..0xff)
+template <int CTRL>
+NATSL_DEVICE float lane_mirror(const float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+NATSL_DEVICE float uniform_f(const float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+// index of operand (t, s) of TmB / P among the six that are stored (the two above the diagonal are skipped)
+NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t : 2 * t - 2 + s; }
+
+// LDS of the reverse scan: two stages, each one chunk's inputs exactly as they lie in memory (filled by LDS-DMA).
 template <int DK>
 struct BwdScanLds {
-  static constexpr int KP = DK + 8;
-  // q^, k^ [64][KP]; dO (later dX) and v_new [64][TP]; TmB as stored (eight 1 KiB operands); P^T as six 1 KiB operands
-  static constexpr int QN = 0, KN = QN + CB * KP, DO = KN + CB * KP, VN = DO + CB * TP, TM = VN + CB * TP, PT = TM + 8 * 512;
-  static constexpr int ELEMS = PT + 6 * 512;
-  static constexpr int FL = ELEMS * 2;            // byte offset of the float area
-  static constexpr int TOTAL = FL + 7 * CB * 4;
+  static constexpr int KROW = DK * 2, VROW = 128;        // bytes per k / q row, per dO / v_new row (64 columns)
+  static constexpr int KB = CB * KROW, VB = CB * VROW, TB = 6 * 1024, SCB = 1024;
+  static constexpr int OFF_K = 0, OFF_Q = OFF_K + KB, OFF_DO = OFF_Q + KB, OFF_VN = OFF_DO + VB, OFF_T = OFF_VN + VB,
+                       OFF_P = OFF_T + TB, OFF_SC = OFF_P + TB;
+  static constexpr int STAGE = OFF_SC + SCB;
+  // Up to K = 128 a fifth wave does nothing but issue the requests (it shares a SIMD with a compute wave, so every wave has
+  // to fit 256 registers: for K = 128 the held-back state gradient of a rolled-back block waits in LDS instead of
+  // registers); K = 192 has neither the registers nor the LDS for that, and its compute waves issue the requests themselves.
+  static constexpr bool DMAW = DK <= 128, PEND_LDS = DK == 128;
+  static constexpr int PEND = (DK / 16) * 4 * 64 * 4;    // bytes per wave
+  static constexpr int TOTAL = 2 * STAGE + (PEND_LDS ? 4 * PEND : 0);
+  static constexpr int THREADS = DMAW ? 320 : 256;
 };
 
+// The inputs of a chunk are the forward scan's: raw q, k rows (the reciprocal norms ride in the scale vectors), the prep
+// kernel's TmB, P and scale vectors {se = e^gamma rk, sq = scale rq e^gamma, sk = rk e^{G-gamma}, {e^G, G, is_linear}} from
+// the workspace (Mamba: {gamma log2 e, scale e^gamma, e^{min(G-gamma,0)}, ...}; no TmB, P), plus dO and v_new.  Every wave
+// requests its share of chunk c - 1 by LDS-DMA right after the barrier that opens chunk c; nothing is staged in registers.
+// The state gradient uses the forward scan's row order: tile m, lane group g, register r hold K row
+// 32 (m / 2) + 8 g + 4 (m % 2) + r, so that two tiles side by side are eight consecutive K rows (one 16-byte piece of a k / q
+// row as the A operand of K~ dS', one 16-byte store of dS').
 template <int DK, bool DELTA>
-__global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams p) {
+__global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kernel(const LinBwdParams p) {
   using L = BwdScanLds<DK>;
-  constexpr int KP = L::KP, KT16 = DK / 16, KS = DK / 32;
-  extern __shared__ __align__(16) unsigned char smem[];
-  bf16_t* const sm = reinterpret_cast<bf16_t*>(smem);
-  bf16_t* const Qn = sm + L::QN;
-  bf16_t* const Kn = sm + L::KN;
-  bf16_t* const DOs = sm + L::DO;
-  bf16_t* const VNs = sm + L::VN;
-  bf16_t* const TmS = sm + L::TM;
-  bf16_t* const PTs = sm + L::PT;
-  float* const fl = reinterpret_cast<float*>(smem + L::FL);
-  float *gam = fl, *eg = fl + CB, *ek = fl + 2 * CB, *bet = fl + 3 * CB, *rq = fl + 4 * CB, *rk = fl + 5 * CB, *sqv = fl + 6 * CB;
+  constexpr int KT = DK / 16, KS = DK / 32;
+  constexpr bool DMAW = L::DMAW, PEND_LDS = L::PEND_LDS;
+  extern __shared__ __align__(1024) unsigned char smem[];
+  const unsigned lds0 = (unsigned)(size_t)smem;
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nsplit = p.V / 64;
   const int chain = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
   const int n = chain / p.H, h = chain % p.H;
@@ -256,280 +306,462 @@ __global__ __launch_bounds__(256) void linear_bwd_scan_kernel(const LinBwdParams
   const int col = vcol0 + 16 * wave + x16;
   const int per = p.block / CB;
   const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0, intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
-  const bool l2 = DELTA && (p.flags & NATSL_QK_L2NORM) != 0;
-  const int hn = h / (p.H / p.HN);
 
-  f32x4 dS[KT16], pend[KT16];
+  auto krow_of = [&](const int m, const int r) { return 32 * (m >> 1) + 8 * g4 + 4 * (m & 1) + r; };
+  f32x4 dS[KT], pend[PEND_LDS ? 1 : KT];
+  typedef __attribute__((address_space(3))) float* lds_wf_t;
+  const unsigned a_pend = lds0 + 2 * L::STAGE + (wave & 3) * L::PEND + 4 * lane;   // value (m, r) of this lane at + 256 (4 m + r)
+  if (wave < 4) {
 #pragma unroll
-  for (int m = 0; m < KT16; ++m)
+    for (int m = 0; m < KT; ++m)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      dS[m][r] = p.dht ? p.dht[((size_t)chain * DK + 16 * m + 4 * g4 + r) * p.V + col] : 0.f;
-      pend[m][r] = 0.f;
-    }
-
-  // ---- what a thread fetches for a chunk; requested one chunk ahead, under the state-gradient update of the chunk before ----
-  QkRegs<DK> qk;
-  u32x4 do_r[2], vn_r[2], tm_r[2];
-  // (scalars are fetched raw and interpreted when the chunk's turn comes: anything computed from them here would make
-  // the wave wait for all of the requests)
-  float g_r = 0.f, gs_r = 0.f;
-  unsigned beta_r = 0u, ty_r = 0u;
-  auto fetch = [&](const int cc) __attribute__((always_inline)) {
-    const int t0 = cc * CB, nvalid = min(CB, len - t0);
-    const size_t row0 = (size_t)bos + t0;
-    load_qk<DK>(p, tid, row0, nvalid, h, qk);
-    load_tokens64(p.d_o, tid, row0, nvalid, p.H, p.V, h, vcol0, do_r);
-    if (DELTA) {
-      load_tokens64(p.vn, tid, row0, nvalid, p.H, p.V, h, vcol0, vn_r);
-      // TmB: a straight copy of the six stored operands (operand (t, s) at 2 t + s; 0, 2, 4..7 exist)
-      const bf16_t* tm = p.ws_tm + ((size_t)(chunk_off + cc) * p.H + h) * (CB * CB);
-#pragma unroll
-      for (int it = 0; it < 2; ++it) {
-        const int pc = tid + 256 * it;
-        if (pc < 6 * 64) {
-          const int oi = pc >> 6, o = oi < 2 ? 2 * oi : oi + 2;
-          tm_r[it] = *reinterpret_cast<const u32x4*>(tm + o * 512 + (pc & 63) * 8);
-        }
+      for (int r = 0; r < 4; ++r) {
+        dS[m][r] = p.dht ? p.dht[((size_t)chain * DK + krow_of(m, r)) * p.V + col] : 0.f;
+        if (!PEND_LDS) pend[m][r] = 0.f;
       }
+  }
+  if (NT <= 0) return;
+
+  // ---- requests: piece u of a tile covers its LDS bytes [1024 u, 1024 u + 1024); lane l fills byte 1024 u + 16 l, i.e. some
+  //      row and 16-byte position of the tile, from the source segment position ^ swizzle(row); wave w moves pieces w, w + 4, ..
+  const size_t qk_pitch = (size_t)p.H * DK * 2, v_pitch = (size_t)p.H * p.V * 2;   // bytes per token
+  constexpr int KQ_PER = L::KB / 1024 / 4, V_PER = L::VB / 1024 / 4;
+  unsigned kq_off[KQ_PER], v_off[V_PER];
+  auto set_offsets = [&](const int nvalid) __attribute__((always_inline)) {
+    // (rows past the end of the sequence: the last valid row once more; what they produce is never stored and meets zero weights)
+#pragma unroll
+    for (int j = 0; j < KQ_PER; ++j) {
+      const int byte = 1024 * (wave + 4 * j) + 16 * lane, row = byte / L::KROW, pos = (byte % L::KROW) / 16;
+      kq_off[j] = (unsigned)((size_t)min(row, nvalid - 1) * qk_pitch) + 16u * (unsigned)(pos ^ kq_swz<DK>(row));
     }
-    if (wave == 0) {
-      const size_t gi = (row0 + min(lane, nvalid - 1)) * p.H + h;
-      g_r = p.g[gi];
-      if (DELTA) beta_r = p.beta[gi];
+#pragma unroll
+    for (int j = 0; j < V_PER; ++j) {
+      const int byte = 1024 * (wave + 4 * j) + 16 * lane, row = byte / L::VROW, pos = (byte % L::VROW) / 16;
+      v_off[j] = (unsigned)((size_t)min(row, nvalid - 1) * v_pitch) + 16u * (unsigned)(pos ^ v_swz(row));
     }
-    const int blk = t0 / p.block;
-    const size_t ti = ((size_t)(blk0 + blk) * p.HN + hn) * 2 + 1;
-    if (p.types_dtype == NATSL_F32) ty_r = reinterpret_cast<const unsigned*>(p.types)[ti];
-    else ty_r = reinterpret_cast<const bf16_t*>(p.types)[ti];
-    gs_r = p.gsum_blk[((size_t)blk0 + blk) * p.H + h];
   };
-  fetch(NT - 1);
+  if constexpr (DMAW) {
+    if (wave == 4) {
+      // ======================= the data-movement wave: all requests of chunk c - 1 during step c =======================
+      // (the CU's memory pipe takes one 1 KiB request per ~44 cycles, 61 KiB per chunk: a compute wave that issues them
+      // waits for the pipe; this wave has nothing else to do)
+      constexpr int KQ_ALL = L::KB / 1024, V_ALL = L::VB / 1024;
+      unsigned ko[KQ_ALL], vo[V_ALL], wo[6];
+      auto offsets = [&](const int nvalid) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < KQ_ALL; ++u) {
+          const int byte = 1024 * u + 16 * lane, row = byte / L::KROW, pos = (byte % L::KROW) / 16;
+          ko[u] = (unsigned)((size_t)min(row, nvalid - 1) * qk_pitch) + 16u * (unsigned)(pos ^ kq_swz<DK>(row));
+        }
+#pragma unroll
+        for (int u = 0; u < V_ALL; ++u) {
+          const int byte = 1024 * u + 16 * lane, row = byte / L::VROW, pos = (byte % L::VROW) / 16;
+          vo[u] = (unsigned)((size_t)min(row, nvalid - 1) * v_pitch) + 16u * (unsigned)(pos ^ v_swz(row));
+        }
+      };
+#pragma unroll
+      for (int v = 0; v < 6; ++v) wo[v] = 16u * lane + 1024u * (v < 2 ? 2 * v : v + 2);
+      auto request_all = [&](const int cc) __attribute__((always_inline)) {
+        const unsigned st = lds0 + (cc & 1) * L::STAGE;
+        const size_t tok = ((size_t)bos + (size_t)cc * CB) * p.H + h;
+        const size_t unit = (size_t)(chunk_off + cc) * p.H + h;
+        // in the order the compute waves need them: scale vectors, k, dO, P, TmB, v_new, q
+        dma16(p.ws_sc + unit * (4 * CB), 16u * lane, st + L::OFF_SC);
+        const char* kb = reinterpret_cast<const char*>(p.k + tok * DK);
+#pragma unroll
+        for (int u = 0; u < KQ_ALL; ++u) dma16(kb, ko[u], st + L::OFF_K + 1024 * u);
+        const char* dob = reinterpret_cast<const char*>(p.d_o + tok * p.V + vcol0);
+#pragma unroll
+        for (int u = 0; u < V_ALL; ++u) dma16(dob, vo[u], st + L::OFF_DO + 1024 * u);
+        if (DELTA) {
+          if (intra) {
+            const char* pb = reinterpret_cast<const char*>(p.ws_p + unit * (CB * CB));
+#pragma unroll
+            for (int v = 0; v < 6; ++v) dma16(pb, wo[v], st + L::OFF_P + 1024 * v);
+          }
+          const char* tb = reinterpret_cast<const char*>(p.ws_tm + unit * (CB * CB));
+#pragma unroll
+          for (int v = 0; v < 6; ++v) dma16(tb, wo[v], st + L::OFF_T + 1024 * v);
+          const char* vnb = reinterpret_cast<const char*>(p.vn + tok * p.V + vcol0);
+#pragma unroll
+          for (int u = 0; u < V_ALL; ++u) dma16(vnb, vo[u], st + L::OFF_VN + 1024 * u);
+        }
+        const char* qb = reinterpret_cast<const char*>(p.q + tok * DK);
+#pragma unroll
+        for (int u = 0; u < KQ_ALL; ++u) dma16(qb, ko[u], st + L::OFF_Q + 1024 * u);
+      };
+      const int nlast = min(CB, len - (NT - 1) * CB);
+      offsets(nlast);
+      request_all(NT - 1);
+      if (nlast < CB) offsets(CB);
+      for (int c = NT - 1; c >= 0; --c) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);   // chunk c has landed
+        __syncthreads();                      // .. and every compute wave is done with the other stage
+        if (c > 0) request_all(c - 1);
+        if (!DELTA && intra) __syncthreads();   // (the compute waves' exchange of P^T)
+      }
+      return;
+    }
+  }
+  // TmB / P: six 1 KiB operands each (stored at 0, 2, 4..7 of eight), plain copies; wave w moves operands w and w + 4
+  const unsigned ws_off0 = 16u * lane + 1024u * (wave < 2 ? 2 * wave : wave + 2), ws_off1 = 16u * lane + 1024u * (wave + 6);
+  // The CU's memory pipe takes one such 1 KiB instruction per ~44 cycles (61 KiB per chunk: 2 800 cycles), and a wave that
+  // issues its 16 in one go waits for all of them to be accepted; so a chunk's requests are spread over the step in groups
+  // (request<G>(cc), G = 0..NGROUPS-1), each small enough to find the pipe free.
+  constexpr int NGROUPS = 7;
+  const char *rq_k = nullptr, *rq_q = nullptr, *rq_do = nullptr, *rq_vn = nullptr, *rq_t = nullptr, *rq_p = nullptr, *rq_sc = nullptr;
+  auto request_bases = [&](const int cc) __attribute__((always_inline)) {
+    const size_t tok = ((size_t)bos + (size_t)cc * CB) * p.H + h;
+    const size_t unit = (size_t)(chunk_off + cc) * p.H + h;
+    rq_k = reinterpret_cast<const char*>(p.k + tok * DK);
+    rq_q = reinterpret_cast<const char*>(p.q + tok * DK);
+    rq_do = reinterpret_cast<const char*>(p.d_o + tok * p.V + vcol0);
+    rq_vn = reinterpret_cast<const char*>(p.vn + tok * p.V + vcol0);
+    rq_t = reinterpret_cast<const char*>(p.ws_tm + unit * (CB * CB));
+    rq_p = reinterpret_cast<const char*>(p.ws_p + unit * (CB * CB));
+    rq_sc = reinterpret_cast<const char*>(p.ws_sc + unit * (4 * CB));
+  };
+  auto request = [&](const int grp, const int cc) __attribute__((always_inline)) {
+    const unsigned st = lds0 + (cc & 1) * L::STAGE;
+    constexpr int KH = (KQ_PER + 1) / 2;
+    if (grp == 0) {
+      if (wave == 3) dma16(rq_sc, 16u * lane, st + L::OFF_SC);
+#pragma unroll
+      for (int j = 0; j < KH; ++j) dma16(rq_k, kq_off[j], st + L::OFF_K + 1024 * (wave + 4 * j));
+    } else if (grp == 1) {
+#pragma unroll
+      for (int j = KH; j < KQ_PER; ++j) dma16(rq_k, kq_off[j], st + L::OFF_K + 1024 * (wave + 4 * j));
+    } else if (grp == 2) {
+#pragma unroll
+      for (int j = 0; j < V_PER; ++j) dma16(rq_do, v_off[j], st + L::OFF_DO + 1024 * (wave + 4 * j));
+    } else if (grp == 3) {
+      if (DELTA && intra) {
+        dma16(rq_p, ws_off0, st + L::OFF_P + 1024 * wave);
+        if (wave < 2) dma16(rq_p, ws_off1, st + L::OFF_P + 1024 * (wave + 4));
+      }
+    } else if (grp == 4) {
+      if (DELTA) {
+        dma16(rq_t, ws_off0, st + L::OFF_T + 1024 * wave);
+        if (wave < 2) dma16(rq_t, ws_off1, st + L::OFF_T + 1024 * (wave + 4));
+      }
+    } else if (grp == 5) {
+      if (DELTA) {
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) dma16(rq_vn, v_off[j], st + L::OFF_VN + 1024 * (wave + 4 * j));
+      }
+#pragma unroll
+      for (int j = 0; j < KH; ++j) dma16(rq_q, kq_off[j], st + L::OFF_Q + 1024 * (wave + 4 * j));
+    } else {
+#pragma unroll
+      for (int j = KH; j < KQ_PER; ++j) dma16(rq_q, kq_off[j], st + L::OFF_Q + 1024 * (wave + 4 * j));
+    }
+  };
+
+  // ---- per-lane operand addresses inside a stage (the forward scan's) -----------------------------------------------------
+  // k / q rows as an operand (token tile t, k-step s): row 16 t + x16, segment 4 s + g4; t goes into the offset
+  unsigned a_kq[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) a_kq[s] = (unsigned)(x16 * L::KROW) + 16u * (unsigned)((4 * s + g4) ^ kq_swz<DK>(x16));
+  // q^T / k^T as A operand (state tile m, token k-step s2, read rd): lane x16 names token 32 s2 + 16 rd + 4 g4 + x16 / 4 and
+  // the four K rows 32 (m / 2) + 8 (x16 % 4) + 4 (m % 2) ..: segment 4 (m / 2) + x16 % 4, half m % 2
+  unsigned a_kt[KT / 2];
+  {
+    const int tk = 4 * g4 + (x16 >> 2);
+#pragma unroll
+    for (int mh = 0; mh < KT / 2; ++mh)
+      a_kt[mh] = (unsigned)(tk * L::KROW) + 16u * (unsigned)((4 * mh + (x16 & 3)) ^ kq_swz<DK>(tk));
+  }
+  // dO / v_new through the transposing read (token tile t): lane x16 names token 16 t + 4 g4 + x16 / 4, columns
+  // 16 wave + 4 (x16 % 4) ..; it receives tokens 16 t + 4 g4 + 0..3 of column 16 wave + x16 (the accumulator layout)
+  unsigned a_v;
+  {
+    const int tk = 4 * g4 + (x16 >> 2), seg = 2 * wave + ((x16 & 3) >> 1);
+    a_v = (unsigned)(tk * L::VROW) + 16u * (unsigned)(seg ^ v_swz(tk)) + 8u * (x16 & 1);
+  }
+  // TmB^T / P^T as A operand: element (row i, column cc) of the stored matrix sits in operand (i / 16, cc / 32), lane slot
+  // 16 ((cc % 16) / 4) + i % 16, element 4 ((cc % 32) / 16) + cc % 4: four consecutive columns are contiguous, so the
+  // transposing read applies with "rows" = lane slots; lane x16 names slot 16 (x16 % 4) + 4 g4 + x16 / 4
+  const unsigned a_tm = 16u * (unsigned)(16 * (x16 & 3) + 4 * g4 + (x16 >> 2));
+  const unsigned a_sc = 16u * g4;    // this lane group's four tokens in a row of the scale vectors
+
+  {
+    const int nlast = min(CB, len - (NT - 1) * CB);
+    if constexpr (!DMAW) {
+      set_offsets(nlast);
+      request_bases(NT - 1);
+#pragma unroll
+      for (int grp = 0; grp < NGROUPS; ++grp) request(grp, NT - 1);
+      if (nlast < CB) set_offsets(CB);
+    }
+  }
+  float gs_next = p.gsum_blk[((size_t)blk0 + ((NT - 1) * CB) / p.block) * p.H + h];
+  bool have_pend = false;
 
   for (int c = NT - 1; c >= 0; --c) {
+    const unsigned st = lds0 + (c & 1) * L::STAGE;
     const int t0 = c * CB, nvalid = min(CB, len - t0);
     const size_t row0 = (size_t)bos + t0;
-    __syncthreads();   // every wave is done with the previous chunk's tiles
-    if (wave == 0)
-      store_scalars<DELTA>(lane, lane < nvalid ? g_r : 0.f, lane < nvalid ? bf16_to_f32((bf16_t)beta_r) : 0.f, p.scale, gam, eg, ek, sqv, bet);
-    store_qk<DK>(qk, tid, l2, Qn, Kn, rq, rk);
-    store_tokens64(do_r, tid, DOs);
-    if (DELTA) {
-      store_tokens64(vn_r, tid, VNs);
-#pragma unroll
-      for (int it = 0; it < 2; ++it) {
-        const int pc = tid + 256 * it;
-        if (pc < 6 * 64) {
-          const int oi = pc >> 6, o = oi < 2 ? 2 * oi : oi + 2;
-          *reinterpret_cast<u32x4*>(TmS + o * 512 + (pc & 63) * 8) = tm_r[it];
-        }
-      }
+    // chunk c has landed (a wave's vector memory operations complete in order) and every wave is done with the other stage
+    if constexpr (!DMAW) __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    const float gs_r = gs_next;
+    const bool more = !DMAW && c > 0;     // (requests from the compute waves)
+    if (more) {
+      request_bases(c - 1);
+      request(0, c - 1);
     }
-    const bool lin = rintf(__uint_as_float(p.types_dtype == NATSL_F32 ? ty_r : ty_r << 16)) == 1.0f;
+    const float dec = uniform_f(*reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * CB)));
+    const bool lin = uniform_f(*reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (3 * CB + 2))) != 0.f;
     const float f_blk = decay ? __expf(gs_r) : 1.f;
-    {
-      // dS' of this chunk goes out as it arrived
-      bf16_t* dso = p.ds_all + (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 4 * g4;
+    // dS' of this chunk as it arrived: it goes out at the end of the step (every global store of the compute waves does: right
+    // after the barrier the CU's memory pipe is busy with the requests for the next chunk, and a store would wait behind them)
+    bf16x8 DSB[KS];
 #pragma unroll
-      for (int m = 0; m < KT16; ++m) {
-        u32x2 w = {pack_bf16x2(dS[m][0], dS[m][1]), pack_bf16x2(dS[m][2], dS[m][3])};
-        *reinterpret_cast<u32x2*>(dso + 16 * m) = w;
-      }
-    }
-    __syncthreads();   // the tiles are there
-
-    // ---- P^T as operands, once per workgroup: Z = q^ k^^T leaves lane (x, g) with key 16 tj + x against queries
-    //      16 ti + 4 g + r, the four slots this lane holds of operand (tj, ti / 2), half ti % 2.  Operand (tj, s2) at index
-    //      tj < 2 ? 2 tj + s2 : 2 + tj; waves 0..3 form {(0,0), (1,0)}, {(0,1), (3,1)}, {(1,1)}, {(2,1)}: 3, 3, 2, 2 tiles. ----
-    if (intra) {
-      auto make_operand = [&](const int tj, const int s2) __attribute__((always_inline)) {
-        const float gj = gam[16 * tj + x16];
-        f32x4 Z[2];
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          const int ti = 2 * s2 + hf;
-          Z[hf] = (f32x4){0.f, 0.f, 0.f, 0.f};
-          if (ti >= tj) {
-#pragma unroll
-            for (int s = 0; s < KS; ++s) {
-              const bf16x8 a = *reinterpret_cast<const bf16x8*>(Qn + (16 * ti + x16) * KP + 32 * s + 8 * g4);
-              const bf16x8 b = *reinterpret_cast<const bf16x8*>(Kn + (16 * tj + x16) * KP + 32 * s + 8 * g4);
-              Z[hf] = mfma16(a, b, Z[hf]);
-            }
-            const f32x4 gi = *reinterpret_cast<const f32x4*>(gam + 16 * ti + 4 * g4);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const bool vis = ti > tj || 4 * g4 + r >= x16;
-              Z[hf][r] = vis ? Z[hf][r] * p.scale * __expf(gi[r] - gj) : 0.f;
-            }
-          }
-        }
-        *reinterpret_cast<bf16x8*>(PTs + (tj < 2 ? 2 * tj + s2 : 2 + tj) * 512 + lane * 8) = pack8(Z[0], Z[1]);
-      };
-      if (wave == 0) { make_operand(0, 0); make_operand(1, 0); }
-      else if (wave == 1) { make_operand(0, 1); make_operand(3, 1); }
-      else if (wave == 2) make_operand(1, 1);
-      else make_operand(2, 1);
-    }
+    for (int s = 0; s < KS; ++s) DSB[s] = pack8(dS[2 * s], dS[2 * s + 1]);
     // ---- a rolled-back block's dS' leaves the chain here ---------------------------------------------------------------
     const bool last = ((c + 1) % per == 0) || (c == NT - 1);
-    if (last) {
-      const float f = lin ? 0.f : f_blk;
+    // (pend is zero here: it was handed over at the first chunk of the block behind this one)
+    if (last && !lin) {
 #pragma unroll
-      for (int m = 0; m < KT16; ++m)
+      for (int m = 0; m < KT; ++m)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          pend[m][r] = dS[m][r] * f;
-          if (!lin) dS[m][r] = 0.f;
+          if constexpr (PEND_LDS) *reinterpret_cast<lds_wf_t>(a_pend + 256 * (4 * m + r)) = dS[m][r] * f_blk;
+          else pend[m][r] = dS[m][r] * f_blk;
+          dS[m][r] = 0.f;
         }
+      have_pend = true;
     }
-    const float dec = __expf(gam[CB - 1]);
+    if (more) request(1, c - 1);
 
     // ---- Y1 = K~ dS' ----------------------------------------------------------------------------------------------------
     f32x4 DV[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) DV[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    {
-      bf16x8 DSB[KS];
+    if (!(last && !lin)) {   // (behind a rolled-back block dS' is zero)
 #pragma unroll
-      for (int s = 0; s < KS; ++s) DSB[s] = pack8(dS[2 * s], dS[2 * s + 1]);
+      for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          const bf16_t* kr = Kn + (16 * t + x16) * KP + 32 * s + 4 * g4;
-          const bf16x8 a = join_u2(*reinterpret_cast<const u32x2*>(kr), *reinterpret_cast<const u32x2*>(kr + 16));
-          DV[t] = mfma16(a, DSB[s], DV[t]);
-        }
+        for (int t = 0; t < 4; ++t)
+          DV[t] = mfma16(*reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + t * 16 * L::KROW), DSB[s], DV[t]);
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const f32x4 e4 = *reinterpret_cast<const f32x4*>(ek + 16 * t + 4 * g4);
+        const f32x4 e4 = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * (2 * CB) + a_sc + 64 * t);
 #pragma unroll
         for (int r = 0; r < 4; ++r) DV[t][r] *= e4[r];
       }
     }
-    // ---- dO in accumulator layout (lane = column, registers = tokens 16 t + 4 g + r) ------------------------------------
+    if (more) request(2, c - 1);
+    // ---- dO in accumulator layout (lane = column, registers = tokens 16 t + 4 g + r); zero past the end of the sequence ----
     f32x4 DOc[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 4; ++t) {
+      const s16x4 w = lds_tr4_at(st + L::OFF_DO + a_v + t * 16 * L::VROW);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) DOc[t][r] = bf16_to_f32(DOs[(16 * t + 4 * g4 + r) * TP + 16 * wave + x16]);
-    __syncthreads();   // P^T
+      for (int r = 0; r < 4; ++r) DOc[t][r] = bf16_to_f32((bf16_t)w[r]);
+    }
+    if (__builtin_expect(nvalid < CB, 0)) {
+      asm volatile("" ::: "memory");   // (keeps this a branch: it runs once per chain)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (16 * t + 4 * g4 + r >= nvalid) DOc[t][r] = 0.f;
+    }
+    if (more) request(3, c - 1);
     // ---- Y2 = P^T dO ----------------------------------------------------------------------------------------------------
     if (intra) {
       const bf16x8 DOB[2] = {pack8(DOc[0], DOc[1]), pack8(DOc[2], DOc[3])};
+      if constexpr (DELTA) {
+        // P as the prep kernel stored it, read transposed (see a_tm): rows i = 32 s2 + 16 hf + 4 g + j of column 16 tj + x
 #pragma unroll
-      for (int tj = 0; tj < 4; ++tj)
+        for (int tj = 0; tj < 4; ++tj)
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-          if (tj < 2 || s2 == 1)
-            DV[tj] = mfma16(*reinterpret_cast<const bf16x8*>(PTs + (tj < 2 ? 2 * tj + s2 : 2 + tj) * 512 + lane * 8), DOB[s2], DV[tj]);
+          for (int s2 = 0; s2 < 2; ++s2)
+            if (2 * s2 + 1 >= tj) {
+              const unsigned lo = st + L::OFF_P + 1024 * tri_slot(2 * s2, tj >> 1) + a_tm + 8 * (tj & 1);
+              const unsigned hi = st + L::OFF_P + 1024 * tri_slot(2 * s2 + 1, tj >> 1) + a_tm + 8 * (tj & 1);
+              DV[tj] = mfma16(join4(lds_tr4_at(lo), lds_tr4_at(hi)), DOB[s2], DV[tj]);
+            }
+      } else {
+        // P^T formed here, once per workgroup: Z = q k^T leaves lane (x, g) with key 16 tj + x against queries
+        // 16 ti + 4 g + r, the four slots this lane holds of operand (tj, ti / 2), half ti % 2.  Operand (tj, s2) at index
+        // tj < 2 ? 2 tj + s2 : 2 + tj; waves 0..3 form {(0,0), (1,0)}, {(0,1), (3,1)}, {(1,1)}, {(2,1)}: 3, 3, 2, 2 tiles.
+        auto make_operand = [&](const int tj, const int s2) __attribute__((always_inline)) {
+          const float gj = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (16 * tj + x16));   // gamma in log2 units
+          f32x4 Z[2];
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf) {
+            const int ti = 2 * s2 + hf;
+            Z[hf] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            if (ti >= tj) {
+#pragma unroll
+              for (int s = 0; s < KS; ++s) {
+                const bf16x8 a = *reinterpret_cast<lds_b128_t>(st + L::OFF_Q + a_kq[s] + ti * 16 * L::KROW);
+                const bf16x8 b = *reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + tj * 16 * L::KROW);
+                Z[hf] = mfma16(a, b, Z[hf]);
+              }
+              const f32x4 gi = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + a_sc + 64 * ti);
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const bool vis = ti > tj || 4 * g4 + r >= x16;
+                Z[hf][r] = vis ? Z[hf][r] * p.scale * __builtin_amdgcn_exp2f(gi[r] - gj) : 0.f;
+              }
+            }
+          }
+          *reinterpret_cast<lds_w128_t>(st + L::OFF_P + 1024 * (tj < 2 ? 2 * tj + s2 : 2 + tj) + 16 * lane) = pack8(Z[0], Z[1]);
+        };
+        if (wave == 0) { make_operand(0, 0); make_operand(1, 0); }
+        else if (wave == 1) { make_operand(0, 1); make_operand(3, 1); }
+        else if (wave == 2) make_operand(1, 1);
+        else make_operand(2, 1);
+        __syncthreads();   // P^T
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+            if (tj < 2 || s2 == 1)
+              DV[tj] = mfma16(*reinterpret_cast<lds_b128_t>(st + L::OFF_P + 1024 * (tj < 2 ? 2 * tj + s2 : 2 + tj) + 16 * lane), DOB[s2], DV[tj]);
+      }
     }
-    // ---- dX = TmB^T dv_new (dv_new as two operands).  Element (row i, column cc) of TmB sits in stored operand
-    //      (i / 16, cc / 32), lane slot 16 ((cc % 16) / 4) + i % 16, element 4 ((cc % 32) / 16) + cc % 4: four consecutive
-    //      columns are contiguous, so the transposing read applies with "rows" = lane slots ------------------------------
+    if (more) request(4, c - 1);
+    // ---- dX = TmB^T dv_new (dv_new as two operands: the truncated value and the remainder) ------------------------------------
     f32x4 DX[4];
-    if (DELTA) {
+    if constexpr (DELTA) {
       const bf16x8 DVB[2] = {pack8_trunc(DV[0], DV[1]), pack8_trunc(DV[2], DV[3])};
       const bf16x8 DVR[2] = {pack8_rest(DV[0], DV[1]), pack8_rest(DV[2], DV[3])};
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) {
         DX[tj] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
+        for (int s2 = 0; s2 < 2; ++s2)
           if (2 * s2 + 1 >= tj) {
-            // rows i = 32 s2 + 16 hf + 4 g + j of column 16 tj + x: lane l names slot 16 (l % 4) + 4 g + l / 4 of operand
-            // (2 s2 + hf, tj / 2), elements 4 (tj % 2) ..
-            const int slot = 16 * (x16 & 3) + 4 * g4 + (x16 >> 2);
-            const bf16_t* lo = TmS + (2 * (2 * s2) + (tj >> 1)) * 512 + slot * 8 + 4 * (tj & 1);
-            const bf16x8 a = join4(lds_tr4(lo), lds_tr4(lo + 2 * 512));
+            const unsigned lo = st + L::OFF_T + 1024 * tri_slot(2 * s2, tj >> 1) + a_tm + 8 * (tj & 1);
+            const unsigned hi = st + L::OFF_T + 1024 * tri_slot(2 * s2 + 1, tj >> 1) + a_tm + 8 * (tj & 1);
+            const bf16x8 a = join4(lds_tr4_at(lo), lds_tr4_at(hi));
             DX[tj] = mfma16(a, DVR[s2], DX[tj]);
             DX[tj] = mfma16(a, DVB[s2], DX[tj]);
           }
-        }
       }
     } else {
 #pragma unroll
       for (int t = 0; t < 4; ++t) DX[t] = DV[t];
     }
-    // dv = dX, through this wave's 16 columns of the dO tile (read above, by this wave only) so that it leaves in whole rows
+    if (more) request(5, c - 1);
+    // ---- dv = dX, through this wave's own 16 columns of the dO tile (read above, by this wave only) so that it leaves as
+    //      16-byte pieces; no other wave touches these bytes, so no barrier ----------------------------------------------------
+    float dbeta_part = 0.f;
     {
       float pb[16];
+      f32x4 VNc[4];
+      if constexpr (DELTA) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const s16x4 w = lds_tr4_at(st + L::OFF_VN + a_v + t * 16 * L::VROW);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) VNc[t][r] = bf16_to_f32((bf16_t)w[r]);
+        }
+      }
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int tok = 16 * t + 4 * g4 + r;
-          DOs[tok * TP + 16 * wave + x16] = f32_to_bf16(DX[t][r]);
-          if (DELTA) pb[4 * t + r] = DX[t][r] * bf16_to_f32(VNs[tok * TP + 16 * wave + x16]);
+          const int tk = 16 * t + 4 * g4 + r;
+          *reinterpret_cast<lds_h_t>(st + L::OFF_DO + tk * L::VROW + 16 * ((2 * wave + (x16 >> 3)) ^ v_swz(tk)) + 2 * (x16 & 7)) = f32_to_bf16(DX[t][r]);
+          if constexpr (DELTA) pb[4 * t + r] = DX[t][r] * VNc[t][r];
         }
-      if (DELTA) {
+      if constexpr (DELTA) {
         // for dbeta_i = <dX_i, v_new_i> / beta_i^2: this wave's 16 columns of the inner product (dX still in fp32).  Sixteen
         // sums over sixteen lanes as a butterfly: in every step a lane hands half of its values to its partner and adds
-        // the partner's other half to the rest; lane x ends up with sum number x.
-#pragma unroll
-        for (int d = 8; d >= 1; d >>= 1) {
+        // the partner's other half to the rest; lane x ends up with sum number x.  The partner is the lane's mirror image in
+        // its group of 16, 8, 4, 2 lanes (what the cross-lane operand modifiers of the vector ALU offer: no LDS round trip).
+        auto step = [&](const int d, auto mirror) __attribute__((always_inline)) {
           const bool up = (x16 & d) != 0;
 #pragma unroll
-          for (int i = 0; i < d; ++i) {
-            const float send = up ? pb[i] : pb[i + d], keep = up ? pb[i + d] : pb[i];
-            pb[i] = keep + __shfl_xor(send, d);
-          }
-        }
-        const int tok = 16 * (x16 >> 2) + 4 * g4 + (x16 & 3);
-        if (tok < nvalid) p.dbeta_parts[((row0 + tok) * p.H + h) * (p.V / 16) + 4 * split + wave] = pb[0];
+          for (int i = 0; i < 8; ++i)
+            if (i < d) {
+              const float send = up ? pb[i] : pb[i + d], keep = up ? pb[i + d] : pb[i];
+              pb[i] = keep + mirror(send);
+            }
+        };
+        step(8, [](const float x) { return lane_mirror<0x140>(x); });   // lane 15 - x of the row of 16
+        step(4, [](const float x) { return lane_mirror<0x141>(x); });   // 7 - x % 8 within each half row
+        step(2, [](const float x) { return lane_mirror<0x1b>(x); });    // quad order 3, 2, 1, 0
+        step(1, [](const float x) { return lane_mirror<0xb1>(x); });    // quad order 1, 0, 3, 2
+        dbeta_part = pb[0];
       }
     }
-    __syncthreads();   // the dX tile
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int pc = tid + 256 * it, row = pc >> 3, seg = pc & 7;
-      if (row < nvalid)
-        *reinterpret_cast<u32x4*>(p.dv + ((row0 + row) * p.H + h) * p.V + vcol0 + seg * 8) = *reinterpret_cast<const u32x4*>(DOs + row * TP + seg * 8);
-    }
-    // ---- dS = e^G dS' + Q~^T dO - W^T dX, with the next chunk's requests in flight ------------------------------------------
+    if (more) request(6, c - 1);
+    // ---- dS = e^G dS' + Q~^T dO - W^T dX ----------------------------------------------------------------------------------------
     {
       f32x4 A1[4], A2[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const f32x4 s4 = *reinterpret_cast<const f32x4*>(sqv + 16 * t + 4 * g4);
-        const f32x4 e4 = *reinterpret_cast<const f32x4*>(eg + 16 * t + 4 * g4);
+        const f32x4 s4 = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * CB + a_sc + 64 * t);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          A1[t][r] = DOc[t][r] * s4[r];
-          A2[t][r] = -DX[t][r] * e4[r];
+        for (int r = 0; r < 4; ++r) A1[t][r] = DOc[t][r] * s4[r];
+        if constexpr (DELTA) {
+          const f32x4 e4 = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + a_sc + 64 * t);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) A2[t][r] = -DX[t][r] * e4[r];
         }
       }
       const bf16x8 B1[2] = {pack8(A1[0], A1[1]), pack8(A1[2], A1[3])};
-      const bf16x8 B2[2] = {pack8(A2[0], A2[1]), pack8(A2[2], A2[3])};
-      if (c > 0) fetch(c - 1);
+      bf16x8 B2[2];
+      if constexpr (DELTA) { B2[0] = pack8(A2[0], A2[1]); B2[1] = pack8(A2[2], A2[3]); }
+      auto ld_t = [&](const int off, const int m, const int s2) __attribute__((always_inline)) -> bf16x8 {
+        const unsigned a = st + off + a_kt[m >> 1] + 8u * (m & 1) + (32 * s2) * L::KROW;
+        return join4(lds_tr4_at(a), lds_tr4_at(a + 16 * L::KROW));
+      };
 #pragma unroll
-      for (int m = 0; m < KT16; ++m) {
+      for (int m = 0; m < KT; ++m) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) dS[m][r] *= dec;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          // rows = K index 16 m + x, slots = tokens 32 s2 + 4 g + j and 32 s2 + 16 + 4 g + j
-          dS[m] = mfma16(tr_operand(Qn, KP, 32 * s2 + 4 * g4, 32 * s2 + 16 + 4 * g4, 16 * m, x16), B1[s2], dS[m]);
-          if (DELTA) dS[m] = mfma16(tr_operand(Kn, KP, 32 * s2 + 4 * g4, 32 * s2 + 16 + 4 * g4, 16 * m, x16), B2[s2], dS[m]);
+          dS[m] = mfma16(ld_t(L::OFF_Q, m, s2), B1[s2], dS[m]);
+          if constexpr (DELTA) dS[m] = mfma16(ld_t(L::OFF_K, m, s2), B2[s2], dS[m]);
         }
       }
     }
-    if (c % per == 0) {
+    // ---- this step's global stores (and the one scalar the next step needs) -----------------------------------------------
+    {
+      // eight consecutive K rows of this lane's column per 16-byte store
+      bf16_t* dso = p.ds_all + (((size_t)(chunk_off + c) * p.H + h) * p.V + col) * DK + 8 * g4;
 #pragma unroll
-      for (int m = 0; m < KT16; ++m)
+      for (int s = 0; s < KS; ++s) *reinterpret_cast<bf16x8*>(dso + 32 * s) = DSB[s];
+      // (the tile's writes above come first: same wave, and the LDS pipe keeps their order)
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+        const int pc = lane + 64 * it, row = pc >> 1, half = pc & 1;
+        const bf16x8 w = *reinterpret_cast<lds_b128_t>(st + L::OFF_DO + row * L::VROW + 16 * ((2 * wave + half) ^ v_swz(row)));
+        if (row < nvalid) *reinterpret_cast<bf16x8*>(p.dv + ((row0 + row) * p.H + h) * p.V + vcol0 + 16 * wave + 8 * half) = w;
+      }
+      if constexpr (DELTA) {
+        const int tk = 16 * (x16 >> 2) + 4 * g4 + (x16 & 3);
+        if (tk < nvalid) p.dbeta_parts[((row0 + tk) * p.H + h) * (p.V / 16) + 4 * split + wave] = dbeta_part;
+      }
+      if (c > 0) gs_next = p.gsum_blk[((size_t)blk0 + ((c - 1) * CB) / p.block) * p.H + h];
+    }
+    if (c % per == 0 && have_pend) {
+#pragma unroll
+      for (int m = 0; m < KT; ++m)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          dS[m][r] += pend[m][r];
-          pend[m][r] = 0.f;
+          if constexpr (PEND_LDS) dS[m][r] += *reinterpret_cast<lds_f1_t>(a_pend + 256 * (4 * m + r));
+          else {
+            dS[m][r] += pend[m][r];
+            pend[m][r] = 0.f;
+          }
         }
+      have_pend = false;
     }
   }
   if (p.dh0) {
 #pragma unroll
-    for (int m = 0; m < KT16; ++m)
+    for (int m = 0; m < KT; ++m)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) p.dh0[((size_t)chain * DK + 16 * m + 4 * g4 + r) * p.V + col] = dS[m][r];
+      for (int r = 0; r < 4; ++r) p.dh0[((size_t)chain * DK + krow_of(m, r)) * p.V + col] = dS[m][r];
   }
 }
 
@@ -857,7 +1089,7 @@ static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* wha
     auto kern = linear_bwd_scan_kernel<DK, DELTA>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)((p.seqs ? p.n_seqs : p.B) * p.H * (p.V / 64))), dim3(256), L::TOTAL, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((p.seqs ? p.n_seqs : p.B) * p.H * (p.V / 64))), dim3(L::THREADS), L::TOTAL, stream, p);
     const int rc = check_launch(what);
     if (rc != NATSL_OK) return rc;
   }
@@ -883,7 +1115,7 @@ extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void*
                                       const natsl_seq_row* seqs, int n_seqs, int total_chunks, natsl_stream_t stream) {
   const char* what = "natsl_linear_chunk_bwd";
   if (!q || !k || !v_new || !g || !d_o || !chunk_states || !types || !g_block_sums || !d_chunk_states || !dq || !dk || !dv || !dg ||
-      !d_gate || !d_rollback || (delta_rule && (!beta || !dbeta || !dbeta_parts || !workspace)))
+      !d_gate || !d_rollback || !workspace || (delta_rule && (!beta || !dbeta || !dbeta_parts)))
     return fail(NATSL_ERR_INVALID, "%s: null pointer argument", what);
   if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "%s: only bf16 tensors are supported (got dtype %d)", what, dtype);
   if (types_dtype != NATSL_BF16 && types_dtype != NATSL_F32) return fail(NATSL_ERR_UNSUPPORTED, "%s: block types must be f32 or bf16", what);
@@ -896,7 +1128,13 @@ extern "C" int natsl_linear_chunk_bwd(int delta_rule, const void* q, const void*
   LinBwdParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.vn = (const bf16_t*)v_new; p.d_o = (const bf16_t*)d_o; p.g = g;
   p.beta = (const bf16_t*)beta; p.s_all = (const bf16_t*)chunk_states; p.ds_all = (bf16_t*)d_chunk_states; p.dv = (bf16_t*)dv;
-  p.dht = dht; p.dh0 = dh0; p.gsum_blk = g_block_sums; p.ws_tm = (const bf16_t*)workspace; p.types = types; p.types_dtype = types_dtype;
+  p.dht = dht; p.dh0 = dh0; p.gsum_blk = g_block_sums; p.ws_tm = (const bf16_t*)workspace; p.types = types;
+  {
+    // (the layout natsl_gdn_chunk_fwd / natsl_mamba_chunk_fwd gave the workspace)
+    const size_t units = (size_t)(seqs ? total_chunks : B * cdiv(T, CB)) * (size_t)H;
+    p.ws_p = p.ws_tm + units * (CB * CB);
+    p.ws_sc = reinterpret_cast<const float*>(p.ws_p + units * (CB * CB));
+  } p.types_dtype = types_dtype;
   p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dg = dg; p.dbeta = dbeta; p.dbeta_parts = dbeta_parts; p.gate = d_gate; p.rb = d_rollback;
   p.B = B; p.T = T; p.H = H; p.HN = HN; p.V = V; p.TN = TN; p.block = block; p.nt = cdiv(T, CB);
   p.seqs = reinterpret_cast<const SeqRow*>(seqs); p.n_seqs = seqs ? n_seqs : 0; p.total_chunks = seqs ? total_chunks : B * p.nt;

@@ -335,8 +335,10 @@ def test_c2_gdn_backward_full_depth(c2):
     names = ['dq', 'dk', 'dv', 'dg', 'dbeta']
     for j, name in enumerate(names):
         assert torch.isfinite(got[j].float()).all(), name
-        # (a gradient passes through many more products than an output: one element in 100 000)
-        _assert_doubles(got2[j], got[j], f"{name}(2 dO) vs 2 {name}(dO)", 100_000)
+        # (a gradient passes through many more products than an output, and the state gradient's share from far-away chunks
+        # decays through the denormal range on its way to zero: a few elements in 100 000, by less than 1e-7)
+        _assert_doubles(got2[j], got[j], f"{name}(2 dO) vs 2 {name}(dO)", 20_000)
+        assert float((got2[j].float() - 2 * got[j].float()).abs().max()) <= 1e-7, name
         r = _rel(got[j], ref[j])
         assert r <= (1e-2 if name in ('dg', 'dbeta') else 5e-3), f"{name} against the torch formulation: rel-L2 {r:.3e}"
     r = _rel(got[6], ref[6])
