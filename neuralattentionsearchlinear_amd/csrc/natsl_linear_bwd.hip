@@ -292,8 +292,13 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
 
   const int tid = threadIdx.x, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // the 64-column slices of one chain sit on one XCD (workgroup ids go round the eight XCDs): what they share -- q, k, TmB,
+  // P -- is then fetched from HBM once
   const int nsplit = p.V / 64;
-  const int chain = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
+  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int split = slot % nsplit, chain = (slot / nsplit) * 8 + xcd;
+  if (chain >= n_chains) return;
   const int n = chain / p.H, h = chain % p.H;
   int bos, len, chunk_off, blk0;   // first token, length, first chunk and first selector block of the sequence
   if (p.seqs == nullptr) {
@@ -1089,7 +1094,8 @@ static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* wha
     auto kern = linear_bwd_scan_kernel<DK, DELTA>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)((p.seqs ? p.n_seqs : p.B) * p.H * (p.V / 64))), dim3(L::THREADS), L::TOTAL, stream, p);
+    const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((n_chains + 7) / 8 * 8 * (p.V / 64))), dim3(L::THREADS), L::TOTAL, stream, p);
     const int rc = check_launch(what);
     if (rc != NATSL_OK) return rc;
   }
