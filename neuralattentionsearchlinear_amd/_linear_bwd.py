@@ -211,7 +211,13 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
             _, _, states, v_new, ws = linear_chunk_fwd(kind, qb, kb, vb, gf, bb, h0f, ty, scale, block, flags, False, seqs,
                                                        chunk_states=True)
         tok0, tok1, ch0, ch1, tok_blk = _block_maps(B, T, block, seqs, dev)
-        gsum = _range_sums(gf.view(B * T, H), tok0, tok1).contiguous()                  # [all blocks, H]
+        # sum of g over every selector block [all blocks, H], from the chunk sums the forward left in its workspace (behind
+        # the TmB and P areas: four vectors of 64 floats per chunk and head, the fourth {e^G, G, is_linear, ..}; they are
+        # what the forward's own roll-back decay was made of)
+        units = NTtot * H
+        g_chunk = ws[units * (2 * C * C * 2):].view(f32).view(units, 4 * C)[:, 3 * C + 1].reshape(NTtot, H)
+        one_chunk_blocks = block == C
+        gsum = g_chunk.contiguous() if one_chunk_blocks else _range_sums(g_chunk, ch0, ch1).contiguous()
         d_states = torch.empty_like(states)
         dq, dk, dv = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
         dg = torch.empty(B, T, H, dtype=f32, device=dev)
@@ -233,7 +239,7 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
             # the decay of a rolled-back block acts on every token of the block (rb is non-zero at such a block's last chunk)
             dg.view(B * T, H).add_(rb[ch1 - 1][tok_blk])
         lin = (torch.round(ty[..., 1].float()) == 1).repeat_interleave(H // HN, dim=2).view(-1, H)          # [all blocks, H]
-        dn = torch.where(lin, _range_sums(gate, ch0, ch1), torch.zeros_like(gsum))
+        dn = torch.where(lin, gate if one_chunk_blocks else _range_sums(gate, ch0, ch1), torch.zeros_like(gsum))
         if dnats_for_invalid_blocks:
             # the (zero-valued) gate on the update a block that is not typed linear would have made: its last chunk's
             dn = dn + torch.where(lin, torch.zeros_like(gsum), gate[ch1 - 1])
