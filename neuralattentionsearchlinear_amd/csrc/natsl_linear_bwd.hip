@@ -259,9 +259,10 @@ NATSL_DEVICE float uniform_f(const float x) {
 NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t : 2 * t - 2 + s; }
 
 // LDS of the reverse scan: two stages, each one chunk's inputs exactly as they lie in memory (filled by LDS-DMA).
-template <int DK>
+template <int DK, int NW>
 struct BwdScanLds {
-  static constexpr int KROW = DK * 2, VROW = 128;        // bytes per k / q row, per dO / v_new row (64 columns)
+  static_assert(NW == 4 || (NW == 2 && DK <= 128), "four compute waves, or two where a fifth wave moves the data");
+  static constexpr int KROW = DK * 2, VROW = 32 * NW;    // bytes per k / q row, per dO / v_new row (16 NW columns)
   static constexpr int KB = CB * KROW, VB = CB * VROW, TB = 6 * 1024, SCB = 1024;
   static constexpr int OFF_K = 0, OFF_Q = OFF_K + KB, OFF_DO = OFF_Q + KB, OFF_VN = OFF_DO + VB, OFF_T = OFF_VN + VB,
                        OFF_P = OFF_T + TB, OFF_SC = OFF_P + TB;
@@ -271,8 +272,8 @@ struct BwdScanLds {
   // registers); K = 192 has neither the registers nor the LDS for that, and its compute waves issue the requests themselves.
   static constexpr bool DMAW = DK <= 128, PEND_LDS = DK == 128;
   static constexpr int PEND = (DK / 16) * 4 * 64 * 4;    // bytes per wave
-  static constexpr int TOTAL = 2 * STAGE + (PEND_LDS ? 4 * PEND : 0);
-  static constexpr int THREADS = DMAW ? 320 : 256;
+  static constexpr int TOTAL = 2 * STAGE + (PEND_LDS ? NW * PEND : 0);
+  static constexpr int THREADS = 64 * (DMAW ? NW + 1 : NW);
 };
 
 // The inputs of a chunk are the forward scan's: raw q, k rows (the reciprocal norms ride in the scale vectors), the prep
@@ -282,9 +283,9 @@ struct BwdScanLds {
 // The state gradient uses the forward scan's row order: tile m, lane group g, register r hold K row
 // 32 (m / 2) + 8 g + 4 (m % 2) + r, so that two tiles side by side are eight consecutive K rows (one 16-byte piece of a k / q
 // row as the A operand of K~ dS', one 16-byte store of dS').
-template <int DK, bool DELTA>
-__global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kernel(const LinBwdParams p) {
-  using L = BwdScanLds<DK>;
+template <int DK, bool DELTA, int NW>
+__global__ __launch_bounds__((BwdScanLds<DK, NW>::THREADS)) void linear_bwd_scan_kernel(const LinBwdParams p) {
+  using L = BwdScanLds<DK, NW>;
   constexpr int KT = DK / 16, KS = DK / 32;
   constexpr bool DMAW = L::DMAW, PEND_LDS = L::PEND_LDS;
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // the 64-column slices of one chain sit on one XCD (workgroup ids go round the eight XCDs): what they share -- q, k, TmB,
   // P -- is then fetched from HBM once
-  const int nsplit = p.V / 64;
+  const int nsplit = p.V / (16 * NW);
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int split = slot % nsplit, chain = (slot / nsplit) * 8 + xcd;
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
     bos = p.seqs[n].bos; len = p.seqs[n].eos - bos; chunk_off = p.seqs[n].chunk_off; blk0 = p.seqs[n].bos_nats;
   }
   const int NT = (len + CB - 1) / CB;
-  const int vcol0 = split * 64;
+  const int vcol0 = split * (16 * NW);
   const int col = vcol0 + 16 * wave + x16;
   const int per = p.block / CB;
   const bool decay = (p.flags & NATSL_DECAY_NON_LINEAR) != 0, intra = (p.flags & NATSL_INTRA_CHUNK) != 0;
@@ -315,8 +316,8 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
   auto krow_of = [&](const int m, const int r) { return 32 * (m >> 1) + 8 * g4 + 4 * (m & 1) + r; };
   f32x4 dS[KT], pend[PEND_LDS ? 1 : KT];
   typedef __attribute__((address_space(3))) float* lds_wf_t;
-  const unsigned a_pend = lds0 + 2 * L::STAGE + (wave & 3) * L::PEND + 4 * lane;   // value (m, r) of this lane at + 256 (4 m + r)
-  if (wave < 4) {
+  const unsigned a_pend = lds0 + 2 * L::STAGE + (wave % NW) * L::PEND + 4 * lane;   // value (m, r) of this lane at + 256 (4 m + r)
+  if (wave < NW) {
 #pragma unroll
     for (int m = 0; m < KT; ++m)
 #pragma unroll
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
     }
   };
   if constexpr (DMAW) {
-    if (wave == 4) {
+    if (wave == NW) {
       // ======================= the data-movement wave: all requests of chunk c - 1 during step c =======================
       // (the CU's memory pipe takes one 1 KiB request per ~44 cycles, 61 KiB per chunk: a compute wave that issues them
       // waits for the pipe; this wave has nothing else to do)
@@ -618,8 +619,8 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
         };
         if (wave == 0) { make_operand(0, 0); make_operand(1, 0); }
         else if (wave == 1) { make_operand(0, 1); make_operand(3, 1); }
-        else if (wave == 2) make_operand(1, 1);
-        else make_operand(2, 1);
+        if (wave == NW - 2) make_operand(1, 1);
+        if (wave == NW - 1) make_operand(2, 1);
         __syncthreads();   // P^T
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj)
@@ -744,7 +745,7 @@ __global__ __launch_bounds__(BwdScanLds<DK>::THREADS) void linear_bwd_scan_kerne
       }
       if constexpr (DELTA) {
         const int tk = 16 * (x16 >> 2) + 4 * g4 + (x16 & 3);
-        if (tk < nvalid) p.dbeta_parts[((row0 + tk) * p.H + h) * (p.V / 16) + 4 * split + wave] = dbeta_part;
+        if (tk < nvalid) p.dbeta_parts[((row0 + tk) * p.H + h) * (p.V / 16) + NW * split + wave] = dbeta_part;
       }
       if (c > 0) gs_next = p.gsum_blk[((size_t)blk0 + ((c - 1) * CB) / p.block) * p.H + h];
     }
@@ -1087,16 +1088,38 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
   }
 }
 
+static int bwd_cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <int DK, bool DELTA, int NW>
+static int launch_bwd_scan(const LinBwdParams& p, hipStream_t stream, const char* what) {
+  using L = BwdScanLds<DK, NW>;
+  auto kern = linear_bwd_scan_kernel<DK, DELTA, NW>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
+  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
+  const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
+  hipLaunchKernelGGL(kern, dim3((unsigned)((n_chains + 7) / 8 * 8 * (p.V / (16 * NW)))), dim3(L::THREADS), L::TOTAL, stream, p);
+  return check_launch(what);
+}
+
 template <int DK, bool DELTA>
 static int launch_bwd(const LinBwdParams& p, hipStream_t stream, const char* what) {
   {
-    using L = BwdScanLds<DK>;
-    auto kern = linear_bwd_scan_kernel<DK, DELTA>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
-    if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
-    const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((n_chains + 7) / 8 * 8 * (p.V / 64))), dim3(L::THREADS), L::TOTAL, stream, p);
-    const int rc = check_launch(what);
+    // one workgroup per CU at most (LDS): 32-column workgroups (two compute waves) when the 64-column ones would leave
+    // half of the CUs without work
+    const long long wgs64 = (long long)(p.seqs ? p.n_seqs : p.B) * p.H * (p.V / 64);
+    int rc;
+    if constexpr (DK <= 128) rc = 2 * wgs64 <= bwd_cu_count() ? launch_bwd_scan<DK, DELTA, 2>(p, stream, what) : launch_bwd_scan<DK, DELTA, 4>(p, stream, what);
+    else rc = launch_bwd_scan<DK, DELTA, 4>(p, stream, what);
     if (rc != NATSL_OK) return rc;
   }
   {
