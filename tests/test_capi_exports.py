@@ -85,3 +85,8 @@ def test_backward_entry_rejects_what_is_not_built():
                                 0.1, 7, 1, None, 0, 0, None)
     assert L.natsl_linear_chunk_bwd(*args(96, 64, 64)) == -2 and b"K=96" in L.natsl_last_error()
     assert L.natsl_linear_chunk_bwd(*args(128, 48, 64)) == -2 and b"V=48" in L.natsl_last_error()
+    # both forms read the forward's workspace (the Mamba form its scale vectors)
+    for delta_rule in (1, 0):
+        a = list(args(128, 64, 64))
+        a[0], a[12] = delta_rule, None
+        assert L.natsl_linear_chunk_bwd(*a) == -1 and b"null pointer" in L.natsl_last_error()
