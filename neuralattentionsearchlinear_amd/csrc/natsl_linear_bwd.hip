@@ -860,24 +860,35 @@ __global__ __launch_bounds__(256, DK <= 128 ? 2 : 1) void linear_bwd_chunk_kerne
     store_tokens64(w_do, tid, DOs);
     store_tokens64(w_vn, tid, VNs);
     if (DELTA) store_tokens64(w_dx, tid, DXs);
-    // the state and its gradient as they lie in memory: [64 columns][K]
-    for (int pc = tid; pc < 64 * (DK / 8); pc += 256) {
-      const int v = pc / (DK / 8), seg = pc % (DK / 8);
-      const size_t off = (size_t)(64 * vs + v) * DK + seg * 8;
-      const u32x4 ws = *reinterpret_cast<const u32x4*>(s_src + off);
-      const u32x4 wd = *reinterpret_cast<const u32x4*>(ds_src + off);
-      *reinterpret_cast<u32x4*>(Sn + v * KP + seg * 8) = ws;
-      *reinterpret_cast<u32x4*>(DSn + v * KP + seg * 8) = wd;
-      float fs[8], fd[8];
-      unpack8f(ws, fs);
-      unpack8f(wd, fd);
+    // the state and its gradient as they lie in memory: [64 columns][K]; a thread's pieces are all requested before the
+    // first of them is used
+    {
+      constexpr int NP = 64 * (DK / 8) / 256;
+      u32x4 ws[NP], wd[NP];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sds += fs[e] * fd[e];
-      if (want_rb) {
-        float ff[8];
-        unpack8f(*reinterpret_cast<const u32x4*>(sf_src + off), ff);
+      for (int i = 0; i < NP; ++i) {
+        const int pc = tid + 256 * i, v = pc / (DK / 8), seg = pc % (DK / 8);
+        const size_t off = (size_t)(64 * vs + v) * DK + seg * 8;
+        ws[i] = *reinterpret_cast<const u32x4*>(s_src + off);
+        wd[i] = *reinterpret_cast<const u32x4*>(ds_src + off);
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) srb += ff[e] * fd[e];
+      for (int i = 0; i < NP; ++i) {
+        const int pc = tid + 256 * i, v = pc / (DK / 8), seg = pc % (DK / 8);
+        const size_t off = (size_t)(64 * vs + v) * DK + seg * 8;
+        *reinterpret_cast<u32x4*>(Sn + v * KP + seg * 8) = ws[i];
+        *reinterpret_cast<u32x4*>(DSn + v * KP + seg * 8) = wd[i];
+        float fs[8], fd[8];
+        unpack8f(ws[i], fs);
+        unpack8f(wd[i], fd);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sds += fs[e] * fd[e];
+        if (want_rb) {
+          float ff[8];
+          unpack8f(*reinterpret_cast<const u32x4*>(sf_src + off), ff);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) srb += ff[e] * fd[e];
+        }
       }
     }
     __syncthreads();
