@@ -1,6 +1,7 @@
 """Backward of the linear-recurrent branches (Gated DeltaNet, Mamba2-style SSD) for training.
 
-linear_chunk_backward_hip is the product path: the forward once more with its per-chunk state and v_new outputs, then
+linear_chunk_backward_hip is the product path: the forward's per-chunk state and v_new outputs (kept by the differentiable
+operator from its own forward, else the forward once more), then
 natsl_linear_chunk_bwd (csrc/natsl_linear_bwd.hip: a reverse scan over the chunks and a per-chunk gradient kernel), and the
 few lines of host glue around them (block sums of g, the per-block sums of the gate gradients).  It replaces
 chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart
