@@ -130,9 +130,15 @@ __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams 
     const u32x4* kr = reinterpret_cast<const u32x4*>(p.k + off);
     const u32x4 z = {0u, 0u, 0u, 0u};
     float sq = 0.f, sk = 0.f;
+    u32x4 qa[KL], kb[KL];
 #pragma unroll
     for (int i = 0; i < KL; ++i) {
-      const u32x4 a = ok ? qr[seg + 4 * i] : z, b = ok ? kr[seg + 4 * i] : z;
+      qa[i] = ok ? qr[seg + 4 * i] : z;
+      kb[i] = ok ? kr[seg + 4 * i] : z;
+    }
+#pragma unroll
+    for (int i = 0; i < KL; ++i) {
+      const u32x4 a = qa[i], b = kb[i];
       *reinterpret_cast<u32x4*>(Qs + row * KP + (seg + 4 * i) * 8) = a;
       *reinterpret_cast<u32x4*>(Ks + row * KP + (seg + 4 * i) * 8) = b;
 #pragma unroll

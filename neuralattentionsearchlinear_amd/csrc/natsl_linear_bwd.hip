@@ -293,7 +293,7 @@ __global__ __launch_bounds__((BwdScanLds<DK, NW>::THREADS)) void linear_bwd_scan
 
   const int tid = threadIdx.x, lane = tid & 63, x16 = lane & 15, g4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // the 64-column slices of one chain sit on one XCD (workgroup ids go round the eight XCDs): what they share -- q, k, TmB,
+  // the column slices of one chain sit on one XCD (workgroup ids go round the eight XCDs): what they share -- q, k, TmB,
   // P -- is then fetched from HBM once
   const int nsplit = p.V / (16 * NW);
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
