@@ -77,13 +77,14 @@ def test_linear_branch_backward(case, which):
     _check(out, ref, kind, h0)
 
 
-@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
-def test_packed_sequences_equal_separate_calls(kind):
+@pytest.mark.parametrize("kind,wide", [('gdn', False), ('mamba', False), ('gdn', True), ('mamba', True)])
+def test_packed_sequences_equal_separate_calls(kind, wide):
     """One call over packed sequences gives, bit for bit, what one call per sequence gives (own initial state, own
-    final-state gradient, own blocks; ragged lengths)."""
+    final-state gradient, own blocks; ragged lengths).  The wide case has enough (sequence, head, column slice) chains for the
+    reverse scan to run 64 state columns per workgroup in the packed call and 32 in the calls per sequence: the same bits."""
     from neuralattentionsearchlinear_amd import _linear_bwd as B_
     from neuralattentionsearchlinear_amd.nats_util import pack_sequences
-    lens, H, HN, K, V, block = [200, 64, 450, 129], 4, 2, 128, 64, 128
+    lens, H, HN, K, V, block = ([200, 64, 450, 129], 16, 4, 128, 256, 128) if wide else ([200, 64, 450, 129], 4, 2, 128, 64, 128)
     T = sum(lens)
     cu = [0]
     for n in lens:
