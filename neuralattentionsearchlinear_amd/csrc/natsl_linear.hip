@@ -935,13 +935,21 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
   else hipLaunchKernelGGL(mamba_scale_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, p);
   int rc = check_launch(what);
   if (rc != NATSL_OK) return rc;
-  // Waves per workgroup (16 state columns each): the widest workgroup that still gives every CU one, so that the
-  // chunk's inputs are staged once for as many columns as possible without leaving CUs idle.
+  // Waves per workgroup (16 state columns each).  A CU holds one workgroup (LDS), so a launch takes
+  // ceil(workgroups / CUs) rounds of the chain's length, and a step of a wider workgroup takes longer (measured: 2 700, 3 000,
+  // 4 400 cycles for one, two, four waves): the width with the least rounds x step time.  (Wider also means a chunk's inputs
+  // are staged once for more columns.)
   const long long n_chains = (long long)(p.seqs ? p.n_seqs : p.B) * p.H;
   const int cus = cu_count_linear();
+  auto cost = [&](const int nw, const double step) {
+    const long long wgs = n_chains * (p.V / (16 * nw));
+    return (double)((wgs + cus - 1) / cus) * step;
+  };
   // (K = 192: five waves of that size do not fit the registers of a CU without spilling; three do)
-  if (DK <= 128 && p.V % 64 == 0 && n_chains * (p.V / 64) >= cus) return launch_scan<DK <= 128 ? DK : 128, DELTA, 4>(p, stream, what);
-  if (p.V % 32 == 0 && n_chains * (p.V / 32) >= cus) return launch_scan<DK, DELTA, 2>(p, stream, what);
+  const bool ok4 = DK <= 128 && p.V % 64 == 0, ok2 = p.V % 32 == 0;
+  const double c1 = cost(1, 1.0), c2 = ok2 ? cost(2, 1.1) : 1e30, c4 = ok4 ? cost(4, 1.65) : 1e30;
+  if (c4 <= c2 && c4 <= c1) return launch_scan<DK <= 128 ? DK : 128, DELTA, 4>(p, stream, what);
+  if (c2 <= c1) return launch_scan<DK, DELTA, 2>(p, stream, what);
   return launch_scan<DK, DELTA, 1>(p, stream, what);
 }
 
