@@ -123,15 +123,22 @@ def measured_traffic(workload):
 
 
 def clock_probe(torch, device):
-    """Shader clock and matrix rate of a pure v_mfma_f32_32x32x16_bf16 loop, right after the timed steps."""
-    from neuralattentionsearchlinear_amd import _capi
+    """Shader clock and matrix rate of a pure v_mfma_f32_32x32x16_bf16 loop, right after the timed steps.  The probe kernel
+    is a benchmark aid in a library of its own (csrc/libnatsl_bench.so, built with the package), not part of the C ABI."""
+    import ctypes
+    from neuralattentionsearchlinear_amd import _build, _capi
+    if not os.path.exists(_build.BENCH_LIB):
+        return dict(note="csrc/libnatsl_bench.so is not built: no clock measurement")
+    L = ctypes.CDLL(_build.BENCH_LIB)
+    L.natsl_bench_mfma_clock_probe.restype = ctypes.c_int
+    L.natsl_bench_mfma_clock_probe.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     cus = torch.cuda.get_device_properties(device).multi_processor_count
     n_wg, iters = 2 * cus, 40000
     out = torch.zeros(2 * n_wg, dtype=torch.int64, device=device)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    _capi.check(_capi.lib().natsl_mfma_clock_probe(_capi.ptr(out), n_wg, 2000, _capi.stream_ptr(device)), "natsl_mfma_clock_probe")
+    assert L.natsl_bench_mfma_clock_probe(_capi.ptr(out), n_wg, 2000, _capi.stream_ptr(device)) == 0
     ev[0].record()
-    _capi.check(_capi.lib().natsl_mfma_clock_probe(_capi.ptr(out), n_wg, iters, _capi.stream_ptr(device)), "natsl_mfma_clock_probe")
+    assert L.natsl_bench_mfma_clock_probe(_capi.ptr(out), n_wg, iters, _capi.stream_ptr(device)) == 0
     ev[1].record()
     torch.cuda.synchronize()
     ms = ev[0].elapsed_time(ev[1])
@@ -140,6 +147,13 @@ def clock_probe(torch, device):
     tflops = n_wg * 4 * iters * 4 * 32768.0 / (ms * 1e-3) / 1e12
     return dict(clock_mhz_under_load=mhz, mfma_loop_tflops=tflops,
                 note="pure 32x32x16 bf16 MFMA loop, 2 workgroups x 4 waves per CU, launched right after the timed steps")
+
+
+def softmax_kernel_name(B, T, H, block):
+    """The kernel natsl_softmax_sparse_fwd runs for this problem, as the library itself reports it."""
+    from neuralattentionsearchlinear_amd import _capi
+    v = _capi.lib().natsl_softmax_fwd_variant(B, T, H, H, block, 0)
+    return {0: "softmax_sparse_fwd_kernel<4 waves>", 1: "softmax_sparse_fwd_kernel<8 waves>", 2: "softmax_stream_kernel"}.get(v, f"unknown ({v})")
 
 
 def softmax_flops(types, T, block, K, V):
@@ -539,7 +553,7 @@ def main():
                     launch_ms_alone=lin_alone_ms)
     if f_attn >= f_gdn:
         achieved = f_attn / (sm_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", kernel="softmax_stream_kernel" if T % 256 == 0 and B * H * (T // 256) >= 512 else "softmax_sparse_fwd_kernel", achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
+        roof = dict(bound="mfma", kernel=softmax_kernel_name(B, T, H, w["block"]), achieved=achieved, peak=PEAK_BF16_MFMA_TFLOPS,
                     unit="TFLOP/s", frac=achieved / PEAK_BF16_MFMA_TFLOPS, traffic=(traffic or {}).get("softmax_bytes"),
                     traffic_source=traffic_source, launch_ms=sm_ms, algorithmic_flops=f_attn,
                     # the same kernel with the GPU to itself (branches launched one after the other, outside the timed region)

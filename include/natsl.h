@@ -5,9 +5,13 @@
  * Plain pointers and sizes only: every pointer is DEVICE memory owned by the caller unless a
  * comment says "host"; tensors are dense, token-major [B,T,H,D] as in the reference
  * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:49-50 makes its inputs contiguous).  Nothing here
- * allocates, synchronises with the host or keeps state between calls; work is enqueued on
- * `stream`.  Each function returns NATSL_OK or a negative natsl_status; natsl_last_error()
- * gives the message for the calling thread.
+ * allocates or synchronises with the host; work is enqueued on `stream`.  Two pieces of device
+ * memory belong to the library and are shared by all calls on one GPU: the ticket counters of
+ * natsl_softmax_sparse_fwd's persistent kernel (64 slots used in rotation, each zeroed on the
+ * caller's stream ahead of the launch that uses it) and the scratch of
+ * natsl_attn_masked_fwd_static; their comments say what that means for overlapping calls.
+ * Each function returns NATSL_OK or a negative natsl_status; natsl_last_error() gives the
+ * message for the calling thread.
  *
  * Each entry point names the reference interface it replaces (paths relative to the
  * reference repository root).
@@ -100,14 +104,30 @@ int natsl_route(const void* types, int types_dtype, int B, int TN, int HN, int T
  * called at src/nats/ops/mixed_ops/mixed_attn_gdn.py:111-117.
  * K, V in {64, 128}.  Unpacked input of whole 256-query tiles, at least two per compute unit (T % 256 == 0,
  * T <= 65536, block <= 2048), runs as a persistent kernel whose work queues are ticket counters in device
- * memory owned by the library (64 slots in rotation, each launch sets its slot back to zero): launches may
- * overlap across streams; NATSL_SOFTMAX_NO_STREAM=1 in the environment selects the per-tile kernel, whose
- * results are the same bit for bit. */
+ * memory owned by the library: 64 slots used in rotation, the launch's slot zeroed by a small fill kernel
+ * enqueued on `stream` right before it (both kernels can be captured into a HIP graph).  Launches may overlap
+ * across streams as long as fewer than 64 of them are in flight on one GPU; a captured launch keeps the slot it
+ * drew at capture, so replay it on the stream that also carries the eager launches. */
 int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                              const void* types, int types_dtype, const int32_t* nats_block_indices,
                              const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
                              int V, int TN, int block, float scale, int same_block_visible, int dtype,
                              const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
+
+/* The same operation with the same results bit for bit, always as one workgroup per query tile (what
+ * natsl_softmax_sparse_fwd itself runs for packed input, ragged lengths and small problems): for callers that
+ * want no library-owned device state in the launch, and the regression check of the persistent kernel.
+ * Same reference interface as natsl_softmax_sparse_fwd. */
+int natsl_softmax_sparse_fwd_per_tile(const void* q, const void* k, const void* v, void* o, float* lse,
+                             const void* types, int types_dtype, const int32_t* nats_block_indices,
+                             const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
+                             int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                             const natsl_seq_row* seqs, int n_seqs, int total_units, natsl_stream_t stream);
+
+/* Which kernel natsl_softmax_sparse_fwd runs for a problem on the current device (host-side query, no launch;
+ * the choice that src/nats/ops/attns/attns.py:1497-1512 leaves to Triton's autotuner). */
+enum natsl_softmax_variant { NATSL_SOFTMAX_TILE_128 = 0, NATSL_SOFTMAX_TILE_256 = 1, NATSL_SOFTMAX_PERSISTENT = 2 };
+int natsl_softmax_fwd_variant(int B, int T, int HQ, int HKV, int block, int packed);
 
 
 /* Backward of the softmax branch: dq [B,T,HQ,K], dk [B,T,HKV,K], dv [B,T,HKV,V] (bf16, summed over the query heads of
@@ -326,11 +346,6 @@ int natsl_kv_compact(const void* src_k, const void* src_v, long long src_tokens,
                      int HN, int K, int V, int dtype, int block, int NB, int n_complete, int tail_dst, int tail_tokens,
                      natsl_stream_t stream);
 
-/* Measurement aid (no counterpart in the reference; used by the benchmark only): n_workgroups workgroups of 4 waves each
- * run `iters` rounds of four independent 32x32x16 bf16 matrix instructions per wave (iters * 4 * 32768 FLOPs per wave) and
- * write, per workgroup, out[2i] = shader-clock cycles and out[2i+1] = ticks of the constant 100 MHz counter the loop took:
- * cycles / ticks * 100 is the shader clock in MHz under a dense matrix load. */
-int natsl_mfma_clock_probe(unsigned long long* out, int n_workgroups, int iters, natsl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -1,4 +1,5 @@
-"""Builds csrc/*.hip into csrc/libnatsl.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+"""Builds csrc/*.hip into csrc/libnatsl.so for gfx950 with hipcc (cross-compiles without a GPU), and the benchmark's
+clock probe (csrc/bench/) into csrc/libnatsl_bench.so, which is not part of the C ABI."""
 from __future__ import annotations
 
 import os
@@ -8,7 +9,8 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libnatsl.so")
-SOURCES = ["natsl_route.hip", "natsl_softmax.hip", "natsl_softmax_bwd.hip", "natsl_linear.hip", "natsl_linear_bwd.hip", "natsl_norm_gate.hip", "natsl_conv.hip", "natsl_decode.hip", "natsl_cache.hip", "natsl_probe.hip"]
+BENCH_LIB = os.path.join(CSRC, "libnatsl_bench.so")
+SOURCES = ["natsl_route.hip", "natsl_softmax.hip", "natsl_softmax_bwd.hip", "natsl_linear.hip", "natsl_linear_bwd.hip", "natsl_norm_gate.hip", "natsl_conv.hip", "natsl_decode.hip", "natsl_cache.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
     # keep the compiler from forming packed-fp32 VALU ops
@@ -45,6 +47,9 @@ def build(verbose: bool = False) -> str:
     r = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
+    r = subprocess.run([hipcc, *FLAGS, "-shared", os.path.join(CSRC, "bench", "bench_probe.hip"), "-o", BENCH_LIB], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on bench/bench_probe.hip:\n{r.stderr}")
     return LIB
 
 

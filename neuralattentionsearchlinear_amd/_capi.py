@@ -29,6 +29,10 @@ _SIGNATURES = {
     "natsl_softmax_sparse_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                          c_void_p, c_int, c_int, c_void_p]),
+    "natsl_softmax_sparse_fwd_per_tile": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                         c_void_p, c_int, c_int, c_void_p]),
+    "natsl_softmax_fwd_variant": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "natsl_softmax_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "natsl_softmax_sparse_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -67,7 +71,6 @@ _SIGNATURES = {
     "natsl_attn_masked_static_scratch_bytes": (c_size_t, []),
     "natsl_attn_masked_fwd_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                              c_int, c_int, c_float, c_int, c_void_p]),
-    "natsl_mfma_clock_probe": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "natsl_kv_compact": (c_int, [c_void_p, c_void_p, c_longlong, c_int, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }

@@ -1,12 +1,12 @@
-// Measurement aid: a dense bf16 matrix-core loop that reports how fast the shader clock ran while it executed.
+// Benchmark aid, NOT part of libnatsl.so or of the C ABI in include/natsl.h: built into csrc/libnatsl_bench.so, which only
+// bench.py loads.  A dense bf16 matrix-core loop that reports how fast the shader clock ran while it executed.
 //
 // Roofline fractions are quoted against the published peak, which assumes the 2.4 GHz boost clock; under a
 // sustained matrix load the clock settles lower.  This kernel runs `iters` rounds of four independent
 // v_mfma_f32_32x32x16_bf16 per wave on every workgroup and records, per workgroup, the shader-clock cycles and the
 // ticks of the constant 100 MHz real-time counter it took, so that a benchmark can print the clock under load and the
 // matrix rate a pure MFMA loop reaches on the same box right after its timed steps.
-#include "natsl_device.h"
-#include "natsl_host.h"
+#include "../natsl_device.h"
 
 namespace natsl {
 
@@ -44,8 +44,10 @@ __global__ __launch_bounds__(256) void mfma_clock_probe_kernel(unsigned long lon
 
 using namespace natsl;
 
-extern "C" int natsl_mfma_clock_probe(unsigned long long* out, int n_workgroups, int iters, natsl_stream_t stream) {
-  if (!out || n_workgroups <= 0 || iters <= 0) return fail(NATSL_ERR_INVALID, "natsl_mfma_clock_probe: bad argument");
+// out[2i] = shader-clock cycles, out[2i+1] = ticks of the constant 100 MHz counter that workgroup i's loop took
+// (iters * 4 * 32768 FLOPs per wave, 4 waves per workgroup).  Returns 0, or -1 for a bad argument / refused launch.
+extern "C" int natsl_bench_mfma_clock_probe(unsigned long long* out, int n_workgroups, int iters, void* stream) {
+  if (!out || n_workgroups <= 0 || iters <= 0) return -1;
   hipLaunchKernelGGL(mfma_clock_probe_kernel, dim3((unsigned)n_workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, iters);
-  return check_launch("natsl_mfma_clock_probe");
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -14,7 +14,6 @@
 #include "natsl_host.h"
 #include <atomic>
 #include <mutex>
-#include <stdlib.h>
 #include <type_traits>
 
 namespace natsl {
@@ -976,7 +975,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
 // Tiles come from eight queues, one per XCD (a workgroup reads which XCD it runs on): queue x lists the tiles of
 // (batch, head) pairs x, x+8, ... pair after pair, heaviest tile first, so the tiles that share a pair's K/V run
 // together on one L2; a workgroup whose queue is used up takes from the others.  A queue is a ticket counter in device
-// memory; the last workgroup to finish sets the counters back to zero.
+// memory, zeroed on the launch's stream by a small fill kernel right before the launch (see launch_softmax_stream).
 constexpr int STREAM_ROWS = 1088;  // chunk table of a tile: up to 1024 + 32 chunks of its own and four of the next tile (two tiles' tables are resident)
 constexpr int STREAM_QUEUES = 8;
 constexpr int STREAM_SLOT_WORDS = 16;  // per launch slot: 8 ticket counters, 1 count of finished workgroups
@@ -1443,15 +1442,19 @@ void softmax_stream_kernel(const SoftmaxParams p, unsigned* queue) {
     a ^= 1;
   }
 
-  // ---- the last workgroup to finish sets the queues back to zero for the next launch --------------------------------
-  if (tid == 0) {
-    __threadfence();
-    const unsigned done = atomicAdd(&queue[STREAM_QUEUES], 1u);
-    if (done == gridDim.x - 1) {
-#pragma unroll
-      for (int i = 0; i <= STREAM_QUEUES; ++i) atomicExch(&queue[i], 0u);
-    }
-  }
+}
+
+// The LDS reservation of a kernel is an attribute of the function per device: set when a device first runs it.
+static int reserve_lds(const void* kern, std::atomic<unsigned long long>& done, size_t lds) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot name the current device (%s)", hipGetErrorString(e));
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (dev < 64 && (done.load(std::memory_order_acquire) & bit)) return NATSL_OK;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+  if (dev < 64) done.fetch_or(bit, std::memory_order_release);
+  return NATSL_OK;
 }
 
 template <int DK, int DV, int NWAVES>
@@ -1463,8 +1466,8 @@ static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   const size_t ring = ((size_t)4 * 64 * DK + (size_t)2 * 64 * DV + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;  // 8 waves: four K tiles, two raw and three transposed V tiles, 1 KiB aligned
   if (NWAVES == 8 && ring > lds) lds = ring;
   auto kern = softmax_sparse_fwd_kernel<DK, DV, NWAVES>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+  static std::atomic<unsigned long long> reserved{0};
+  if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), reserved, lds)) return rc;
   const long long grid = p.seqs ? (long long)p.total_tiles * (QTILE_TABLE / QTILE) * p.HQ
                                 : (long long)8 * ((p.B * p.HQ + 7) / 8) * ((p.T + QTILE - 1) / QTILE);
   if (grid <= 0) return NATSL_OK;
@@ -1472,11 +1475,20 @@ static int launch_softmax(const SoftmaxParams& p, hipStream_t stream) {
   return check_launch("natsl_softmax_sparse_fwd");
 }
 
-// Ticket counters of the persistent kernel: zero when the library is loaded, and set back to zero by every launch's last
-// workgroup.  Consecutive launches rotate through the slots, so launches that overlap on one GPU (two streams) do not
-// share counters unless STREAM_SLOTS launches lie between them.
+// Ticket counters of the persistent kernel: library-owned device memory, STREAM_SLOTS slots of counters.  Consecutive
+// launches rotate through the slots, and each launch is preceded ON ITS STREAM by a fill kernel that zeroes its slot (a
+// kernel, not hipMemsetAsync, so that both can be captured into a HIP graph and replayed).  Nothing is left to set
+// back afterwards: a launch that was cut short cannot poison a later one.  Two launches use one slot at the same time
+// only if STREAM_SLOTS launches lie between them and both are still running, or if a captured graph (whose slot was
+// fixed at capture) is replayed next to an eager launch that drew the same slot; the launches would then share each
+// other's tickets and leave tiles uncomputed, so keep fewer than STREAM_SLOTS launches of this entry in flight per GPU
+// and replay captured launches on the stream that also carries the eager ones.
 constexpr int STREAM_SLOTS = 64;
 static __device__ __align__(256) unsigned stream_queues[STREAM_SLOTS * STREAM_SLOT_WORDS];
+
+__global__ void stream_queue_clear_kernel(unsigned* slot) {
+  if (threadIdx.x < STREAM_SLOT_WORDS) slot[threadIdx.x] = 0u;
+}
 
 struct StreamDevice {
   unsigned* queues = nullptr;
@@ -1513,25 +1525,42 @@ static const StreamDevice* stream_device(int* rc) {
 template <int DK, int DV>
 static int launch_softmax_stream(const SoftmaxParams& p, const StreamDevice* d, hipStream_t stream) {
   static std::atomic<unsigned> launches{0};
+  static std::atomic<unsigned long long> reserved{0};
   const size_t lds = ((size_t)4 * 64 * DK + (size_t)2 * 64 * DV + (size_t)3 * DV * VTP) * sizeof(bf16_t) + 1024;
   auto kern = softmax_stream_kernel<DK, DV>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+  if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), reserved, lds)) return rc;
   unsigned* queue = d->queues + (size_t)(launches.fetch_add(1) % STREAM_SLOTS) * STREAM_SLOT_WORDS;
+  hipLaunchKernelGGL(stream_queue_clear_kernel, dim3(1), dim3(64), 0, stream, queue);
   hipLaunchKernelGGL(kern, dim3((unsigned)d->cus), dim3(512), lds, stream, p, queue);
   return check_launch("natsl_softmax_sparse_fwd");
+}
+
+// Which kernel natsl_softmax_sparse_fwd runs for a problem: the persistent one for unpacked input of whole 256-query
+// tiles, at least two per compute unit (its per-tile saving needs a tile to follow); else one workgroup per tile, of 256
+// queries on 8 waves once there is at least one such tile per compute unit (measured: from there on that shape is the
+// faster one; below, 128-query tiles fill more compute units).
+static int softmax_variant(int B, int T, int HQ, int HKV, int block, bool packed, bool allow_persistent, const StreamDevice** sd, int* rc) {
+  *sd = nullptr;
+  *rc = NATSL_OK;
+  if (allow_persistent && !packed && T % 256 == 0 && T <= 65536 && block <= 2048 && (long long)B * T * HKV < (1ll << 31)) {
+    const StreamDevice* d = stream_device(rc);
+    if (!d) return -1;
+    if ((long long)B * HQ * (T / 256) >= 2ll * d->cus) {
+      *sd = d;
+      return NATSL_SOFTMAX_PERSISTENT;
+    }
+  }
+  return (long long)B * HQ * cdiv(T, 256) >= 256 ? NATSL_SOFTMAX_TILE_256 : NATSL_SOFTMAX_TILE_128;
 }
 
 }  // namespace natsl
 
 using namespace natsl;
 
-extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
-                                        const void* types, int types_dtype, const int32_t* nats_block_indices,
-                                        const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
-                                        int V, int TN, int block, float scale, int same_block_visible, int dtype,
-                                        const natsl_seq_row* seqs, int n_seqs, int total_units,
-                                        natsl_stream_t stream) {
+static int softmax_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const void* types, int types_dtype,
+                       const int32_t* nats_block_indices, const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
+                       int V, int TN, int block, float scale, int same_block_visible, int dtype, const natsl_seq_row* seqs,
+                       int n_seqs, int total_units, natsl_stream_t stream, bool allow_persistent) {
   if (!q || !k || !v || !o || !lse || !types || !nats_block_indices || !n_nats_blocks)
     return fail(NATSL_ERR_INVALID, "softmax: null pointer argument");
   if (dtype != NATSL_BF16) return fail(NATSL_ERR_UNSUPPORTED, "softmax: only bf16 tensors are supported (got dtype %d)", dtype);
@@ -1541,6 +1570,8 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   if (block < 64 || block % 64) return fail(NATSL_ERR_UNSUPPORTED, "softmax: block size %d must be a multiple of 64", block);
   if (seqs ? (B != 1 || n_seqs <= 0) : (TN != cdiv(T, block)))
     return fail(NATSL_ERR_INVALID, "softmax: TN=%d does not match T=%d, block=%d (or packed input with B != 1)", TN, T, block);
+  if (!((K == 64 || K == 128) && (V == 64 || V == 128)))
+    return fail(NATSL_ERR_UNSUPPORTED, "softmax: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", K, V);
 
   SoftmaxParams p;
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (bf16_t*)o; p.lse = lse;
@@ -1553,21 +1584,12 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   p.same_block = same_block_visible ? 1 : 0;
   p.g_kv = HQ / HKV;
   p.g_n = HQ / HN;
-  // 256-query tiles on 8 waves once there is at least one of them per CU (measured: from there on that shape is the
-  // faster one; below, the 128-query tiles fill more CUs)
-  p.variant = (long long)B * HQ * cdiv(T, 256) >= 256 ? 8 : 4;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (!((K == 64 || K == 128) && (V == 64 || V == 128)))
-    return fail(NATSL_ERR_UNSUPPORTED, "softmax: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", K, V);
-  // Whole 256-query tiles, at least two per CU: the persistent kernel (its per-tile saving needs a tile to follow)
   const StreamDevice* sd = nullptr;
-  if (!seqs && T % 256 == 0 && T <= 65536 && block <= 2048 && (long long)B * T * HKV < (1ll << 31) &&
-      getenv("NATSL_SOFTMAX_NO_STREAM") == nullptr) {
-    int rc;
-    sd = stream_device(&rc);
-    if (!sd) return rc;
-    if ((long long)B * HQ * (T / 256) < 2ll * sd->cus) sd = nullptr;
-  }
+  int rc;
+  const int variant = softmax_variant(B, T, HQ, HKV, block, seqs != nullptr, allow_persistent, &sd, &rc);
+  if (variant < 0) return rc;
+  p.variant = variant == NATSL_SOFTMAX_TILE_128 ? 4 : 8;
 #define NATSL_SM(KK, VV)                                              \
   if (K == KK && V == VV) {                                           \
     if (sd) return launch_softmax_stream<KK, VV>(p, sd, s);           \
@@ -1579,4 +1601,31 @@ extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void
   NATSL_SM(128, 64)
 #undef NATSL_SM
   return fail(NATSL_ERR_UNSUPPORTED, "softmax: head dims K=%d, V=%d not built (supported: 64/128 x 64/128)", K, V);
+}
+
+extern "C" int natsl_softmax_sparse_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                                        const void* types, int types_dtype, const int32_t* nats_block_indices,
+                                        const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
+                                        int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                                        const natsl_seq_row* seqs, int n_seqs, int total_units,
+                                        natsl_stream_t stream) {
+  return softmax_fwd(q, k, v, o, lse, types, types_dtype, nats_block_indices, n_nats_blocks, B, T, HQ, HKV, HN, K, V, TN, block,
+                     scale, same_block_visible, dtype, seqs, n_seqs, total_units, stream, true);
+}
+
+extern "C" int natsl_softmax_sparse_fwd_per_tile(const void* q, const void* k, const void* v, void* o, float* lse,
+                                                 const void* types, int types_dtype, const int32_t* nats_block_indices,
+                                                 const int32_t* n_nats_blocks, int B, int T, int HQ, int HKV, int HN, int K,
+                                                 int V, int TN, int block, float scale, int same_block_visible, int dtype,
+                                                 const natsl_seq_row* seqs, int n_seqs, int total_units,
+                                                 natsl_stream_t stream) {
+  return softmax_fwd(q, k, v, o, lse, types, types_dtype, nats_block_indices, n_nats_blocks, B, T, HQ, HKV, HN, K, V, TN, block,
+                     scale, same_block_visible, dtype, seqs, n_seqs, total_units, stream, false);
+}
+
+extern "C" int natsl_softmax_fwd_variant(int B, int T, int HQ, int HKV, int block, int packed) {
+  const StreamDevice* sd = nullptr;
+  int rc;
+  const int variant = softmax_variant(B, T, HQ, HKV, block, packed != 0, true, &sd, &rc);
+  return variant < 0 ? rc : variant;
 }

@@ -1,7 +1,5 @@
 """GPU parity of the persistent softmax kernel (whole 256-query tiles, at least two per CU): against the oracle,
 bit for bit against the per-tile kernel (same chunk order, same arithmetic), and its work queues across launches."""
-import os
-
 import pytest
 import torch
 
@@ -18,19 +16,23 @@ def _inputs(B, T, HQ, H, HN, K, V, block, p_attn, seed, dev):
 
 
 def _call(qd, kd, vd, tyd, K, block, same_block, persistent=True):
-    from neuralattentionsearchlinear_amd import nats_util
-    from neuralattentionsearchlinear_amd.attns import parallel_attn_nats_fwd
+    """The softmax branch through the C ABI: natsl_softmax_sparse_fwd (picks the persistent kernel for these shapes), or
+    natsl_softmax_sparse_fwd_per_tile (one workgroup per query tile, the same results)."""
+    from neuralattentionsearchlinear_amd import _capi, nats_util
     r = nats_util.route(tyd, qd.shape[1], block)
-    old = os.environ.pop("NATSL_SOFTMAX_NO_STREAM", None)
-    if not persistent:
-        os.environ["NATSL_SOFTMAX_NO_STREAM"] = "1"
-    try:
-        o, lse, _ = parallel_attn_nats_fwd(qd, kd, vd, tyd, r['nats_block_indices'], None, K ** -0.5, block,
-                                           compute_incomplete_chunk_scores=same_block, n_nats_blocks=r['n_nats_blocks'])
-    finally:
-        os.environ.pop("NATSL_SOFTMAX_NO_STREAM", None)
-        if old is not None:
-            os.environ["NATSL_SOFTMAX_NO_STREAM"] = old
+    B, T, HQ, _ = qd.shape
+    H, V = kd.shape[2], vd.shape[-1]
+    TN, HN = tyd.shape[1], tyd.shape[2]
+    o = torch.empty(B, T, HQ, V, dtype=vd.dtype, device=qd.device)
+    lse = torch.empty(B, T, HQ, dtype=torch.float32, device=qd.device)
+    L = _capi.lib()
+    fn = L.natsl_softmax_sparse_fwd if persistent else L.natsl_softmax_sparse_fwd_per_tile
+    if persistent:
+        assert L.natsl_softmax_fwd_variant(B, T, HQ, H, block, 0) == 2, "shape does not reach the persistent kernel on this GPU"
+    rc = fn(_capi.ptr(qd), _capi.ptr(kd), _capi.ptr(vd), _capi.ptr(o), _capi.ptr(lse), _capi.ptr(tyd), _capi.dtype_code(tyd.dtype),
+            _capi.ptr(r['nats_block_indices']), _capi.ptr(r['n_nats_blocks']), B, T, HQ, H, HN, K, V, TN, block, float(K ** -0.5),
+            int(bool(same_block)), _capi.dtype_code(qd.dtype), None, 0, 0, _capi.stream_ptr(qd.device))
+    _capi.check(rc, "natsl_softmax_sparse_fwd")
     return o, lse
 
 
@@ -76,7 +78,8 @@ def test_persistent_kernel_equals_the_per_tile_kernel(B, T, HQ, H, HN, K, V, blo
 
 
 def test_persistent_kernel_queues_across_launches_and_streams():
-    """The ticket counters are shared device state: set back by every launch, one slot per launch in rotation."""
+    """The ticket counters are shared device state: one slot per launch in rotation, zeroed on the launch's stream right
+    before it."""
     B, T, HQ, H, HN, K, V, block = 4, 4096, 16, 16, 16, 128, 128, 64
     dev = torch.device('cuda:0')
     assert _enough_tiles(B, HQ, T)
@@ -102,3 +105,40 @@ def test_persistent_kernel_queues_across_launches_and_streams():
     s2.synchronize()
     for (o, l), (orf, lrf) in outs:
         assert torch.equal(o, orf) and torch.equal(l, lrf)
+
+
+def test_persistent_kernel_in_a_captured_graph():
+    """The launch (queue fill kernel + persistent kernel) replays from a HIP graph: every replay, with eager work and
+    synchronisations between the replays, gives the eager result."""
+    B, T, HQ, H, HN, K, V, block = 4, 4096, 16, 16, 16, 128, 128, 64
+    dev = torch.device('cuda:0')
+    assert _enough_tiles(B, HQ, T)
+    _, _, _, _, qd, kd, vd, tyd = _inputs(B, T, HQ, H, HN, K, V, block, 0.25, 7, dev)
+    from neuralattentionsearchlinear_amd import _capi, nats_util
+    r = nats_util.route(tyd, T, block)
+    o_ref, l_ref = _call(qd, kd, vd, tyd, K, block, True, persistent=False)
+    o = torch.empty_like(o_ref)
+    lse = torch.empty_like(l_ref)
+    L = _capi.lib()
+
+    def launch():
+        rc = L.natsl_softmax_sparse_fwd(_capi.ptr(qd), _capi.ptr(kd), _capi.ptr(vd), _capi.ptr(o), _capi.ptr(lse), _capi.ptr(tyd),
+                                        _capi.dtype_code(tyd.dtype), _capi.ptr(r['nats_block_indices']), _capi.ptr(r['n_nats_blocks']),
+                                        B, T, HQ, H, HN, K, V, tyd.shape[1], block, float(K ** -0.5), 1, _capi.dtype_code(qd.dtype),
+                                        None, 0, 0, _capi.stream_ptr(dev))
+        _capi.check(rc, "natsl_softmax_sparse_fwd")
+
+    launch()   # first use on the device outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch()
+    for i in range(4):
+        o.fill_(float('nan'))
+        lse.fill_(float('nan'))
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref) and torch.equal(lse, l_ref), f"replay {i}"
+        if i & 1:
+            _call(qd, kd, vd, tyd, K, block, True)   # an eager launch between replays, on the same stream
+            torch.cuda.synchronize()
