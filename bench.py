@@ -388,7 +388,9 @@ def bench_layer(args):
     projections are torch GEMMs, everything else this package's kernels.  'train' = forward + backward of a scalar loss."""
     import torch
     from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd import _mixed_common
     from neuralattentionsearchlinear_amd.natsl_attn_gdn import NeuralAttentionSearchLinearAttnGDN
+    _mixed_common.SAVE_CHUNK_STATES = dict(auto=None, on=True, off=False)[args.save_chunk_states]
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
         sys.exit(2)
@@ -419,12 +421,14 @@ def bench_layer(args):
     print(json.dumps(dict(
         metric="GDN layer (340M geometry) " + ("training step" if w["train"] else "forward") + " tokens/sec bf16", value=w["B"] * w["T"] / (ms * 1e-3),
         unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms, higher_is_better=True, scaling="weak",
-        vs_baseline=None, dtype="bf16", data="synthetic", config=dict(workload=args.workload, **w))))
+        vs_baseline=None, dtype="bf16", data="synthetic", config=dict(workload=args.workload, save_chunk_states=args.save_chunk_states, **w))))
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--save-chunk-states", choices=["auto", "on", "off"], default="auto",
+                    help="layer workloads: what the differentiable operator keeps for the linear backward (_mixed_common.SAVE_CHUNK_STATES)")
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="hybrid_gdn_B8_T8192_H16_d128_p25", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS) + sorted(CACHE_WORKLOADS) + sorted(BACKWARD_WORKLOADS) + sorted(LINEAR_BACKWARD_WORKLOADS) + sorted(LAYER_WORKLOADS))

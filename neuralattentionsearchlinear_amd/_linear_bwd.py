@@ -125,7 +125,17 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
     types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None; seqs: packed sequences (B = 1) or None; saved: what
     linear_chunk_fwd(..., chunk_states=True) returned after (o, final_state) on these same inputs, if the caller kept it.  The
     HIP kernels (natsl_linear_chunk_bwd) where they are built (K in 64/128/192, V a multiple of 64), else the torch formulation
-    below, one sequence at a time."""
+    below, one sequence at a time.
+
+    dnats_for_invalid_blocks with block > 64 raises NotImplementedError: for a block of several chunks that is not typed
+    linear the reference sums a virtual key gradient v . dh over EVERY chunk of the block
+    (src/nats/ops/common/chunk_o.py:446-491, summed per block at :1571), each against the dh its compacted reverse scan holds
+    at that chunk (src/nats/ops/common/chunk_delta_h.py:492-509); that definition has not been restated here.  With one
+    chunk per block it is the gradient of a zero gate on the block's state update, which is what this function returns."""
+    if dnats_for_invalid_blocks and block > C:
+        raise NotImplementedError(
+            f"compute_dnats_for_invalid_blocks_linear_att=True is built for nats_block_size == {C} only (got {block}): "
+            "pass compute_dnats_for_invalid_blocks_linear_att=False (the layers' default)")
     if hip_backward_is_built(q.shape[-1], v.shape[-1]):
         return linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
                                          dnats_for_invalid_blocks, seqs, saved)
@@ -242,7 +252,7 @@ def linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, d
         lin = (torch.round(ty[..., 1].float()) == 1).repeat_interleave(H // HN, dim=2).view(-1, H)          # [all blocks, H]
         dn = torch.where(lin, gate if one_chunk_blocks else _range_sums(gate, ch0, ch1), torch.zeros_like(gsum))
         if dnats_for_invalid_blocks:
-            # the (zero-valued) gate on the update a block that is not typed linear would have made: its last chunk's
+            # the (zero-valued) gate on the update a block that is not typed linear would have made (one chunk per block here)
             dn = dn + torch.where(lin, torch.zeros_like(gsum), gate[ch1 - 1])
         dn = dn.view(B, NB, HN, H // HN).sum(3)
     return (dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), dg, None if dbeta is None else dbeta.to(beta.dtype), dh0, dn)

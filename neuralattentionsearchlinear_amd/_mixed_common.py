@@ -24,12 +24,17 @@ TIMING_HOOK = None
 # machine alone, running them side by side gains nothing (measured) and only blurs timings.
 CONCURRENT_BRANCHES = None
 
-# What the differentiable operator keeps from its forward for the linear branch's backward.  True: the state entering every
-# chunk (bf16, K*V per chunk and head), v_new and the prep kernel's workspace (17 KiB per chunk and head) stay in device
-# memory until the backward, which then starts at its reverse scan.  False: only the inputs are kept and the backward runs
-# the forward's two kernels once more, as the reference's backward does
-# (src/nats/ops/gated_delta_rule/chunk.py:170-332 recomputes h).  The gradients are the same bit for bit either way.
-SAVE_CHUNK_STATES = True
+# What the differentiable operator keeps from its forward for the linear branch's backward.  Keeping means: the state entering
+# every chunk (bf16, K*V per chunk and head), v_new (64*V bf16) and the prep kernel's workspace (17 KiB) stay in device memory
+# until the backward, which then starts at its reverse scan - about 66 KiB per chunk and head at K = V = 128, 1.1 GB per call
+# at B8 T8192 H16.  Not keeping means: only the inputs are saved and the backward runs the forward's two kernels once more, as
+# the reference's backward does (src/nats/ops/gated_delta_rule/chunk.py:170-332 recomputes h); a model that fits in memory
+# under the reference then fits here.  The gradients are the same bit for bit either way.
+#   SAVE_CHUNK_STATES = None  (default) keep only when what would be kept is at most SAVE_CHUNK_STATES_MAX_BYTES per call
+#                     = True  always keep        = False  never keep
+SAVE_CHUNK_STATES = None
+SAVE_CHUNK_STATES_MAX_BYTES = 64 << 20
+_PREP_WORKSPACE_BYTES = 17 * 1024   # per chunk and head (csrc/natsl_linear.hip)
 _SCAN_COLUMNS_PER_WG = 16   # state columns of the scan's narrowest workgroup (csrc/natsl_linear.hip)
 
 
@@ -38,6 +43,17 @@ def _run_side_by_side(dev, n_chains: int, V: int) -> bool:
         return bool(CONCURRENT_BRANCHES)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     return n_chains * (V // _SCAN_COLUMNS_PER_WG) < cus
+
+
+def _keep_chunk_states(q, v, cu_seqlens) -> bool:
+    """Whether the differentiable forward keeps the linear branch's chunk states (see SAVE_CHUNK_STATES)."""
+    if SAVE_CHUNK_STATES is not None:
+        return bool(SAVE_CHUNK_STATES)
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    n_seq = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    chunks = -(-B * T // CHUNK_SIZE) + n_seq                       # upper bound on the chunks of all sequences
+    return chunks * H * (2 * K * V + 2 * CHUNK_SIZE * V + _PREP_WORKSPACE_BYTES) <= SAVE_CHUNK_STATES_MAX_BYTES
 
 
 def _mark(name, stream):
@@ -211,7 +227,7 @@ class _MixedFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, cfg, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types):
         from ._linear_bwd import hip_backward_is_built
-        keep = bool(SAVE_CHUNK_STATES) and hip_backward_is_built(q_lattn.shape[-1], v_lattn.shape[-1])
+        keep = _keep_chunk_states(q_lattn, v_lattn, cfg['cu_seqlens']) and hip_backward_is_built(q_lattn.shape[-1], v_lattn.shape[-1])
         with torch.no_grad():
             o_lin, o_attn, ht, aux = _mixed_forward_impl(
                 cfg['kind'], q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types,

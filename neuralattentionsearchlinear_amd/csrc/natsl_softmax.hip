@@ -978,7 +978,7 @@ void softmax_sparse_fwd_kernel(const SoftmaxParams p) {
 // memory, zeroed on the launch's stream by a small fill kernel right before the launch (see launch_softmax_stream).
 constexpr int STREAM_ROWS = 1088;  // chunk table of a tile: up to 1024 + 32 chunks of its own and four of the next tile (two tiles' tables are resident)
 constexpr int STREAM_QUEUES = 8;
-constexpr int STREAM_SLOT_WORDS = 16;  // per launch slot: 8 ticket counters, 1 count of finished workgroups
+constexpr int STREAM_SLOT_WORDS = 16;  // per launch slot: 8 ticket counters (one per XCD), the rest unused padding to a 64-byte line
 
 struct StreamTile {
   int valid, n, hq, tile, hkv, hn, dstart, dblk;  // the tile AFTER the one this record belongs to

@@ -3,8 +3,9 @@
 The reference takes these from flash-linear-attention (ShortConvolution, RMSNorm, L2Norm) and from
 src/nats/modules/fused_norm_gate.py (FusedMultiInputRMSNormGated); parameter names are kept so that
 reference checkpoints load.  Projections stay torch ops (rocBLAS); the short convolution, the RMS / L2 row norms and the
-two-input norm-gate run HIP kernels (natsl_short_conv_fwd, natsl_row_norm_fwd, natsl_norm_gate_fwd) in the forward, with
-torch-evaluated gradients.
+two-input norm-gate run HIP kernels in the forward (natsl_short_conv_fwd, natsl_row_norm_fwd, natsl_norm_gate_fwd) and in
+the backward (natsl_short_conv_bwd, natsl_row_norm_bwd, natsl_norm_gate_bwd) wherever the forward does; the torch formulas
+below cover CPU tensors and widths the kernels are not built for.
 """
 from __future__ import annotations
 

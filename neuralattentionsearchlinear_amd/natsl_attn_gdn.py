@@ -2,8 +2,10 @@
 names of the reference layer (src/nats/layers/natsl_attn_gdn.py:64-666).
 
 Projections, short convolutions and norms are torch; block pooling, the selector, the mixed operator
-and the output norm-gate are the HIP kernels of this package.  Training works: the softmax branch's backward is a HIP
-kernel, the linear branch, the pooling and the norm-gate differentiate through torch operations.  With a NAtSCache
+and the output norm-gate are the HIP kernels of this package.  Training works, with HIP backwards throughout: the softmax
+branch (natsl_softmax_sparse_bwd), the linear branch (natsl_linear_chunk_bwd), the short convolutions
+(natsl_short_conv_bwd), the row norms (natsl_row_norm_bwd) and the norm-gate (natsl_norm_gate_bwd); only the block pooling's
+backward (a broadcast of the block's gradient) and the projections are torch operations.  With a NAtSCache
 the layer prefills once in chunk mode on the empty cache and then decodes in steps of fewer than 64 tokens;
 64 or more new tokens on a cache that already holds tokens run through that decode path in steps (there is no chunked
 kernel that starts from cached keys; the reference's attention operator cannot run this case at all: it sizes its

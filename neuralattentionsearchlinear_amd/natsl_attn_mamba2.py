@@ -1,7 +1,8 @@
 """Mamba2-SSD / softmax hybrid token mixer with the forward signature, returns and parameter names of
 the reference layer (src/nats/layers/natsl_attn_mamba2.py:100-599).  Same scope as the Gated-DeltaNet
-layer: trainable (the linear branch, the pooling and the norm-gate differentiate through torch operations, the
-softmax branch through its HIP backward); with a cache, one chunked prefill on the empty cache and then decode steps of
+layer: trainable with the same HIP backwards (natsl_softmax_sparse_bwd, natsl_linear_chunk_bwd in its Mamba form,
+natsl_short_conv_bwd, natsl_row_norm_bwd, natsl_norm_gate_bwd; the pooling's backward and the projections are torch
+operations); with a cache, one chunked prefill on the empty cache and then decode steps of
 fewer than 64 tokens (longer inputs on a filled cache are fed through the decode path in such steps)."""
 from __future__ import annotations
 

@@ -90,3 +90,34 @@ def test_backward_entry_rejects_what_is_not_built():
         a = list(args(128, 64, 64))
         a[0], a[12] = delta_rule, None
         assert L.natsl_linear_chunk_bwd(*a) == -1 and b"null pointer" in L.natsl_last_error()
+
+
+def test_invalid_block_gradient_is_refused_for_blocks_of_several_chunks():
+    """The linear branch's selector gradient for blocks NOT typed linear is built for one chunk per block only: a
+    larger block with the flag set raises before anything is launched."""
+    import torch
+    from neuralattentionsearchlinear_amd._linear_bwd import linear_chunk_backward
+    q = torch.zeros(1, 128, 2, 64, dtype=torch.bfloat16)
+    ty = torch.zeros(1, 1, 2, 2, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="nats_block_size == 64"):
+        linear_chunk_backward('gdn', q, q, q, torch.zeros(1, 128, 2), torch.zeros(1, 128, 2, dtype=torch.bfloat16), None, ty, 1.0, 128,
+                              True, True, True, q, None, True)
+
+
+def test_chunk_state_saving_follows_the_byte_budget():
+    """_mixed_common.SAVE_CHUNK_STATES = None keeps the linear branch's chunk states for the backward only while they fit
+    SAVE_CHUNK_STATES_MAX_BYTES; True / False force it."""
+    import torch
+    import neuralattentionsearchlinear_amd._mixed_common as MC
+    small = torch.empty(1, 512, 4, 128, device='meta')
+    big = torch.empty(8, 8192, 16, 128, device='meta')
+    old = MC.SAVE_CHUNK_STATES
+    try:
+        MC.SAVE_CHUNK_STATES = None
+        assert MC._keep_chunk_states(small, small, None) and not MC._keep_chunk_states(big, big, None)
+        MC.SAVE_CHUNK_STATES = True
+        assert MC._keep_chunk_states(big, big, None)
+        MC.SAVE_CHUNK_STATES = False
+        assert not MC._keep_chunk_states(small, small, None)
+    finally:
+        MC.SAVE_CHUNK_STATES = old

@@ -244,7 +244,7 @@ def test_short_convolution(W, D, act, bias, dtype):
         outs.append(y3)
         close(torch.cat(outs, 1), ref)
         assert torch.equal(st.cpu(), x[:, -W:].transpose(1, 2))
-    # gradients (HIP forward, torch-evaluated backward) against autograd through the fp32 formula
+    # gradients (HIP forward, HIP backward: natsl_short_conv_bwd) against autograd through the fp32 formula
     xd = x.to(DEV).requires_grad_(True)
     yg, _ = conv(xd)
     dy = torch.randn(B, T, D, generator=g)

@@ -19,9 +19,9 @@ DEV = 'cuda:0'
 CASES = [
     # kind, B, T, H, HN, K, V, block, decay, intra, h0, dht, invalid
     ('gdn', 2, 512, 4, 2, 128, 128, 64, True, True, True, True, False),
-    ('gdn', 1, 300, 4, 2, 64, 64, 128, True, True, False, True, True),      # ragged last chunk, incomplete last block
-    ('gdn', 1, 640, 2, 1, 192, 384, 256, True, True, True, False, True),    # the 760M geometry
-    ('gdn', 1, 512, 6, 6, 128, 256, 64, False, True, True, True, False),    # the 340M geometry, no decay on rolled-back blocks
+    ('gdn', 1, 300, 4, 2, 64, 64, 128, True, True, False, True, False),     # ragged last chunk, incomplete last block
+    ('gdn', 1, 640, 2, 1, 192, 384, 256, True, True, True, False, False),   # the 760M geometry
+    ('gdn', 1, 512, 6, 6, 128, 256, 64, False, True, True, True, True),     # the 340M geometry, no decay on rolled-back blocks
     ('gdn', 1, 256, 2, 2, 128, 64, 64, True, False, True, True, True),      # no intra-chunk term
     ('mamba', 2, 512, 4, 2, 128, 64, 64, True, True, True, True, True),
     ('mamba', 1, 330, 4, 4, 64, 128, 128, False, True, False, True, False),

@@ -25,7 +25,7 @@ def _close(a, b, what, rl_tol=5e-3):
 
 @pytest.mark.parametrize("kind,K,V,block,h0,invalid", [('gdn', 128, 128, 64, False, False), ('gdn', 64, 64, 64, True, True),
                                                         ('gdn', 128, 64, 128, True, False), ('mamba', 128, 64, 64, True, False),
-                                                        ('mamba', 64, 64, 256, False, True)])
+                                                        ('mamba', 64, 64, 256, False, False), ('mamba', 64, 128, 64, False, True)])
 def test_mixed_operator_backward(kind, K, V, block, h0, invalid):
     from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn
     from neuralattentionsearchlinear_amd.mixed_attn_mamba import nats_mixed_attn_mamba
