@@ -51,7 +51,7 @@ def _keep_chunk_states(q, v, cu_seqlens) -> bool:
         return bool(SAVE_CHUNK_STATES)
     B, T, H, K = q.shape
     V = v.shape[-1]
-    n_seq = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    n_seq = B if cu_seqlens is None else len(cu_seqlens) - 1                     # (a host list here)
     chunks = -(-B * T // CHUNK_SIZE) + n_seq                       # upper bound on the chunks of all sequences
     return chunks * H * (2 * K * V + 2 * CHUNK_SIZE * V + _PREP_WORKSPACE_BYTES) <= SAVE_CHUNK_STATES_MAX_BYTES
 

@@ -1,4 +1,6 @@
 """Shared helpers for the GPU parity tests."""
+import os
+
 import torch
 import torch.nn.functional as F
 
@@ -20,6 +22,15 @@ def assert_close(a, b, what=""):
     ma, rl = max_abs(a, b), rel_l2(a, b)
     assert ma <= MAX_ABS_TOL and rl <= REL_L2_TOL, f"{what}: max-abs {ma:.3e} (tol {MAX_ABS_TOL}), rel-L2 {rl:.3e} (tol {REL_L2_TOL})"
     return ma, rl
+
+
+def record_parity(what, **errors):
+    """Appends one line of measured errors to the text file the environment variable NATSL_PARITY_LOG names (no file when it
+    is unset): the full-size tests call this, so that a run leaves the measured figures behind and not only pass / fail."""
+    path = os.environ.get("NATSL_PARITY_LOG")
+    if path:
+        with open(path, "a") as f:
+            f.write(f"{what}: " + "  ".join(f"{k} {v:.3e}" for k, v in errors.items()) + "\n")
 
 
 def make_types(B, NB, HN, p_attn, seed, dtype=torch.float32, force_last=True):

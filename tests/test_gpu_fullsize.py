@@ -15,10 +15,18 @@ import torch
 import torch.nn.functional as F
 
 from oracle import softmax_branch as SB
-from tests._util import assert_close, make_types
+from tests import _util
+from tests._util import make_types, record_parity
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
+
+
+def assert_close(a, b, what=""):
+    """tests._util.assert_close (max-abs 2e-2, rel-L2 5e-3), with the measured errors recorded."""
+    ma, rl = _util.assert_close(a, b, what)
+    record_parity(what, max_abs=ma, rel_l2=rl)
+    return ma, rl
 
 
 def _randn(shape, seed, dtype=torch.bfloat16):
@@ -87,7 +95,7 @@ def test_c2_softmax_slices_against_dense_fp32(c2, same_block):
         seen = mask.any(-1)
         p = torch.softmax(s, -1).nan_to_num(0.0)          # rows that see no key give 0
         ref = p @ vf
-        assert_close(o[b, :, h].float(), ref, f"o_attn[{b},:,{h}]")
+        assert_close(o[b, :, h].float(), ref, f"c2 o_attn[{b},:,{h}] (own block {'visible' if same_block else 'hidden'}) against the dense fp32 masked softmax")
         lse_ref = torch.where(seen, torch.logsumexp(s, -1) * 1.4426950408889634, torch.zeros_like(seen, dtype=torch.float32))
         assert float((lse[b, :, h] - lse_ref).abs().max()) <= 2e-2, "lse (log2 units)"
 
@@ -120,6 +128,7 @@ def test_c2_softmax_backward_slices_against_dense_fp32(c2):
             rl = float((g_ - r_).norm() / r_.norm())
             ma, top = float((g_ - r_).abs().max()), float(r_.abs().max())
             assert rl <= 5e-3 and ma <= 2e-2 * max(top, 1.0), f"{name}[{b},:,{h}]: rel-L2 {rl:.3e}, max-abs {ma:.3e} of {top:.3e}"
+            record_parity(f"c2 softmax backward {name}[{b},:,{h}] against dense fp32 autograd", max_abs=ma, rel_l2=rl, largest_reference=top)
         # selector gradient of block j: sum of dS over (queries of later blocks) x (keys of block j), for blocks typed attention
         with torch.no_grad():
             dp = do[b, :, h].float() @ vf.detach().T
@@ -178,8 +187,8 @@ def test_c1_all_linear_matches_token_recurrence_on_a_slice():
         sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()
         lin = torch.ones(1, T // block, 1)
         o_ref, s_ref = LB.gdn_token_recurrence(sl(q), sl(k), sl(v), sl(g), sl(beta), lin, scale, None, block=block)
-        assert_close(o[b:b + 1, :, h:h + 1].float(), o_ref, f"o_gdn[{b},:,{h}]")
-        assert_close(s[b:b + 1, h:h + 1], s_ref, f"final_state[{b},{h}]")
+        assert_close(o[b:b + 1, :, h:h + 1].float(), o_ref, f"c1 o_gdn[{b},:,{h}] against the fp64 token recurrence")
+        assert_close(s[b:b + 1, h:h + 1], s_ref, f"c1 final_state[{b},{h}] against the fp64 token recurrence")
 
 
 # --------------------------------------------------------------------------------------------
@@ -236,7 +245,7 @@ def test_c4_mamba_homogeneity_and_hand_off():
     mask = SB.visibility_mask(ty[1, :, 4, 0].float().cpu(), T, block, True).to(DEV)
     sc = (q[1, :, 4].float() @ k[1, :, 4].float().T) * K ** -0.5
     ref = torch.softmax(sc.masked_fill(~mask, float('-inf')), -1) @ v[1, :, 4].float()
-    assert_close(oa1[1, :, 4].float(), ref, "o_attn slice")
+    assert_close(oa1[1, :, 4].float(), ref, "c4 shape, N(0,1) inputs: o_attn[1,:,4] against the dense fp32 masked softmax")
 
 
 # --------------------------------------------------------------------------------------------
@@ -354,3 +363,81 @@ def test_c2_gdn_backward_full_depth(c2):
         e_n = _rel(got[6][b:b + 1, :, h:h + 1], o['dnats'])
         assert e_n <= 1e-2, f"dnats[{b},:,{h}] against the fp64 oracle: rel-L2 {e_n:.3e}"
         print(f"\nc2 backward slice ({b},{h}): " + "  ".join(f"{n} {e:.2e}" for n, e in errs.items()) + f"  dnats {e_n:.2e}", flush=True)
+        record_parity(f"c2 GDN backward slice ({b},{h}) against the fp64 oracle, rel-L2", **errs, dnats=e_n)
+
+
+def _c4_draw(seed=1700):
+    """c4's own distributions: dt = softplus(N(0,1) - 4); A = -exp(U(0, log 16)) per head; B, C ~ N(0,1) in ONE group shared by
+    all heads (k = B, q = C, state dim 128); X ~ N(0,1), head dim 64; the operator takes v = X dt and g = A dt
+    (src/nats/layers/natsl_attn_mamba2.py:472-474); selector blocks of 256 tokens, 25 % typed attention."""
+    B, T, H, K, V, block = 4, 8192, 32, 128, 64, 256
+    dt = F.softplus(_randn((B, T, H), seed, torch.float32) - 4.0)
+    gen = torch.Generator(device=DEV).manual_seed(seed + 1)
+    A = -torch.exp(torch.rand(H, device=DEV, generator=gen) * torch.log(torch.tensor(16.0)))
+    q = _randn((B, T, 1, K), seed + 2).expand(B, T, H, K).contiguous()
+    k = _randn((B, T, 1, K), seed + 3).expand(B, T, H, K).contiguous()
+    x = _randn((B, T, H, V), seed + 4)
+    v = (x.float() * dt.unsqueeze(-1)).to(torch.bfloat16)
+    g = A.view(1, 1, H) * dt
+    ty = make_types(B, T // block, H, 0.25, 17, torch.bfloat16).to(DEV)
+    return dict(q=q, k=k, v=v, g=g, ty=ty, x=x, B=B, T=T, H=H, K=K, V=V, block=block)
+
+
+def test_c4_mamba_config_draw_slices_against_token_recurrence():
+    """c4 as its configuration draws it (un-normalised B and C shared across heads, small dt, strong per-head decay): two
+    (sequence, head) slices of the Mamba branch's output and the final SSM state against the fp64 token recurrence, and
+    one slice of the softmax branch (K = 128, V = 64, block 256) against the dense fp32 masked softmax."""
+    from oracle import linear_branch as LB
+    d = _c4_draw()
+    T, K, block = d['T'], d['K'], d['block']
+    o, s = _linear('mamba', d['q'], d['k'], d['v'], d['g'], None, None, d['ty'], block, 1.0)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(s).all()
+    for b, h in ((0, 0), (3, 26)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()
+        lin = d['ty'][b:b + 1, :, h:h + 1, 1].float().cpu()
+        o_ref, s_ref = LB.mamba_token_recurrence(sl(d['q']), sl(d['k']), sl(d['v']), sl(d['g']), lin, 1.0, None, block=block)
+        # the outputs here reach far beyond 1 (|B.C| ~ 11 per key, tens of keys in the decay window): the absolute bound scales
+        top = float(o_ref.abs().max())
+        ma, rl = _util.max_abs(o[b:b + 1, :, h:h + 1].float(), o_ref), _util.rel_l2(o[b:b + 1, :, h:h + 1].float(), o_ref)
+        record_parity(f"c4 o_mamba[{b},:,{h}] against the fp64 token recurrence", max_abs=ma, rel_l2=rl, largest_reference=top)
+        assert rl <= _util.REL_L2_TOL and ma <= _util.MAX_ABS_TOL * max(top, 1.0), f"o_mamba[{b},:,{h}]: rel-L2 {rl:.3e}, max-abs {ma:.3e} of {top:.3e}"
+        top = float(s_ref.abs().max())
+        ma, rl = _util.max_abs(s[b:b + 1, h:h + 1], s_ref), _util.rel_l2(s[b:b + 1, h:h + 1], s_ref)
+        record_parity(f"c4 final SSM state[{b},{h}] against the fp64 token recurrence", max_abs=ma, rel_l2=rl, largest_reference=top)
+        assert rl <= _util.REL_L2_TOL and ma <= _util.MAX_ABS_TOL * max(top, 1.0), f"final state[{b},{h}]: rel-L2 {rl:.3e}, max-abs {ma:.3e} of {top:.3e}"
+    # the attention view reads the un-scaled X (src/nats/layers/natsl_attn_mamba2.py:391-393, :442)
+    oa, _ = _softmax(d['q'], d['k'], d['x'], d['ty'], block, K ** -0.5)
+    b, h = 2, 9
+    mask = SB.visibility_mask(d['ty'][b, :, h, 0].float().cpu(), T, block, True).to(DEV)
+    sc = (d['q'][b, :, h].float() @ d['k'][b, :, h].float().T) * K ** -0.5
+    ref = torch.softmax(sc.masked_fill(~mask, float('-inf')), -1) @ d['x'][b, :, h].float()
+    assert_close(oa[b, :, h].float(), ref, f"c4 o_attn[{b},:,{h}] against the dense fp32 masked softmax")
+
+
+def test_c4_mamba_backward_slices():
+    """The linear branch's backward in its Mamba form at c4 (32 blocks of 4 chunks, the configuration's draw): two
+    (sequence, head) slices of dq, dk, dv, dg and the selector's gradient against autograd through the fp64 chunked oracle
+    on that slice alone, and exact linearity in dO.  Tolerances as in tests/test_gpu_linear_bwd.py."""
+    from oracle import linear_branch as LB
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    d = _c4_draw()
+    do = _randn((d['B'], d['T'], d['H'], d['V']), 1800)
+    args = ('mamba', d['q'], d['k'], d['v'], d['g'], None, None, d['ty'], 1.0, d['block'], True, False, True)
+    with torch.no_grad():
+        got = B_.linear_chunk_backward_hip(*args, do, None, False)
+        got2 = B_.linear_chunk_backward_hip(*args, do * 2, None, False)
+    names = ['dq', 'dk', 'dv', 'dg']
+    for j, name in enumerate(names):
+        assert torch.isfinite(got[j].float()).all(), name
+        _assert_doubles(got2[j], got[j], f"{name}(2 dO) vs 2 {name}(dO)", 20_000)
+    for b, h in ((0, 0), (3, 26)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].cpu()
+        o = LB.linear_branch_bwd('mamba', sl(d['q']), sl(d['k']), sl(d['v']), sl(d['g']), None, d['ty'][b:b + 1, :, h:h + 1, 1].cpu(),
+                                 1.0, sl(do), None, None, d['block'], True, False, True, False)
+        errs = {}
+        for j, name in enumerate(names):
+            errs[name] = _rel(got[j][b:b + 1, :, h:h + 1], o[name])
+            assert errs[name] <= (1e-2 if name == 'dg' else 5e-3), f"{name}[{b},:,{h}] against the fp64 oracle: rel-L2 {errs[name]:.3e}"
+        e_n = _rel(got[6][b:b + 1, :, h:h + 1], o['dnats'])
+        assert e_n <= 1e-2, f"dnats[{b},:,{h}] against the fp64 oracle: rel-L2 {e_n:.3e}"
+        record_parity(f"c4 Mamba backward slice ({b},{h}) against the fp64 oracle, rel-L2", **errs, dnats=e_n)
