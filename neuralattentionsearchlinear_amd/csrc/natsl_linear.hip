@@ -80,21 +80,26 @@ NATSL_DEVICE bool lin_type(const void* types, int dtype, size_t i) {
 // =============================================================================================
 // prep
 // =============================================================================================
-template <int DK, bool DELTA>
+// PF ("P formed by the scan"): the kernel reads k only -- no q tile, no q k^T product, no P -- and leaves TmB and six scale
+// vectors; the two extra ones (in the first 512 bytes of the unit's P area) are the exponents the scan needs to form
+// P_ij = rq_i (q_i . k_j) exp2(gq_i - gk_j):   gk = gamma log2(e) - log2 rk,   gq = gamma log2(e) + log2 scale,
+// and sq comes without its 1/|q| factor (the scan takes the row norms of q from the tile it holds anyway).
+template <int DK, bool DELTA, bool PF>
 __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams p) {
+  static_assert(DELTA || !PF, "the Mamba form has its own prep");
   constexpr int KP = DK + 8;   // bf16 row pitch
   constexpr int KL = DK / 32;  // 16-byte loads per thread per tile
   // The 64x64 fp32 matrices of the solve are kept as their ten lower 16x16 blocks, block (i, k) at
   // index i(i+1)/2 + k, rows of BP floats.  A = strictly lower system matrix; X = (I+A)^-1 row-major;
   // Xt = the four DIAGONAL blocks of X transposed (so that such a block serves as an MFMA B operand with one 16-byte read).
   constexpr int BP = 20, BLK = 16 * BP, NBLK = 10;
-  constexpr int TILE_BYTES = 2 * C * KP * 2, SOLVE_BYTES = (2 * NBLK + 4) * BLK * 4;
+  constexpr int TILE_BYTES = (PF ? 1 : 2) * C * KP * 2, SOLVE_BYTES = (2 * NBLK + 4) * BLK * 4;
   // LDS: the q, k tiles are dead once the Gram products are done; the solve reuses their space
   constexpr int REGION0 = (DELTA && SOLVE_BYTES > TILE_BYTES) ? SOLVE_BYTES : TILE_BYTES;
   __shared__ __align__(16) unsigned char region0[REGION0];
   __shared__ __align__(16) float gam[C], rq[C], rk[C], bet[C];
   bf16_t* Qs = reinterpret_cast<bf16_t*>(region0);
-  bf16_t* Ks = Qs + C * KP;
+  bf16_t* Ks = PF ? Qs : Qs + C * KP;   // (no q tile with PF)
   float* Ab = reinterpret_cast<float*>(region0);
   float* Xb = Ab + NBLK * BLK;
   float* Xt = Xb + NBLK * BLK;
@@ -133,13 +138,13 @@ __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams 
     u32x4 qa[KL], kb[KL];
 #pragma unroll
     for (int i = 0; i < KL; ++i) {
-      qa[i] = ok ? qr[seg + 4 * i] : z;
+      qa[i] = (ok && !PF) ? qr[seg + 4 * i] : z;
       kb[i] = ok ? kr[seg + 4 * i] : z;
     }
 #pragma unroll
     for (int i = 0; i < KL; ++i) {
       const u32x4 a = qa[i], b = kb[i];
-      *reinterpret_cast<u32x4*>(Qs + row * KP + (seg + 4 * i) * 8) = a;
+      if (!PF) *reinterpret_cast<u32x4*>(Qs + row * KP + (seg + 4 * i) * 8) = a;
       *reinterpret_cast<u32x4*>(Ks + row * KP + (seg + 4 * i) * 8) = b;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams 
     sq += __shfl_xor(sq, 1); sq += __shfl_xor(sq, 2);
     sk += __shfl_xor(sk, 1); sk += __shfl_xor(sk, 2);
     if (seg == 0) {
-      rq[row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
+      rq[row] = (l2 && !PF) ? rsqrtf(sq + 1e-6f) : 1.f;
       rk[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
     }
   }
@@ -194,14 +199,16 @@ __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams 
 #pragma unroll
       for (int s = 0; s < DK / 16; ++s) {
         const bf16x8 kb = ld8(Ks + (32 * tj + l32) * KP + 16 * s + 8 * hf);
-        const bf16x8 qa = ld8(Qs + (32 * ti + l32) * KP + 16 * s + 8 * hf);
-        gq = mfma32(kb, qa, gq);  // transposed: lane = query row i, registers = key tokens j
+        if (!PF) {
+          const bf16x8 qa = ld8(Qs + (32 * ti + l32) * KP + 16 * s + 8 * hf);
+          gq = mfma32(kb, qa, gq);  // transposed: lane = query row i, registers = key tokens j
+        }
         if (DELTA) {
           const bf16x8 ka = ld8(Ks + (32 * ti + l32) * KP + 16 * s + 8 * hf);
           gk = mfma32(ka, kb, gk);  // lane = column j, registers = rows i
         }
       }
-      {
+      if (!PF) {
         // this lane's 16 key tokens are four runs of four: 16-byte reads of their gamma and 1/|k|
         const float gi = gam[i], fi = p.scale * rq[i];
         // this lane holds tokens 8 q4 + 4 hf + e of the tile: q4 = 0, 2 are the two halves of group hf's slots,
@@ -250,6 +257,11 @@ __global__ __launch_bounds__(256, 4) void linear_prep_kernel(const LinearParams 
     Sout[lane] = eg * rk[lane];
     Sout[C + lane] = p.scale * rq[lane] * eg;
     Sout[2 * C + lane] = rk[lane] * __expf(dk);
+    if (PF) {
+      float* Eout = reinterpret_cast<float*>(Pout);
+      Eout[lane] = gt * 1.4426950408889634f - __builtin_amdgcn_logf(rk[lane]);
+      Eout[C + lane] = gt * 1.4426950408889634f + __builtin_amdgcn_logf(p.scale);
+    }
     if (lane == 0) Sout[3 * C] = __expf(gl);
     if (lane == 1) Sout[3 * C + 1] = gl;
     if (lane == 2) {
@@ -427,20 +439,24 @@ NATSL_DEVICE s16x4 lds_tr4_at(const unsigned addr) {
 }
 
 // LDS layout of the scan kernel: two or three stages and two output tiles.
-template <int DK, int NW>
+template <int DK, int NW, bool PF = false>
 struct ScanLds {
   static constexpr int BVW = 16 * NW;                 // state columns of the workgroup
   static constexpr int KROW = DK * 2;                 // bytes per k / q row
   static constexpr int VROW = BVW * 2;                // bytes per v row
-  static constexpr int KB = 64 * KROW, VB = 64 * VROW, TB = 6 * 1024, PB = 6 * 1024, SCB = 1024;
+  // (with PF, P is formed and used within one step: one area for all stages, behind them; and two more scale vectors arrive)
+  static constexpr int KB = 64 * KROW, VB = 64 * VROW, TB = 6 * 1024, PB = PF ? 0 : 6 * 1024, SCB = PF ? 2048 : 1024;
+  static constexpr int PSHARED = PF ? 6 * 1024 : 0;
   static constexpr int OFF_K = 0, OFF_Q = OFF_K + KB, OFF_V = OFF_Q + KB, OFF_T = OFF_V + VB, OFF_P = OFF_T + TB, OFF_SC = OFF_P + PB;
   static constexpr int STAGE = OFF_SC + SCB;
   static constexpr int OROW = VROW + 16;              // output tile row pitch (bytes)
   static constexpr int OB = 64 * OROW;
   // Stages: chunk c lives in stage c % NSTAGE.  Three when they fit (narrow workgroups): the requests of chunk c + 2
   // are issued in step c and have a whole step more to land; two otherwise (requests of chunk c + 1 in step c).
-  static constexpr int NSTAGE = 3 * STAGE + 2 * OB <= 160 * 1024 ? 3 : 2;
-  static constexpr int TOTAL = NSTAGE * STAGE + 2 * OB;
+  static constexpr int NSTAGE = 3 * STAGE + PSHARED + 2 * OB <= 160 * 1024 ? 3 : 2;
+  static constexpr int OFF_PS = NSTAGE * STAGE;          // the shared P area (PF)
+  static constexpr int OFF_OUT = OFF_PS + PSHARED;       // the two output tiles
+  static constexpr int TOTAL = OFF_OUT + 2 * OB;
 };
 
 // index of A operand (t, s) of TmB / P among the six that are stored (the two above the diagonal are skipped)
@@ -455,9 +471,14 @@ NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t
   __launch_bounds__(64 * (NW + 2)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
 
 // NW compute waves (16 state columns each) + two data-movement waves.
-template <int DK, bool DELTA, int NW>
+// PF (delta rule, four compute waves): P does not come from the workspace; the two data-movement waves form it from the
+// stage's k and q tiles while the compute waves work on the state (three of the six A operands each, written to the stage's
+// P area), take the q rows' reciprocal norms from the operands they read for that and complete sq; a second barrier in the
+// middle of the step hands both over.
+template <int DK, bool DELTA, int NW, bool PF>
 __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p) {
-  using L = ScanLds<DK, NW>;
+  static_assert(!PF || (DELTA && NW == 4), "P is formed in the scan only by the four-wave delta-rule shape");
+  using L = ScanLds<DK, NW, PF>;
   constexpr int KS = DK / 32;   // matrix k-steps over the key dimension
   constexpr int KT = DK / 16;   // 16-row state tiles
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -496,6 +517,12 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     // store the output tile of chunk c - 1 (wave NW + 1), wait for the requests, meet the barrier.  The compute waves
     // never touch global memory inside the loop.  (One wave issues about 1 KiB per 36 cycles; two share the 53 KiB.)
     const bool first = wave == NW;
+    // (operand addresses of the k / q tiles and of a row of the scale vectors, as the compute waves use them below)
+    unsigned a_kq[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) a_kq[s] = (unsigned)(i16 * L::KROW) + 16u * (unsigned)((4 * s + g4) ^ kq_swizzle<DK>(i16));
+    const unsigned a_sc = 16u * g4;
+    const bool l2n = (p.flags & NATSL_QK_L2NORM) != 0;
     const size_t qk_pitch = (size_t)p.H * DK * 2, v_pitch = (size_t)p.H * p.V * 2;   // bytes per token
     const char* kb = reinterpret_cast<const char*>(p.k + ((size_t)bos * p.H + h) * DK);
     const ptrdiff_t q_minus_k = reinterpret_cast<const char*>(p.q) - reinterpret_cast<const char*>(p.k);
@@ -544,6 +571,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       if (first) {
         // in the order the compute waves need them: sc, k (R = k S comes first), q
         dma16(sb, 16u * lane, st + L::OFF_SC);
+        if (PF) dma16(pb, 16u * lane, st + L::OFF_SC + 1024);   // the two exponent vectors (and 512 bytes nobody reads)
 #pragma unroll
         for (int u = 0; u < KQ_PIECES; ++u) dma16(kb, kq_off[u], st + L::OFF_K + 1024 * u);
 #pragma unroll
@@ -555,7 +583,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
 #pragma unroll
           for (int v = 0; v < 6; ++v) dma16(tb, ws_off[v], st + L::OFF_T + 1024 * v);
         }
-        if (DELTA) {
+        if (DELTA && !PF) {
 #pragma unroll
           for (int v = 0; v < 6; ++v) dma16(pb, ws_off[v], st + L::OFF_P + 1024 * v);
         }
@@ -582,7 +610,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       o_glb[j] = (unsigned)((size_t)o_tok[j] * v_pitch) + 2u * (unsigned)(cbase + (WIDE ? 8 : 4) * (i16 >> 2));
     }
     auto store_out = [&](const int cc) __attribute__((always_inline)) {
-      const unsigned ob = lds0 + L::NSTAGE * L::STAGE + (cc & 1) * L::OB;
+      const unsigned ob = lds0 + L::OFF_OUT + (cc & 1) * L::OB;
       const int nvalid = len - cc * C;
 #pragma unroll
       for (int j = 0; j < O_PASSES; ++j) {
@@ -601,7 +629,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     // stores issued after them) may still be in flight at the barrier: vector memory operations complete in the order
     // they were issued, so allowing as many outstanding as one step issues leaves exactly the older step's complete.
     constexpr int AHEAD = L::NSTAGE - 1;
-    constexpr int PER_STEP_FIRST = 1 + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? 12 : 0) + O_PASSES;
+    constexpr int PER_STEP_FIRST = 1 + (PF ? 1 : 0) + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? (PF ? 6 : 12) : 0) + O_PASSES;
     static_assert(PER_STEP_FIRST <= 63 && PER_STEP_SECOND <= 63, "the wait counter has six bits");
     constexpr int VM_FIRST = (PER_STEP_FIRST & 15) | ((PER_STEP_FIRST >> 4) << 14) | 0x0f70;
     constexpr int VM_SECOND = (PER_STEP_SECOND & 15) | ((PER_STEP_SECOND >> 4) << 14) | 0x0f70;
@@ -610,18 +638,118 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       if (a < NT) request(a);
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
-    for (int c = 0; c < NT; ++c) {
-      // into the stage that step c - 1 read: every wave is past the barrier that ended it
-      const bool more = c + AHEAD < NT;
-      if (more) request(c + AHEAD);
-      if (c > 0 && !first) store_out(c - 1);
-      if (AHEAD == 2 && more) {
-        if (first) __builtin_amdgcn_s_waitcnt(VM_FIRST);
-        else __builtin_amdgcn_s_waitcnt(VM_SECOND);
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0f70);
+    if constexpr (PF) {
+      // P = scale tril(rq_i rk_j (q_i . k_j) e^{gamma_i - gamma_j}) of chunk c is formed HERE, from the tiles of chunk c's stage,
+      // while the compute waves work on the state.  Z^T = k_tile(t2) q_tile(t)^T leaves lane (i16, g4) with query 16 t + i16
+      // against keys 16 t2 + 4 g4 .. + 3: the four slots this lane holds of A operand (t, t2 / 2), half t2 % 2.  Each of the two
+      // waves forms the operands of two row tiles (five of the ten tiles) and completes sq = scale e^{gamma} / |q| for their
+      // rows; |q_i|^2 is the diagonal of q_tile q_tile^T (a lane's 16 bytes are the same slots of its row as A and as B
+      // operand), found in lane group i16 / 4, register i16 % 4.
+      // Both rows of a wave go through ONE straight piece of code: every operand read first (the k tiles are shared by the two
+      // rows), then the matrix instructions of all chains interleaved, then the exponentials, then the stores.  The row norm
+      // multiplies at the end, so the exponentials do not wait for it.
+      auto form_two_rows = [&](const int ta, const int tb_, const unsigned st) __attribute__((always_inline)) {
+        const int tmax = ta > tb_ ? ta : tb_;
+        const int tr[2] = {ta, tb_};
+        bf16x8 qb[2][KS], ka[4][KS];
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+#pragma unroll
+          for (int s = 0; s < KS; ++s) qb[w][s] = *reinterpret_cast<lds_b128_t>(st + L::OFF_Q + a_kq[s] + tr[w] * 16 * L::KROW);
+#pragma unroll
+        for (int t2 = 0; t2 < 4; ++t2)
+#pragma unroll
+          for (int s = 0; s < KS; ++s)
+            if (t2 <= tmax) ka[t2][s] = *reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + t2 * 16 * L::KROW);
+        f32x4 gj[4];
+#pragma unroll
+        for (int t2 = 0; t2 < 4; ++t2)
+          if (t2 <= tmax) gj[t2] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * (4 * C) + a_sc + 64 * t2);
+        float gq[2], sq0[2];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          gq[w] = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (5 * C + 16 * tr[w] + i16));
+          sq0[w] = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (C + 16 * tr[w] + i16));
+        }
+        f32x4 D[2], Z[2][4];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          D[w] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int t2 = 0; t2 < 4; ++t2) Z[w][t2] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            D[w] = mfma16(qb[w][s], qb[w][s], D[w]);
+#pragma unroll
+            for (int t2 = 0; t2 < 4; ++t2)
+              if (t2 <= tr[w]) Z[w][t2] = mfma16(ka[t2][s], qb[w][s], Z[w][t2]);
+          }
+        const int rsel = i16 & 3;
+        float rqi[2];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const float dsel = rsel == 0 ? D[w][0] : rsel == 1 ? D[w][1] : rsel == 2 ? D[w][2] : D[w][3];
+          const float ss = __shfl(dsel, 16 * (i16 >> 2) + i16);
+          rqi[w] = l2n ? rsqrtf(ss + 1e-6f) : 1.f;
+        }
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+#pragma unroll
+          for (int t2 = 0; t2 < 4; ++t2)
+            if (t2 <= tr[w]) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float e = Z[w][t2][r] * __builtin_amdgcn_exp2f(gq[w] - gj[t2][r]);
+                Z[w][t2][r] = (t2 < tr[w] || i16 >= 4 * g4 + r) ? e * rqi[w] : 0.f;
+              }
+            }
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+#pragma unroll
+          for (int sp = 0; sp < 2; ++sp)
+            if (2 * sp <= tr[w])
+              *reinterpret_cast<__attribute__((address_space(3))) bf16x8*>(lds0 + L::OFF_PS + 1024 * tri_slot(tr[w], sp) + 16 * lane) = pack8(Z[w][2 * sp], Z[w][2 * sp + 1]);
+          if (g4 == 0) {
+            typedef __attribute__((address_space(3))) float* lds_fw_t;
+            *reinterpret_cast<lds_fw_t>(st + L::OFF_SC + 4 * (C + 16 * tr[w] + i16)) = sq0[w] * rqi[w];
+          }
+        }
+      };
+      for (int c = 0; c < NT; ++c) {
+        // requests go into the stage that step c - 1 read: every wave is past the barrier that ended it
+        const bool more = c + AHEAD < NT;
+        const unsigned st = lds0 + (c % L::NSTAGE) * L::STAGE;
+        if (more) request(c + AHEAD);
+        if (c > 0 && !first) store_out(c - 1);
+        // five tiles each: rows 48..63 and 0..15 here, rows 32..47 and 16..31 there
+        if (first) form_two_rows(3, 0, st);
+        else form_two_rows(2, 1, st);
+        __syncthreads();   // hand-over of P and sq in the middle of the compute waves' step
+        if (AHEAD == 2 && more) {
+          if (first) __builtin_amdgcn_s_waitcnt(VM_FIRST);
+          else __builtin_amdgcn_s_waitcnt(VM_SECOND);
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+        }
+        __syncthreads();
       }
-      __syncthreads();
+    } else {
+      for (int c = 0; c < NT; ++c) {
+        // into the stage that step c - 1 read: every wave is past the barrier that ended it
+        const bool more = c + AHEAD < NT;
+        if (more) request(c + AHEAD);
+        if (c > 0 && !first) store_out(c - 1);
+        if (AHEAD == 2 && more) {
+          if (first) __builtin_amdgcn_s_waitcnt(VM_FIRST);
+          else __builtin_amdgcn_s_waitcnt(VM_SECOND);
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+        }
+        __syncthreads();
+      }
     }
     if (NT > 0 && !first) store_out(NT - 1);
     return;
@@ -811,8 +939,9 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         for (int r = 0; r < 4; ++r) S[m][r] = Ssave[m][r] * f;
     }
     // (4) o = sq * O1 + P v_new, into the (transposed) output tile: the four token tiles side by side
+    if constexpr (PF) __syncthreads();   // P and sq of this step are complete
     {
-      const unsigned ob = lds0 + L::NSTAGE * L::STAGE + (c & 1) * L::OB;
+      const unsigned ob = lds0 + L::OFF_OUT + (c & 1) * L::OB;
       f32x4 O[4];
       bf16x8 PA[6];
 #pragma unroll
@@ -820,7 +949,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       if (intra) {
         if constexpr (DELTA) {
 #pragma unroll
-          for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>(st + L::OFF_P + 1024 * v + 16 * lane);
+          for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>((PF ? lds0 + L::OFF_PS : st + L::OFF_P) + 1024 * v + 16 * lane);
         } else {
           // P = scale tril(q k^T e^{gamma_i - gamma_j}) formed here, from the tiles of this stage: Z^T = k_tile(t') q_tile(t)^T
           // leaves lane (i16, g4) with query 16 t + i16 against keys 16 t' + 4 g4 .. + 3 -- the four slots this lane holds of
@@ -915,10 +1044,10 @@ inline int cu_count_linear() {
   return n;
 }
 
-template <int DK, bool DELTA, int NW>
+template <int DK, bool DELTA, int NW, bool PF>
 static int launch_scan(const LinearParams& p, hipStream_t stream, const char* what) {
-  using L = ScanLds<DK, NW>;
-  auto kern = linear_scan_kernel<DK, DELTA, NW>;
+  using L = ScanLds<DK, NW, PF>;
+  auto kern = linear_scan_kernel<DK, DELTA, NW, PF>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
@@ -931,10 +1060,6 @@ template <int DK, bool DELTA>
 static int launch_linear(const LinearParams& p, hipStream_t stream, const char* what) {
   const long long units = (long long)p.total_chunks * p.H;
   if (units <= 0) return NATSL_OK;
-  if constexpr (DELTA) hipLaunchKernelGGL((linear_prep_kernel<DK, true>), dim3((unsigned)units), dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL(mamba_scale_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, p);
-  int rc = check_launch(what);
-  if (rc != NATSL_OK) return rc;
   // Waves per workgroup (16 state columns each).  A CU holds one workgroup (LDS), so a launch takes
   // ceil(workgroups / CUs) rounds of the chain's length, and a step of a wider workgroup takes longer (measured: 2 700, 3 000,
   // 4 400 cycles for one, two, four waves): the width with the least rounds x step time.  (Wider also means a chunk's inputs
@@ -948,9 +1073,33 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
   // (K = 192: five waves of that size do not fit the registers of a CU without spilling; three do)
   const bool ok4 = DK <= 128 && p.V % 64 == 0, ok2 = p.V % 32 == 0;
   const double c1 = cost(1, 1.0), c2 = ok2 ? cost(2, 1.1) : 1e30, c4 = ok4 ? cost(4, 1.65) : 1e30;
-  if (c4 <= c2 && c4 <= c1) return launch_scan<DK <= 128 ? DK : 128, DELTA, 4>(p, stream, what);
-  if (c2 <= c1) return launch_scan<DK, DELTA, 2>(p, stream, what);
-  return launch_scan<DK, DELTA, 1>(p, stream, what);
+  const int nw = (c4 <= c2 && c4 <= c1) ? 4 : (c2 <= c1 ? 2 : 1);
+  // The delta rule's four-wave scan forms P itself and the prep reads k only, when the launch fills the machine: prep and scan
+  // are then bound by their HBM traffic, which this cuts by a fifth (measured at B8 T8192 H16: 0.46 -> 0.43 ms), while a launch
+  // that leaves CUs idle is bound by the scan's step and only gets slower from the extra work in it (B8 T4096 H6 V256:
+  // 0.152 -> 0.176 ms; the narrower shapes likewise: 1.67 -> 1.90 ms at B1 T65536 H32 with one compute wave).  Not when the
+  // caller wants the chunk states for a backward: the backward kernels read P and the complete scale vectors from the workspace.
+  constexpr bool CAN_PF = DELTA && DK <= 128;
+  const bool pf = CAN_PF && nw == 4 && p.s_out == nullptr && n_chains * (p.V / 64) >= cus;
+  if constexpr (DELTA) {
+    if (pf) {
+      if constexpr (CAN_PF) hipLaunchKernelGGL((linear_prep_kernel<DK, true, true>), dim3((unsigned)units), dim3(256), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((linear_prep_kernel<DK, true, false>), dim3((unsigned)units), dim3(256), 0, stream, p);
+    }
+  } else {
+    hipLaunchKernelGGL(mamba_scale_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, p);
+  }
+  int rc = check_launch(what);
+  if (rc != NATSL_OK) return rc;
+  if (nw == 4) {
+    if constexpr (CAN_PF) {
+      if (pf) return launch_scan<DK, true, 4, true>(p, stream, what);
+    }
+    return launch_scan<DK <= 128 ? DK : 128, DELTA, 4, false>(p, stream, what);
+  }
+  if (nw == 2) return launch_scan<DK, DELTA, 2, false>(p, stream, what);
+  return launch_scan<DK, DELTA, 1, false>(p, stream, what);
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,

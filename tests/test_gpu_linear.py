@@ -134,3 +134,24 @@ def test_gdn_and_mamba_scan_with_64_columns_per_workgroup():
     _gdn(B, 320, H, 16, 128, V, 64, 0.3, True, seed=26, h0=True)
     _gdn(B, 256, H, 4, 64, V, 128, 0.5, False, seed=27)
     _mamba(B, 256, H, 8, 128, V, 64, 0.3, True, seed=28, h0=True)
+
+
+@pytest.mark.parametrize("K", [128, 64])
+def test_gdn_p_formed_by_the_scan_agrees_with_p_from_the_prep(K):
+    """A four-wave launch that fills the machine forms P inside the scan (the prep reads k only); a call that also returns the
+    chunk states for a backward takes P from the prep kernel through the workspace.  Same inputs: the states are bit-identical
+    (P does not enter them), the outputs agree to the rounding of P's bf16 tiles."""
+    from neuralattentionsearchlinear_amd import _capi
+    from neuralattentionsearchlinear_amd._mixed_common import linear_chunk_fwd
+    B, T, H, V, block = 8, 448, 16, 128, 64
+    assert B * H * (V // 64) >= _cus()
+    q, k, v = make_qkv(B, T, H, K, V, 40)
+    g, beta = make_gates(B, T, H, 41)
+    ty = make_types(B, T // block, H, 0.3, 42, torch.bfloat16)
+    flags = _capi.DECAY_NON_LINEAR | _capi.QK_L2NORM | _capi.INTRA_CHUNK
+    args = [t.to(DEV) for t in (q, k, v, g, beta)]
+    o1, s1 = linear_chunk_fwd('gdn', *args, None, ty.to(DEV), K ** -0.5, block, flags, True, None)
+    o2, s2 = linear_chunk_fwd('gdn', *args, None, ty.to(DEV), K ** -0.5, block, flags, True, None, chunk_states=True)[:2]
+    assert torch.equal(s1, s2)
+    rl = float((o1.float() - o2.float()).norm() / o2.float().norm())
+    assert 0 < rl <= 5e-4, rl          # (0 would mean both calls took the same path)
