@@ -6,7 +6,7 @@ natsl_linear_chunk_bwd (csrc/natsl_linear_bwd.hip: a reverse scan over the chunk
 few lines of host glue around them (block sums of g, the per-block sums of the gate gradients).  It replaces
 chunk_gated_delta_rule_nats_bwd (src/nats/ops/gated_delta_rule/chunk.py:170-332) and the Mamba counterpart
 (src/nats/ops/mamba/chunk.py:112-260) in function.  linear_chunk_backward_torch is the same method as fp32 torch operations
-on the GPU, for the shapes the kernels are not built for (V not a multiple of 64) and as its plain statement; both follow the
+on the GPU, for key widths the kernels are not built for and as the method's plain statement; both follow the
 chunked algorithm of the forward kernels (csrc/natsl_linear.hip), so the gradients belong to the forward that was actually
 computed, up to its bf16 rounding.
 
@@ -124,8 +124,8 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
     """Gradients of the chunked linear branch: -> (dq, dk, dv, dg fp32, dbeta or None, dh0 or None, dnats fp32 [B,NB,HN]).
     types [B,NB,HN,2]; do [B,T,H,V]; dht [N,H,K,V] or None; seqs: packed sequences (B = 1) or None; saved: what
     linear_chunk_fwd(..., chunk_states=True) returned after (o, final_state) on these same inputs, if the caller kept it.  The
-    HIP kernels (natsl_linear_chunk_bwd) where they are built (K in 64/128/192, V a multiple of 64), else the torch formulation
-    below, one sequence at a time.
+    HIP kernels (natsl_linear_chunk_bwd) for K in 64/128/192 -- V a multiple of 64 as it is, other multiples of 16 behind zero
+    columns --, else the torch formulation below, one sequence at a time.
 
     dnats_for_invalid_blocks with block > 64 raises NotImplementedError: for a block of several chunks that is not typed
     linear the reference sums a virtual key gradient v . dh over EVERY chunk of the block
@@ -136,9 +136,20 @@ def linear_chunk_backward(kind, q, k, v, g, beta, h0, types, scale, block, decay
         raise NotImplementedError(
             f"compute_dnats_for_invalid_blocks_linear_att=True is built for nats_block_size == {C} only (got {block}): "
             "pass compute_dnats_for_invalid_blocks_linear_att=False (the layers' default)")
-    if hip_backward_is_built(q.shape[-1], v.shape[-1]):
+    K, V = q.shape[-1], v.shape[-1]
+    if hip_backward_is_built(K, V):
         return linear_chunk_backward_hip(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
                                          dnats_for_invalid_blocks, seqs, saved)
+    if hip_backward_is_built(K, 64) and V % 16 == 0:
+        # Value widths the kernels are not built for (16..48, 96, ..): zero columns up to the next multiple of 64.  The state's
+        # columns never mix, a zero column of v and dO stays zero through the whole recurrence and adds nothing to any sum
+        # over V, so the gradients are exactly those of the narrower problem.
+        pad = -V % 64
+        padv = lambda t: None if t is None else torch.nn.functional.pad(t, (0, pad))
+        res = linear_chunk_backward_hip(kind, q, k, padv(v), g, beta, padv(h0), types, scale, block, decay, l2norm, intra, padv(do),
+                                        padv(dht), dnats_for_invalid_blocks, seqs, None)
+        return (res[0], res[1], res[2][..., :V].contiguous(), res[3], res[4], None if res[5] is None else res[5][..., :V].contiguous(),
+                res[6])
     if seqs is None:
         return linear_chunk_backward_torch(kind, q, k, v, g, beta, h0, types, scale, block, decay, l2norm, intra, do, dht,
                                            dnats_for_invalid_blocks)

@@ -145,3 +145,22 @@ def test_linear_branch_backward_random_shapes(seed):
                                        scale, block, decay, l2, intra, d(do), d(dht) if dht_on else None, invalid)
     torch.cuda.synchronize()
     _check(out, ref, kind, h0)
+
+
+@pytest.mark.parametrize("kind,K,V", [('gdn', 64, 32), ('gdn', 128, 96), ('mamba', 128, 48)])
+def test_value_widths_that_are_no_multiple_of_64(kind, K, V):
+    """V = 16..48, 96, ..: the dispatcher runs the kernels on v, dO and the states padded with zero columns to the next multiple
+    of 64 and cuts the gradients back; against the fp64 oracle on the narrow problem."""
+    from neuralattentionsearchlinear_amd import _linear_bwd as B_
+    B, T, H, HN, block = 2, 330, 4, 2, 64
+    q, k, v, g, beta, ty, init, do, dht = _inputs(kind, B, T, H, HN, K, V, block, 900 + V)
+    scale = K ** -0.5 if kind == 'gdn' else 1.0
+    l2 = kind == 'gdn'
+    ref = LB.linear_branch_bwd(kind, q, k, v, g, beta if kind == 'gdn' else None, ty[..., 1], scale, do, dht, init, block, True, l2, True, True)
+    d = lambda t: t.to(DEV)
+    assert not B_.hip_backward_is_built(K, V)
+    out = B_.linear_chunk_backward(kind, d(q), d(k), d(v), d(g), d(beta) if kind == 'gdn' else None, d(init), d(ty), scale, block, True,
+                                   l2, True, d(do), d(dht), True)
+    torch.cuda.synchronize()
+    assert out[2].shape[-1] == V and out[5].shape[-1] == V
+    _check(out, ref, kind, True)
