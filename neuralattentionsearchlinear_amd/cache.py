@@ -37,6 +37,8 @@ class NAtSLayerCache:
         self.nats_block_size = nats_block_size
         self.attn_offset, self.recurrent_offset, self.n_ops = attn_offset, recurrent_offset, n_ops
         self.op_for_incomplete_chunk = op_for_incomplete_chunk
+        # the modes in which the softmax operator does not run on the incomplete block (the Mamba layer's name for it included)
+        self._linear_only = op_for_incomplete_chunk in ('gated_delta_net', 'mamba')
         self.lazy_initialization(None)
         self.seen_tokens = seen_tokens
         self._n_tokens_in_nats_block = n_tokens_in_nats_block
@@ -93,18 +95,22 @@ class NAtSLayerCache:
         head: as many as that head has) followed by the tokens of the incomplete block, new ones included.
 
         n_data > 1 is supported while the new tokens stay inside the current block (the reference builds a mask
-        without the kept blocks there, :246-256, which does not fit the keys it is used with)."""
+        without the kept blocks there, :246-256, which does not fit the keys it is used with).  In the mode whose softmax
+        operator skips the incomplete block ('gated_delta_net' / 'mamba') the keys end at the last whole block and a new token
+        sees the kept blocks only, as in the chunked forward of that mode.  (The reference's one-token rule, :237-243, shows the
+        token that completes a block its own block, which its chunked forward never does; the chunked forward is followed.)"""
         bs, n_in, nmax = self.nats_block_size, self._n_tokens_in_nats_block, self.n_attn_blocks_max
         if n_data == 1:
             cols = self.n_attn_tokens_max + 1
-            if self.op_for_incomplete_chunk == 'gated_delta_net':
+            if self._linear_only:
                 cols = cols // bs * bs
             msk = self.valid_attn_tokens[:, :nmax + 1].repeat_interleave(bs, 1)[:, :cols]
+            if self._linear_only and cols > nmax * bs:
+                msk = msk.clone()
+                msk[:, nmax * bs:] = False          # the token that completes the block: its own block stays hidden
             return msk.transpose(1, 2).unsqueeze(-2).bool()
         if nats_block_types is None or nats_block_types.shape[1] != 1 or n_in + n_data > bs:
             raise NotImplementedError("a mask for several new tokens is built only while they stay inside the current block")
-        if self.op_for_incomplete_chunk == 'gated_delta_net':
-            raise NotImplementedError("several new tokens per step are not built for ops_for_incomplete_chunks='gated_delta_net'")
         if self.valid_attn_tokens is None:
             # an empty cache (a first input shorter than one block): no kept blocks yet, the keys are the new tokens
             dev, (B, _, HN, _) = nats_block_types.device, nats_block_types.shape
@@ -114,6 +120,12 @@ class NAtSLayerCache:
             B, _, HN = self.valid_attn_tokens.shape
             past = self.valid_attn_tokens[:, :nmax].repeat_interleave(bs, 1).transpose(1, 2)          # [B, HN, nmax*bs]
             past = past.unsqueeze(-2).expand(B, HN, n_data, nmax * bs)
+        if self._linear_only:
+            if self.valid_attn_tokens is None:
+                return torch.zeros(B, HN, n_data, n_data, dtype=torch.bool, device=dev)     # (the keys are the new tokens themselves)
+            if n_in + n_data < bs:
+                return past
+            return torch.cat([past, torch.zeros(B, HN, n_data, bs, dtype=torch.bool, device=dev)], dim=-1)
         cur = torch.ones(n_data, n_in + n_data, dtype=torch.bool, device=dev).tril_(n_in) if compute_incomplete_chunk \
             else torch.zeros(n_data, n_in + n_data, dtype=torch.bool, device=dev)
         return torch.cat([past, cur.view(1, 1, n_data, -1).expand(B, HN, -1, -1)], dim=-1)
@@ -151,7 +163,7 @@ class NAtSLayerCache:
         first, last = self.n_attn_blocks_max, _cdiv(start + n_new, bs)
         self.valid_attn_tokens[:, first:last] = True
         end = start + n_new
-        if self.op_for_incomplete_chunk == 'gated_delta_net':
+        if self._linear_only:
             end = end // bs * bs
         return self.attn_k[:, :end], self.attn_v[:, :end]
 

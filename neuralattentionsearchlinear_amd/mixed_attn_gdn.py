@@ -167,6 +167,8 @@ def masked_attention(q, k, v, attn_msk, scale):
     TK, HKV, V = k.shape[1], k.shape[2], v.shape[-1]
     if attn_msk.dim() != 4 or attn_msk.shape[0] != B or attn_msk.shape[2] != TQ or attn_msk.shape[3] != TK:
         raise ValueError(f"attn_msk must be [B, heads, {TQ}, {TK}], got {tuple(attn_msk.shape)}")
+    if TK == 0:
+        return q.new_zeros(B, TQ, HQ, V)          # no cached key yet: every query sees nothing
     q = q.contiguous()
 
     def cache_view(t):

@@ -151,8 +151,7 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
             # 64 or more new tokens on a cache that already holds tokens (a second prompt): there is no chunked kernel that
             # starts from cached keys (the reference's attention operator cannot run this case either,
             # src/nats/ops/attns/attns.py:1439,1491), so the tokens go through the decode path in steps of fewer than 64
-            # (one token per step where the mode's decode operator takes a single token)
-            step = 1 if self.ops_for_incomplete_chunks == 'gated_delta_net' else 63
+            step = 63
             kw = dict(past_key_values=past_key_values, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
             outs = [self.forward(hidden_states[:, t:t + step], attention_mask, **kw)[0] for t in range(0, q_len, step)]
             return torch.cat(outs, 1), None, past_key_values
@@ -160,9 +159,6 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
             raise NotImplementedError("packed sequences are not supported together with a cache")
 
         if cache is not None and mode != 'chunk' and q_len > 1:
-            # refuse BEFORE the cache is touched: a refused step must leave it as it was
-            if self.ops_for_incomplete_chunks == 'gated_delta_net':
-                raise NotImplementedError("several new tokens per decode step are not built for ops_for_incomplete_chunks=gated_delta_net")
             if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
                 # the step crosses a selector-block boundary: the tokens that complete the block first (the block gets its
                 # type and the cache is updated), then the rest as the start of the next block -- what the reference's

@@ -126,17 +126,13 @@ class NeuralAttentionSearchLinearAttnMamba(nn.Module):
             # 64 or more new tokens on a cache that already holds tokens (a second prompt): there is no chunked kernel that
             # starts from cached keys (the reference's attention operator cannot run this case either,
             # src/nats/ops/attns/attns.py:1439,1491), so the tokens go through the decode path in steps of fewer than 64
-            # (one token per step where the mode's decode operator takes a single token)
-            step = 1 if self.ops_for_incomplete_chunks == 'mamba' else 63
+            step = 63
             kw = dict(cache_params=cache_params, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
             return torch.cat([self.forward(hidden_states[:, t:t + step], attention_mask, **kw) for t in range(0, q_len, step)], 1)
         if cache is not None and cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported together with a cache")
 
         if cache is not None and mode != 'chunk' and q_len > 1:
-            # refuse BEFORE the cache is touched: a refused step must leave it as it was
-            if self.ops_for_incomplete_chunks == 'mamba':
-                raise NotImplementedError("several new tokens per decode step are not built for ops_for_incomplete_chunks=mamba")
             if cache._n_tokens_in_nats_block + q_len > self.nats_block_size:
                 # the step crosses a selector-block boundary: the tokens that complete the block first, then the rest as the
                 # start of the next block (src/nats/ops/mamba/fused_recurrent.py handles the two blocks in one call)

@@ -127,7 +127,9 @@ def test_mask_of_the_next_token():
                          + [('gdn', 200, 270, '760M', 'all'), ('gdn', 30, 140, None, 'all')]
                          # the mode in which the linear operator skips the incomplete block: its tokens read the state that
                          # entered the block, and the state advances when the block is complete
-                         + [(k_, a, b, None, 'attn') for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (30, 140))])
+                         + [(k_, a, b, None, 'attn') for k_ in ('gdn', 'mamba') for a, b in ((320, 420), (266, 400), (30, 140))]
+                         # the mode in which the softmax operator skips the incomplete block
+                         + [('gdn', 266, 400, None, 'gated_delta_net'), ('mamba', 30, 140, None, 'mamba')])
 def test_layer_generation_matches_whole_forward(kind, T0, T, geometry, ops):
     """Prefill T0 tokens with a cache, decode up to T token by token (two tokens at a time where the block allows
     it): every output must match the layer's forward over the first T0 tokens resp. the whole sequence at the same
