@@ -122,11 +122,16 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
                   attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
                   incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
                   inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0, return_aux: bool = False,
-                  keep_chunk_states: bool = False):
+                  keep_chunk_states: bool = False, attn_prefix_valid: Optional[torch.Tensor] = None):
     """Shared forward of the mixed operators.  With inference=True it also returns the state at the
     start of the current selector block (4-tuple), as the reference's *_chunk_inference operators do.  With return_aux
     and keep_chunk_states the auxiliary dict also holds what the linear backward would otherwise recompute
-    (`linear_saved`: chunk states, v_new, workspace)."""
+    (`linear_saved`: chunk states, v_new, workspace).
+
+    attn_prefix_valid (bool [B, NP, HN], inference only): k_attn and v_attn start with NP more whole blocks than the other
+    tensors -- cached keys; block j of that prefix is visible to selector head h's queries where the flag is set.  The softmax
+    branch then runs over prefix + tokens with no queries in the prefix (a chunked forward that continues a cache: the
+    reference's attention operator sizes its output by the keys, src/nats/ops/attns/attns.py:1439,1491, and cannot)."""
     if nats_block_size < CHUNK_SIZE:
         raise AssertionError("nats_block_size must be at least the compute chunk (64)")   # mixed_attn_gdn.py:90
     if nats_block_size % CHUNK_SIZE:
@@ -160,7 +165,20 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
     T = q_lattn.shape[1]
     seqs = pack_sequences(cu_seqlens, cu_seqlens_nats, nats_block_size, dev)
 
-    r = route(types, T, nats_block_size, seqs)
+    if attn_prefix_valid is not None:
+        if not inference or seqs is not None:
+            raise NotImplementedError("a key prefix is built for the prefill operators on unpacked input")
+        NP = attn_prefix_valid.shape[1]
+        n_prefix = NP * nats_block_size
+        if k_attn.shape[1] != q_attn.shape[1] + n_prefix or v_attn.shape[1] != k_attn.shape[1]:
+            raise ValueError(f"with a prefix of {NP} blocks the keys must hold {q_attn.shape[1] + n_prefix} tokens, got {k_attn.shape[1]}")
+        pv = attn_prefix_valid.to(types.dtype)
+        types_attn = torch.cat([torch.stack([pv, 1 - pv], -1), types], 1).contiguous()
+        q_attn = torch.cat([q_attn.new_zeros(q_attn.shape[0], n_prefix, *q_attn.shape[2:]), q_attn], 1)
+        r = route(types_attn, T + n_prefix, nats_block_size, None)
+    else:
+        n_prefix, types_attn = 0, types
+        r = route(types, T, nats_block_size, seqs)
     cur = torch.cuda.current_stream(dev)
     n_chains = (seqs.n_seqs if seqs is not None else q_lattn.shape[0]) * q_lattn.shape[2]
     side = _get_attn_stream(dev) if _run_side_by_side(dev, n_chains, v_lattn.shape[-1]) else cur
@@ -169,8 +187,10 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
     with torch.cuda.stream(side):
         _mark("softmax:start", side)
         o_attn, _lse, _ = parallel_attn_nats_fwd(
-            q_attn, k_attn, v_attn, types, r['nats_block_indices'], None, scale_attn, nats_block_size,
+            q_attn, k_attn, v_attn, types_attn, r['nats_block_indices'], None, scale_attn, nats_block_size,
             compute_incomplete_chunk_scores=attn_same_block, n_nats_blocks=r['n_nats_blocks'], seqs=seqs)
+        if n_prefix:
+            o_attn = o_attn[:, n_prefix:]
         _mark("softmax:end", side)
     flags = (_capi.DECAY_NON_LINEAR if decay_non_linear else 0) | (_capi.QK_L2NORM if qk_l2norm else 0) | \
             (_capi.INTRA_CHUNK if lin_intra else 0)
@@ -185,7 +205,7 @@ def _mixed_forward_impl(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn,
         cur.wait_stream(side)
         # tensors allocated on the caller's stream and read on the side stream, and the side stream's own output
         # that the caller's stream goes on to use
-        for t in (q_attn, k_attn, v_attn, types, r['nats_block_indices'], r['n_nats_blocks']):
+        for t in (q_attn, k_attn, v_attn, types_attn, r['nats_block_indices'], r['n_nats_blocks']):
             t.record_stream(side)
         o_attn.record_stream(cur)
         _lse.record_stream(cur)
@@ -293,7 +313,7 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
                   attn_same_block: bool, lin_intra: bool, output_final_state: bool, decay_non_linear: bool,
                   incomplete_block_start_with_ht: bool, use_g_for_attn: bool, qk_l2norm: bool,
                   inference: bool = False, op_type_last_chunk=None, n_tokens_in_current_block: int = 0,
-                  dnats_invalid_attn: bool = False, dnats_invalid_linear: bool = False):
+                  dnats_invalid_attn: bool = False, dnats_invalid_linear: bool = False, attn_prefix_valid=None):
     """Entry of the mixed operators: the plain forward, or, when a tensor requires grad, the differentiable operator."""
     tensors = (q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initial_state, g, beta, nats_block_types)
     # (the prefill operators are plain functions in the reference too: their outputs carry no gradient)
@@ -302,7 +322,9 @@ def mixed_forward(kind, q_attn, k_attn, v_attn, q_lattn, k_lattn, v_lattn, initi
                                    nats_block_types, scale_attn, scale_lattn, cu_seqlens, cu_seqlens_nats, nats_block_size,
                                    attn_sw_size, attn_same_block, lin_intra, output_final_state, decay_non_linear,
                                    incomplete_block_start_with_ht, use_g_for_attn, qk_l2norm, inference, op_type_last_chunk,
-                                   n_tokens_in_current_block)
+                                   n_tokens_in_current_block, attn_prefix_valid=attn_prefix_valid)
+    if attn_prefix_valid is not None:
+        raise NotImplementedError("a key prefix is built for the prefill operators (no gradient)")
     if attn_sw_size is not None or use_g_for_attn or not incomplete_block_start_with_ht:
         raise NotImplementedError("attn_sw_size / use_g_for_attn / incomplete_block_start_with_ht=False are not built")
     cfg = dict(kind=kind, scale_attn=float(scale_attn), scale_lattn=float(scale_lattn), block=int(nats_block_size),

@@ -87,9 +87,12 @@ def nats_mixed_attn_gdn_chunk_inference(
         incomplete_block_start_with_ht: bool = True,
         use_g_for_attn: bool = False,
         lattn_use_qk_l2norm_in_kernel: bool = True,
+        attn_prefix_valid: torch.Tensor | None = None,
 ):
     """Prefill variant (src/nats/ops/mixed_ops/mixed_attn_gdn.py:328-440):
-    -> (o_gated_delta_net, o_attn, final_state, state at the start of the current block)."""
+    -> (o_gated_delta_net, o_attn, final_state, state at the start of the current block).
+    attn_prefix_valid (not in the reference): k_attn / v_attn start with that many more whole blocks of cached keys, visible
+    per selector head where the flag is set; see _mixed_common._mixed_forward_impl."""
     strategy = all_incomplete_ops[ops_for_incomplete_chunks]
     if scale_attn is None:
         scale_attn = k_attn.shape[-1] ** -0.5
@@ -102,7 +105,7 @@ def nats_mixed_attn_gdn_chunk_inference(
         output_final_state=output_final_state_gated_delta, decay_non_linear=decay_for_non_gdn_blocks,
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
         qk_l2norm=lattn_use_qk_l2norm_in_kernel, inference=True, op_type_last_chunk=op_type_last_chunk,
-        n_tokens_in_current_block=n_tokens_in_current_block)
+        n_tokens_in_current_block=n_tokens_in_current_block, attn_prefix_valid=attn_prefix_valid)
 
 
 def fused_recurrent_gated_delta_rule_nats_fwd(q, k, v, g, g_cumsum, beta, nats_block_types, n_tokens_in_current_block,

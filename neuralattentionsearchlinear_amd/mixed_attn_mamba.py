@@ -78,10 +78,13 @@ def nats_mixed_attn_mamba_chunk_inference(
         decay_for_non_mamba_blocks: bool = True,
         incomplete_block_start_with_ht: bool = True,
         use_g_for_attn: bool = False,
+        attn_prefix_valid: torch.Tensor | None = None,
 ):
     """Prefill variant (src/nats/ops/mixed_ops/mixed_attn_mamba.py:363-457):
     -> (o_mamba, o_attn, final_state, state at the start of the current block).
-    As in the reference, scale_lattn defaults to K**-0.5 HERE (and to 1 in nats_mixed_attn_mamba)."""
+    As in the reference, scale_lattn defaults to K**-0.5 HERE (and to 1 in nats_mixed_attn_mamba).
+    attn_prefix_valid (not in the reference): k_attn / v_attn start with that many more whole blocks of cached keys, visible
+    per selector head where the flag is set; see _mixed_common._mixed_forward_impl."""
     strategy = all_incomplete_ops[ops_for_incomplete_chunks]
     if scale_attn is None:
         scale_attn = k_attn.shape[-1] ** -0.5
@@ -94,7 +97,7 @@ def nats_mixed_attn_mamba_chunk_inference(
         output_final_state=output_final_state_mamba, decay_non_linear=decay_for_non_mamba_blocks,
         incomplete_block_start_with_ht=incomplete_block_start_with_ht, use_g_for_attn=use_g_for_attn,
         qk_l2norm=False, inference=True, op_type_last_chunk=op_type_last_chunk,
-        n_tokens_in_current_block=n_tokens_in_current_block)
+        n_tokens_in_current_block=n_tokens_in_current_block, attn_prefix_valid=attn_prefix_valid)
 
 
 def fused_recurrent_mamba_nats_fwd(q, k, v, g, g_cumsum, nats_block_types, n_tokens_in_current_block, nats_block_size, scale,

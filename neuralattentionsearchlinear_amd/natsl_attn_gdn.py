@@ -6,10 +6,10 @@ and the output norm-gate are the HIP kernels of this package.  Training works, w
 branch (natsl_softmax_sparse_bwd), the linear branch (natsl_linear_chunk_bwd), the short convolutions
 (natsl_short_conv_bwd), the row norms (natsl_row_norm_bwd) and the norm-gate (natsl_norm_gate_bwd); only the block pooling's
 backward (a broadcast of the block's gradient) and the projections are torch operations.  With a NAtSCache
-the layer prefills once in chunk mode on the empty cache and then decodes in steps of fewer than 64 tokens;
-64 or more new tokens on a cache that already holds tokens run through that decode path in steps (there is no chunked
-kernel that starts from cached keys; the reference's attention operator cannot run this case at all: it sizes its
-output by the keys, src/nats/ops/attns/attns.py:1439,1491).
+the layer prefills in chunk mode and decodes in steps of fewer than 64 tokens; 64 or more new tokens on a cache that already
+holds tokens (a second prompt) run through the chunked operators again, the linear branch from the state that entered the
+incomplete block and the softmax branch with the kept blocks as a key prefix (the reference's attention operator cannot run
+this case: it sizes its output by the keys, src/nats/ops/attns/attns.py:1439,1491).
 """
 from __future__ import annotations
 
@@ -145,16 +145,10 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
         cache = self._layer_cache(past_key_values)
         if cache is None and mode != 'chunk':
             raise ValueError("fewer than 64 tokens are decoded on a cache: pass past_key_values")
-        if cache is not None and mode == 'chunk' and cache.n_observed_tokens > 0:
-            if cu_seqlens is not None:
-                raise NotImplementedError("packed sequences are not supported together with a cache")
-            # 64 or more new tokens on a cache that already holds tokens (a second prompt): there is no chunked kernel that
-            # starts from cached keys (the reference's attention operator cannot run this case either,
-            # src/nats/ops/attns/attns.py:1439,1491), so the tokens go through the decode path in steps of fewer than 64
-            step = 63
-            kw = dict(past_key_values=past_key_values, use_cache=use_cache, output_attentions=output_attentions, **kwargs)
-            outs = [self.forward(hidden_states[:, t:t + step], attention_mask, **kw)[0] for t in range(0, q_len, step)]
-            return torch.cat(outs, 1), None, past_key_values
+        # 64 or more new tokens on a cache that already holds tokens (a second prompt): the chunked operators run again, the
+        # linear branch from the state that entered the incomplete block (its cached tokens in front of the new ones), the
+        # softmax branch with the kept blocks as a key prefix
+        continuing = cache is not None and mode == 'chunk' and cache.n_observed_tokens > 0
         if cache is not None and cu_seqlens is not None:
             raise NotImplementedError("packed sequences are not supported together with a cache")
 
@@ -220,6 +214,19 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
             k_attn, v_attn = cache.update_attn_cache((k_attn, v_attn), nats_block_types=raw_types)
             k, v, beta, g = cache.update_lattn_cache((k, v), beta, g, mode, self.ops_for_incomplete_chunks)
             state, state_block_start, g_cumsum = cache.recurrent_state, cache.recurrent_state_block_start, cache.g_cumsum
+        n_cached, prefix_valid = 0, None
+        if continuing:
+            # keys: the kept blocks, the incomplete block's cached tokens, the new tokens -- the cache's buffer as it lies; the
+            # linear inputs came back with the incomplete block's tokens in front; the queries of those tokens are not needed
+            n_cached = cache._n_tokens_in_nats_block
+            n_keys = cache.n_attn_tokens_max + q_len
+            k_attn, v_attn = cache.attn_k[:, :n_keys], cache.attn_v[:, :n_keys]
+            if cache.n_attn_blocks_max > 0:
+                prefix_valid = cache.valid_attn_tokens[:, :cache.n_attn_blocks_max]
+            if n_cached:
+                front = lambda t: torch.cat([t.new_zeros(t.shape[0], n_cached, *t.shape[2:]), t], 1)
+                q, q_attn = front(q), front(q_attn)
+                state = state_block_start
 
         common = dict(q_attn=q_attn, k_attn=k_attn, v_attn=v_attn, q_lattn=q, k_lattn=k, v_lattn=v, g=g, beta=beta,
                       scale_attn=k_attn.shape[-1] ** -0.5, scale_lattn=k.shape[-1] ** -0.5, cu_seqlens=cu_seqlens,
@@ -244,8 +251,10 @@ class NeuralAttentionSearchLinearAttnGDN(nn.Module):
                 state_block_start = None
             else:
                 o_lin, o_attn, state, state_block_start = nats_mixed_attn_gdn_chunk_inference(
-                    initial_state_gated_delta_chunk_start=state_block_start, nats_block_types=types, n_nats_blocks=n_nats_blocks,
+                    initial_state_gated_delta_chunk_start=state if continuing else state_block_start, nats_block_types=types,
+                    n_nats_blocks=n_nats_blocks, attn_prefix_valid=prefix_valid,
                     op_type_last_chunk=last_type if k.shape[1] % self.nats_block_size == 0 else None, **common)
+                o_lin, o_attn = o_lin[:, n_cached:], o_attn[:, n_cached:]
         else:
             attn_msk = cache.generate_msk(n_data=q_len, nats_block_types=raw_types,
                                           compute_incomplete_chunk=self.ops_for_incomplete_chunks != 'gated_delta_net')

@@ -215,12 +215,15 @@ def test_decode_step_across_a_block_boundary(kind):
         assert rel_l2(a2.float(), b2.float()) <= 1e-3
 
 
-@pytest.mark.parametrize("kind", ['gdn', 'mamba'])
-def test_long_continuation_on_a_filled_cache(kind):
-    """64 or more new tokens on a cache that already holds tokens (a second prompt) run through the decode path in steps:
-    same outputs and cache state as the tokens one at a time, and close to the whole forward."""
+@pytest.mark.parametrize("kind,ops,T0,T1", [('gdn', 'all', 100, 300), ('mamba', 'all', 100, 300), ('gdn', 'all', 128, 319),
+                                            ('gdn', 'all', 30, 94), ('gdn', 'gated_delta_net', 100, 300), ('mamba', 'mamba', 70, 290),
+                                            ('gdn', 'attn', 100, 300), ('mamba', 'attn', 192, 256)])
+def test_long_continuation_on_a_filled_cache(kind, ops, T0, T1):
+    """64 or more new tokens on a cache that already holds tokens (a second prompt) run through the chunked operators -- the
+    linear branch from the state that entered the incomplete block, the softmax branch with the kept blocks as a key prefix:
+    outputs close to the tokens fed one at a time and to the whole forward, the same cache afterwards."""
     from neuralattentionsearchlinear_amd.cache import NAtSCache, NAtSMamba2Cache
-    layer, cfg, w, x = _layer_case(kind)
+    layer, cfg, w, x = _layer_case(kind, None, ops)
     layer.layer_idx = 0
     layer = layer.to(DEV).to(torch.bfloat16).eval()
     xd = x.to(DEV).bfloat16()                                           # 320 tokens
@@ -230,12 +233,17 @@ def test_long_continuation_on_a_filled_cache(kind):
     with torch.no_grad():
         whole = first(layer(xd))
         a_h, b_h = mk(), mk()
-        layer(xd[:, :100], **kw(a_h))
-        layer(xd[:, :100], **kw(b_h))
-        a = first(layer(xd[:, 100:300], **kw(a_h)))                     # 200 tokens at once
-        b = torch.cat([first(layer(xd[:, t:t + 1], **kw(b_h))) for t in range(100, 300)], 1)
-    assert a.shape == b.shape == (2, 200, xd.shape[-1])
-    assert rel_l2(a.float(), b.float()) <= 1e-3, f"against single-token steps: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
-    assert rel_l2(a.float(), whole[:, 100:300].float()) <= 2e-2, f"against the whole forward: rel-L2 {rel_l2(a.float(), whole[:, 100:300].float()):.3e}"
+        layer(xd[:, :T0], **kw(a_h))
+        layer(xd[:, :T0], **kw(b_h))
+        a = first(layer(xd[:, T0:T1], **kw(a_h)))                       # at once
+        b = torch.cat([first(layer(xd[:, t:t + 1], **kw(b_h))) for t in range(T0, T1)], 1)
+        # and both caches go on to give the same next token
+        a2, b2 = (first(layer(xd[:, T1:T1 + 1], **kw(h))) for h in (a_h, b_h)) if T1 < xd.shape[1] else (None, None)
+    assert a.shape == b.shape == (2, T1 - T0, xd.shape[-1])
+    assert rel_l2(a.float(), b.float()) <= 1e-2, f"against single-token steps: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
+    assert rel_l2(a.float(), whole[:, T0:T1].float()) <= 2e-2, f"against the whole forward: rel-L2 {rel_l2(a.float(), whole[:, T0:T1].float()):.3e}"
     ca, cb = (h[0] if kind == 'gdn' else h.nats_cache[0] for h in (a_h, b_h))
-    assert ca.n_observed_tokens == cb.n_observed_tokens == 300 and torch.equal(ca.n_attn_blocks, cb.n_attn_blocks)
+    assert torch.equal(ca.n_attn_blocks, cb.n_attn_blocks)
+    if a2 is not None:
+        assert ca.n_observed_tokens == cb.n_observed_tokens == T1 + 1
+        assert rel_l2(a2.float(), b2.float()) <= 1e-2, f"the next token: rel-L2 {rel_l2(a2.float(), b2.float()):.3e}"

@@ -193,3 +193,40 @@ def test_mamba_chunk_inference_block_start_state():
         o, _, S, S_start = nats_mixed_attn_mamba_chunk_inference(*_to(q, k, v, q, k, v), None, g.to(DEV), forced.to(DEV), true_ty[:, -1].to(DEV),
                                                                  None, scale_lattn=1, nats_block_size=block)
     assert_close(o.float(), o_ref, "o_mamba"); assert_close(S, S_ref, "final_state"); assert_close(S_start, S_start_ref, "block_start_state")
+
+
+@pytest.mark.parametrize("mode", ['all', 'gated_delta_net'])
+def test_chunk_inference_with_a_key_prefix(mode):
+    """attn_prefix_valid: the keys start with cached blocks (per selector head visible or not) that have no queries; the new
+    tokens' softmax output against a dense fp32 masked softmax over prefix + tokens, the linear branch and the states
+    against the call without a prefix (they do not see it)."""
+    from oracle import softmax_branch as SB
+    from neuralattentionsearchlinear_amd.mixed_attn_gdn import nats_mixed_attn_gdn_chunk_inference
+    B, T, H, HN, K, V, block, NP = 2, 200, 4, 2, 64, 128, 64, 3
+    q, k, v = make_qkv(B, T, H, K, V, 70)
+    g, beta = make_gates(B, T, H, 71)
+    gen = torch.Generator().manual_seed(72)
+    kp, vp = torch.randn(B, NP * block, H, K, generator=gen).bfloat16(), torch.randn(B, NP * block, H, V, generator=gen).bfloat16()
+    valid = torch.rand(B, NP, HN, generator=gen) < 0.6
+    ty = make_types(B, -(-T // block), HN, 0.5, 73, torch.bfloat16)
+    nb = ty.to(torch.int32).sum(1)
+    d = lambda t: t.to(DEV)
+    kw = dict(q_lattn=d(q), k_lattn=d(k), v_lattn=d(v), initial_state_gated_delta_chunk_start=None, g=d(g), beta=d(beta),
+              nats_block_types=d(ty), op_type_last_chunk=None, n_nats_blocks=d(nb), nats_block_size=block,
+              ops_for_incomplete_chunks=mode, output_final_state_gated_delta=True, decay_for_non_gdn_blocks=True)
+    o_l, o_a, s, s0 = nats_mixed_attn_gdn_chunk_inference(q_attn=d(q), k_attn=d(torch.cat([kp, k], 1)), v_attn=d(torch.cat([vp, v], 1)),
+                                                          attn_prefix_valid=d(valid), **kw)
+    o_l0, o_a0, s_0, s0_0 = nats_mixed_attn_gdn_chunk_inference(q_attn=d(q), k_attn=d(k), v_attn=d(v), **kw)
+    assert torch.equal(o_l, o_l0) and torch.equal(s, s_0) and torch.equal(s0, s0_0)
+    assert o_a.shape == o_a0.shape
+    same_block = mode == 'all'
+    for b in range(B):
+        for h in range(H):
+            hn = h // (H // HN)
+            m_new = SB.visibility_mask(ty[b, :, hn, 0].float(), T, block, same_block)                       # [T, T]
+            m_pre = valid[b, :, hn].repeat_interleave(block).view(1, -1).expand(T, -1)                     # [T, NP*block]
+            mask = torch.cat([m_pre, m_new], 1)
+            sc = (q[b, :, h].float() @ torch.cat([kp, k], 1)[b, :, h].float().T) * K ** -0.5
+            p = torch.softmax(sc.masked_fill(~mask, float('-inf')), -1).nan_to_num(0.0)
+            ref = p @ torch.cat([vp, v], 1)[b, :, h].float()
+            assert_close(o_a[b, :, h].float(), ref, f"o_attn[{b},:,{h}] with a key prefix")
