@@ -2,8 +2,8 @@
 the reference layer (src/nats/layers/natsl_attn_mamba2.py:100-599).  Same scope as the Gated-DeltaNet
 layer: trainable with the same HIP backwards (natsl_softmax_sparse_bwd, natsl_linear_chunk_bwd in its Mamba form,
 natsl_short_conv_bwd, natsl_row_norm_bwd, natsl_norm_gate_bwd; the pooling's backward and the projections are torch
-operations); with a cache, one chunked prefill on the empty cache and then decode steps of
-fewer than 64 tokens (longer inputs on a filled cache are fed through the decode path in such steps)."""
+operations); with a cache, chunked prefill (also of a second prompt on a filled cache: the kept blocks as a key prefix, the
+linear branch from the state that entered the incomplete block) and decode steps of fewer than 64 tokens."""
 from __future__ import annotations
 
 import math
