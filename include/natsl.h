@@ -168,6 +168,9 @@ size_t natsl_linear_workspace_bytes(int64_t total_chunks, int H);
  * per-chunk states as `h`, src/nats/ops/common/chunk_delta_h.py:681-683); NULL = not stored.
  * chunk_v_new (optional, for a backward): the delta rule's corrected values v_new of every token, bf16 [B*T][H][V] (the
  * reference's `v_new`, chunk_delta_h.py:684); NULL = not stored.
+ * The workspace is scratch between the entry's two kernels and its contents are the entry's own business, except after a call
+ * with chunk_states: then it holds what natsl_linear_chunk_bwd reads (per chunk and head TmB, P and four scale vectors).  A
+ * call without chunk_states may leave P out (a launch that fills the GPU forms it inside its second kernel).
  * Replaces l2norm_fwd + chunk_gated_delta_rule_nats_fwd
  * (src/nats/ops/mixed_ops/mixed_attn_gdn.py:119-164, src/nats/ops/gated_delta_rule/chunk.py:22-167). */
 int natsl_gdn_chunk_fwd(const void* q, const void* k, const void* v, const float* g, const void* beta,
