@@ -36,7 +36,7 @@
 // and the delta rule's v_new of every token; natsl_linear_bwd.hip reads them, and TmB from the workspace.
 //
 // The Mamba form has no solve: its prep is mamba_scale_kernel (the scale vectors only; q and k are not read), and the
-// scan forms P itself, in registers, from the k and q tiles of the stage.
+// scan's data-movement waves form P from the k and q tiles of the stage.
 #include "natsl_device.h"
 #include "natsl_host.h"
 
@@ -439,13 +439,13 @@ NATSL_DEVICE s16x4 lds_tr4_at(const unsigned addr) {
 }
 
 // LDS layout of the scan kernel: two or three stages and two output tiles.
-template <int DK, int NW, bool PF = false>
+template <int DK, int NW, bool PF = false, bool XVEC = false>
 struct ScanLds {
   static constexpr int BVW = 16 * NW;                 // state columns of the workgroup
   static constexpr int KROW = DK * 2;                 // bytes per k / q row
   static constexpr int VROW = BVW * 2;                // bytes per v row
-  // (with PF, P is formed and used within one step: one area for all stages, behind them; and two more scale vectors arrive)
-  static constexpr int KB = 64 * KROW, VB = 64 * VROW, TB = 6 * 1024, PB = PF ? 0 : 6 * 1024, SCB = PF ? 2048 : 1024;
+  // (with PF, P is formed and used within one step: one area for all stages, behind them; XVEC: two more scale vectors arrive)
+  static constexpr int KB = 64 * KROW, VB = 64 * VROW, TB = 6 * 1024, PB = PF ? 0 : 6 * 1024, SCB = XVEC ? 2048 : 1024;
   static constexpr int PSHARED = PF ? 6 * 1024 : 0;
   static constexpr int OFF_K = 0, OFF_Q = OFF_K + KB, OFF_V = OFF_Q + KB, OFF_T = OFF_V + VB, OFF_P = OFF_T + TB, OFF_SC = OFF_P + PB;
   static constexpr int STAGE = OFF_SC + SCB;
@@ -471,14 +471,16 @@ NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t
   __launch_bounds__(64 * (NW + 2)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
 
 // NW compute waves (16 state columns each) + two data-movement waves.
-// PF (delta rule, four compute waves): P does not come from the workspace; the two data-movement waves form it from the
-// stage's k and q tiles while the compute waves work on the state (three of the six A operands each, written to the stage's
-// P area), take the q rows' reciprocal norms from the operands they read for that and complete sq; a second barrier in the
-// middle of the step hands both over.
+// PF (the Mamba form always; the delta rule in its four-wave shape when the launch asks for it): P does not come from the
+// workspace; the two data-movement waves form it from the stage's k and q tiles while the compute waves work on the state (two
+// of the four row tiles each, written to one P area shared by all stages); for the delta rule they also take the q rows'
+// reciprocal norms from the operands they read for that and complete sq.  A second barrier in the middle of the step hands it
+// over.
 template <int DK, bool DELTA, int NW, bool PF>
 __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p) {
-  static_assert(!PF || (DELTA && NW == 4), "P is formed in the scan only by the four-wave delta-rule shape");
-  using L = ScanLds<DK, NW, PF>;
+  static_assert(!PF || !DELTA || NW == 4, "the delta rule's P is formed by the data-movement waves only in the four-wave shape");
+  static_assert(PF || DELTA, "the Mamba form's P is always formed by the data-movement waves");
+  using L = ScanLds<DK, NW, PF, PF && DELTA>;
   constexpr int KS = DK / 32;   // matrix k-steps over the key dimension
   constexpr int KT = DK / 16;   // 16-row state tiles
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -523,6 +525,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     for (int s = 0; s < KS; ++s) a_kq[s] = (unsigned)(i16 * L::KROW) + 16u * (unsigned)((4 * s + g4) ^ kq_swizzle<DK>(i16));
     const unsigned a_sc = 16u * g4;
     const bool l2n = (p.flags & NATSL_QK_L2NORM) != 0;
+    const float log2_scale_m = __builtin_amdgcn_logf(p.scale);
     const size_t qk_pitch = (size_t)p.H * DK * 2, v_pitch = (size_t)p.H * p.V * 2;   // bytes per token
     const char* kb = reinterpret_cast<const char*>(p.k + ((size_t)bos * p.H + h) * DK);
     const ptrdiff_t q_minus_k = reinterpret_cast<const char*>(p.q) - reinterpret_cast<const char*>(p.k);
@@ -571,7 +574,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
       if (first) {
         // in the order the compute waves need them: sc, k (R = k S comes first), q
         dma16(sb, 16u * lane, st + L::OFF_SC);
-        if (PF) dma16(pb, 16u * lane, st + L::OFF_SC + 1024);   // the two exponent vectors (and 512 bytes nobody reads)
+        if (PF && DELTA) dma16(pb, 16u * lane, st + L::OFF_SC + 1024);   // the two exponent vectors (and 512 bytes nobody reads)
 #pragma unroll
         for (int u = 0; u < KQ_PIECES; ++u) dma16(kb, kq_off[u], st + L::OFF_K + 1024 * u);
 #pragma unroll
@@ -629,7 +632,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     // stores issued after them) may still be in flight at the barrier: vector memory operations complete in the order
     // they were issued, so allowing as many outstanding as one step issues leaves exactly the older step's complete.
     constexpr int AHEAD = L::NSTAGE - 1;
-    constexpr int PER_STEP_FIRST = 1 + (PF ? 1 : 0) + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? (PF ? 6 : 12) : 0) + O_PASSES;
+    constexpr int PER_STEP_FIRST = 1 + (PF && DELTA ? 1 : 0) + 2 * KQ_PIECES, PER_STEP_SECOND = V_PIECES + (DELTA ? (PF ? 6 : 12) : 0) + O_PASSES;
     static_assert(PER_STEP_FIRST <= 63 && PER_STEP_SECOND <= 63, "the wait counter has six bits");
     constexpr int VM_FIRST = (PER_STEP_FIRST & 15) | ((PER_STEP_FIRST >> 4) << 14) | 0x0f70;
     constexpr int VM_SECOND = (PER_STEP_SECOND & 15) | ((PER_STEP_SECOND >> 4) << 14) | 0x0f70;
@@ -661,15 +664,17 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
 #pragma unroll
           for (int s = 0; s < KS; ++s)
             if (t2 <= tmax) ka[t2][s] = *reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + t2 * 16 * L::KROW);
+        // the exponents: two vectors of their own from the delta rule's prep; gamma log2(e) (vector 0) for both in the Mamba form
+        constexpr int GK_ROW = DELTA ? 4 : 0, GQ_ROW = DELTA ? 5 : 0;
         f32x4 gj[4];
 #pragma unroll
         for (int t2 = 0; t2 < 4; ++t2)
-          if (t2 <= tmax) gj[t2] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * (4 * C) + a_sc + 64 * t2);
+          if (t2 <= tmax) gj[t2] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * (GK_ROW * C) + a_sc + 64 * t2);
         float gq[2], sq0[2];
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-          gq[w] = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (5 * C + 16 * tr[w] + i16));
-          sq0[w] = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (C + 16 * tr[w] + i16));
+          gq[w] = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (GQ_ROW * C + 16 * tr[w] + i16)) + (DELTA ? 0.f : log2_scale_m);
+          sq0[w] = DELTA ? *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (C + 16 * tr[w] + i16)) : 0.f;
         }
         f32x4 D[2], Z[2][4];
 #pragma unroll
@@ -682,7 +687,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         for (int s = 0; s < KS; ++s)
 #pragma unroll
           for (int w = 0; w < 2; ++w) {
-            D[w] = mfma16(qb[w][s], qb[w][s], D[w]);
+            if (DELTA) D[w] = mfma16(qb[w][s], qb[w][s], D[w]);
 #pragma unroll
             for (int t2 = 0; t2 < 4; ++t2)
               if (t2 <= tr[w]) Z[w][t2] = mfma16(ka[t2][s], qb[w][s], Z[w][t2]);
@@ -691,9 +696,12 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         float rqi[2];
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-          const float dsel = rsel == 0 ? D[w][0] : rsel == 1 ? D[w][1] : rsel == 2 ? D[w][2] : D[w][3];
-          const float ss = __shfl(dsel, 16 * (i16 >> 2) + i16);
-          rqi[w] = l2n ? rsqrtf(ss + 1e-6f) : 1.f;
+          rqi[w] = 1.f;
+          if (DELTA) {
+            const float dsel = rsel == 0 ? D[w][0] : rsel == 1 ? D[w][1] : rsel == 2 ? D[w][2] : D[w][3];
+            const float ss = __shfl(dsel, 16 * (i16 >> 2) + i16);
+            rqi[w] = l2n ? rsqrtf(ss + 1e-6f) : 1.f;
+          }
         }
 #pragma unroll
         for (int w = 0; w < 2; ++w)
@@ -712,7 +720,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
           for (int sp = 0; sp < 2; ++sp)
             if (2 * sp <= tr[w])
               *reinterpret_cast<__attribute__((address_space(3))) bf16x8*>(lds0 + L::OFF_PS + 1024 * tri_slot(tr[w], sp) + 16 * lane) = pack8(Z[w][2 * sp], Z[w][2 * sp + 1]);
-          if (g4 == 0) {
+          if (DELTA && g4 == 0) {
             typedef __attribute__((address_space(3))) float* lds_fw_t;
             *reinterpret_cast<lds_fw_t>(st + L::OFF_SC + 4 * (C + 16 * tr[w] + i16)) = sq0[w] * rqi[w];
           }
@@ -798,7 +806,6 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
   const unsigned a_sc = 16u * g4;    // this lane group's four tokens in a row of sc
 
   float gsum = 0.f;
-  const float log2_scale = __builtin_amdgcn_logf(p.scale);
   __syncthreads();   // chunk 0 has landed
 
   for (int c = 0; c < NT; ++c) {
@@ -947,48 +954,8 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
 #pragma unroll
       for (int t = 0; t < 4; ++t) O[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + 4 * C + a_sc + 64 * t);
       if (intra) {
-        if constexpr (DELTA) {
 #pragma unroll
-          for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>((PF ? lds0 + L::OFF_PS : st + L::OFF_P) + 1024 * v + 16 * lane);
-        } else {
-          // P = scale tril(q k^T e^{gamma_i - gamma_j}) formed here, from the tiles of this stage: Z^T = k_tile(t') q_tile(t)^T
-          // leaves lane (i16, g4) with query 16 t + i16 against keys 16 t' + 4 g4 .. + 3 -- the four slots this lane holds of
-          // A operand (t, t' / 2), half t' % 2 (see the operand order above); both inputs are plain row reads, the k rows as
-          // A operand, the q rows as B operand (a lane's eight contraction slots = 16 bytes of its row).
-          f32x4 gj[4];
-#pragma unroll
-          for (int t = 0; t < 4; ++t) gj[t] = *reinterpret_cast<lds_f4_t>(st + L::OFF_SC + a_sc + 64 * t);
-          f32x4 Wt[4][4];
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            // (gamma comes in log2 units; the scale rides along as log2(scale))
-            const float gi = *reinterpret_cast<lds_f1_t>(st + L::OFF_SC + 4 * (16 * t + i16)) + log2_scale;
-#pragma unroll
-            for (int t2 = 0; t2 < 4; ++t2) {
-              Wt[t][t2] = (f32x4){0.f, 0.f, 0.f, 0.f};
-              if (t2 <= t) {
-                f32x4 Z = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s = 0; s < KS; ++s) {
-                  const bf16x8 ka = *reinterpret_cast<lds_b128_t>(st + L::OFF_K + a_kq[s] + t2 * 16 * L::KROW);
-                  const bf16x8 qb = *reinterpret_cast<lds_b128_t>(st + L::OFF_Q + a_kq[s] + t * 16 * L::KROW);
-                  Z = mfma16(ka, qb, Z);
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                  const float w = Z[r] * __builtin_amdgcn_exp2f(gi - gj[t2][r]);
-                  Wt[t][t2][r] = (t2 < t || i16 >= 4 * g4 + r) ? w : 0.f;
-                }
-              }
-            }
-          }
-          PA[tri_slot(0, 0)] = pack8(Wt[0][0], Wt[0][1]);
-          PA[tri_slot(1, 0)] = pack8(Wt[1][0], Wt[1][1]);
-          PA[tri_slot(2, 0)] = pack8(Wt[2][0], Wt[2][1]);
-          PA[tri_slot(2, 1)] = pack8(Wt[2][2], Wt[2][3]);
-          PA[tri_slot(3, 0)] = pack8(Wt[3][0], Wt[3][1]);
-          PA[tri_slot(3, 1)] = pack8(Wt[3][2], Wt[3][3]);
-        }
+        for (int v = 0; v < 6; ++v) PA[v] = *reinterpret_cast<lds_b128_t>((PF ? lds0 + L::OFF_PS : st + L::OFF_P) + 1024 * v + 16 * lane);
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t)
@@ -1046,7 +1013,7 @@ inline int cu_count_linear() {
 
 template <int DK, bool DELTA, int NW, bool PF>
 static int launch_scan(const LinearParams& p, hipStream_t stream, const char* what) {
-  using L = ScanLds<DK, NW, PF>;
+  using L = ScanLds<DK, NW, PF, PF && DELTA>;
   auto kern = linear_scan_kernel<DK, DELTA, NW, PF>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
@@ -1092,14 +1059,21 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
   }
   int rc = check_launch(what);
   if (rc != NATSL_OK) return rc;
-  if (nw == 4) {
-    if constexpr (CAN_PF) {
-      if (pf) return launch_scan<DK, true, 4, true>(p, stream, what);
+  if constexpr (!DELTA) {
+    // the Mamba form's P is always formed by the data-movement waves (nothing about it comes from a prep kernel)
+    if (nw == 4) return launch_scan<DK <= 128 ? DK : 128, false, 4, true>(p, stream, what);
+    if (nw == 2) return launch_scan<DK, false, 2, true>(p, stream, what);
+    return launch_scan<DK, false, 1, true>(p, stream, what);
+  } else {
+    if (nw == 4) {
+      if constexpr (CAN_PF) {
+        if (pf) return launch_scan<DK, true, 4, true>(p, stream, what);
+      }
+      return launch_scan<DK <= 128 ? DK : 128, true, 4, false>(p, stream, what);
     }
-    return launch_scan<DK <= 128 ? DK : 128, DELTA, 4, false>(p, stream, what);
+    if (nw == 2) return launch_scan<DK, true, 2, false>(p, stream, what);
+    return launch_scan<DK, true, 1, false>(p, stream, what);
   }
-  if (nw == 2) return launch_scan<DK, DELTA, 2, false>(p, stream, what);
-  return launch_scan<DK, DELTA, 1, false>(p, stream, what);
 }
 
 static int linear_fwd(bool delta, const void* q, const void* k, const void* v, const float* g, const void* beta,
