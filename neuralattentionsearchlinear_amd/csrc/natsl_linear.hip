@@ -468,7 +468,7 @@ NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t
 // second register file and every vector operation on the state costs two extra copies).
 #define NATSL_SCAN_FITS_256(DK) ((DK) <= 128)
 #define NATSL_SCAN_ATTR(DK, NW) \
-  __launch_bounds__(64 * (NW + 2)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
+  __launch_bounds__(64 * ((NW) + 2)) __attribute__((amdgpu_waves_per_eu(NATSL_SCAN_FITS_256(DK) ? 2 : 1, NATSL_SCAN_FITS_256(DK) ? 2 : 1)))
 
 // NW compute waves (16 state columns each) + two data-movement waves.
 // PF (the Mamba form always; the delta rule in its four-wave shape when the launch asks for it): P does not come from the
@@ -476,8 +476,12 @@ NATSL_DEVICE constexpr int tri_slot(const int t, const int s) { return t < 2 ? t
 // of the four row tiles each, written to one P area shared by all stages); for the delta rule they also take the q rows'
 // reciprocal norms from the operands they read for that and complete sq.  A second barrier in the middle of the step hands it
 // over.
-template <int DK, bool DELTA, int NW, bool PF>
-__global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p) {
+// NF = 2 (with four compute waves): two more waves that do nothing but form P (waves NW + 2, NW + 3), so that this work sits on
+// the two SIMDs that host no data-movement wave; with NF = 0 the data-movement waves form P themselves (they have a SIMD of
+// their own when there are one or two compute waves).
+template <int DK, bool DELTA, int NW, bool PF, int NF = 0>
+__global__ NATSL_SCAN_ATTR(DK, NW + NF) void linear_scan_kernel(const LinearParams p) {
+  static_assert(NF == 0 || (NF == 2 && PF), "the extra waves only form P");
   static_assert(!PF || !DELTA || NW == 4, "the delta rule's P is formed by the data-movement waves only in the four-wave shape");
   static_assert(PF || DELTA, "the Mamba form's P is always formed by the data-movement waves");
   using L = ScanLds<DK, NW, PF, PF && DELTA>;
@@ -519,6 +523,9 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     // store the output tile of chunk c - 1 (wave NW + 1), wait for the requests, meet the barrier.  The compute waves
     // never touch global memory inside the loop.  (One wave issues about 1 KiB per 36 cycles; two share the 53 KiB.)
     const bool first = wave == NW;
+    const bool moves = wave < NW + 2;                          // requests, output stores
+    const bool forms = NF == 0 || wave >= NW + 2;              // P (with PF)
+    const bool rows30 = ((wave - NW) & 1) == 0;                // which two row tiles of P this wave forms
     // (operand addresses of the k / q tiles and of a row of the scale vectors, as the compute waves use them below)
     unsigned a_kq[KS];
 #pragma unroll
@@ -636,9 +643,11 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
     static_assert(PER_STEP_FIRST <= 63 && PER_STEP_SECOND <= 63, "the wait counter has six bits");
     constexpr int VM_FIRST = (PER_STEP_FIRST & 15) | ((PER_STEP_FIRST >> 4) << 14) | 0x0f70;
     constexpr int VM_SECOND = (PER_STEP_SECOND & 15) | ((PER_STEP_SECOND >> 4) << 14) | 0x0f70;
+    if (moves) {
 #pragma unroll
-    for (int a = 0; a < AHEAD; ++a)
-      if (a < NT) request(a);
+      for (int a = 0; a < AHEAD; ++a)
+        if (a < NT) request(a);
+    }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     if constexpr (PF) {
@@ -730,13 +739,17 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         // requests go into the stage that step c - 1 read: every wave is past the barrier that ended it
         const bool more = c + AHEAD < NT;
         const unsigned st = lds0 + (c % L::NSTAGE) * L::STAGE;
-        if (more) request(c + AHEAD);
-        if (c > 0 && !first) store_out(c - 1);
-        // five tiles each: rows 48..63 and 0..15 here, rows 32..47 and 16..31 there
-        if (first) form_two_rows(3, 0, st);
-        else form_two_rows(2, 1, st);
+        if (moves) {
+          if (more) request(c + AHEAD);
+          if (c > 0 && !first) store_out(c - 1);
+        }
+        if (forms) {
+          // five tiles each: rows 48..63 and 0..15 here, rows 32..47 and 16..31 there
+          if (rows30) form_two_rows(3, 0, st);
+          else form_two_rows(2, 1, st);
+        }
         __syncthreads();   // hand-over of P and sq in the middle of the compute waves' step
-        if (AHEAD == 2 && more) {
+        if (AHEAD == 2 && more && moves) {
           if (first) __builtin_amdgcn_s_waitcnt(VM_FIRST);
           else __builtin_amdgcn_s_waitcnt(VM_SECOND);
         } else {
@@ -759,7 +772,7 @@ __global__ NATSL_SCAN_ATTR(DK, NW) void linear_scan_kernel(const LinearParams p)
         __syncthreads();
       }
     }
-    if (NT > 0 && !first) store_out(NT - 1);
+    if (NT > 0 && !first && moves) store_out(NT - 1);
     return;
   }
 
@@ -1011,15 +1024,15 @@ inline int cu_count_linear() {
   return n;
 }
 
-template <int DK, bool DELTA, int NW, bool PF>
+template <int DK, bool DELTA, int NW, bool PF, int NF = 0>
 static int launch_scan(const LinearParams& p, hipStream_t stream, const char* what) {
   using L = ScanLds<DK, NW, PF, PF && DELTA>;
-  auto kern = linear_scan_kernel<DK, DELTA, NW, PF>;
+  auto kern = linear_scan_kernel<DK, DELTA, NW, PF, NF>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL);
   if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, L::TOTAL, hipGetErrorString(e));
   const int n_chains = (p.seqs ? p.n_seqs : p.B) * p.H;
   const int grid = 8 * cdiv(n_chains, 8) * (p.V / L::BVW);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (NW + 2)), L::TOTAL, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (NW + 2 + NF)), L::TOTAL, stream, p);
   return check_launch(what);
 }
 
@@ -1061,13 +1074,15 @@ static int launch_linear(const LinearParams& p, hipStream_t stream, const char* 
   if (rc != NATSL_OK) return rc;
   if constexpr (!DELTA) {
     // the Mamba form's P is always formed by the data-movement waves (nothing about it comes from a prep kernel)
-    if (nw == 4) return launch_scan<DK <= 128 ? DK : 128, false, 4, true>(p, stream, what);
+    // (four compute waves: two of them share their SIMD with a data-movement wave, so two more waves, on the other two
+    // SIMDs, form P -- B8 T4096 H16 d128: 137 -> 132 us; the delta rule at B8 T8192 H16: 428 -> 398 us)
+    if (nw == 4) return launch_scan<DK <= 128 ? DK : 128, false, 4, true, 2>(p, stream, what);
     if (nw == 2) return launch_scan<DK, false, 2, true>(p, stream, what);
     return launch_scan<DK, false, 1, true>(p, stream, what);
   } else {
     if (nw == 4) {
       if constexpr (CAN_PF) {
-        if (pf) return launch_scan<DK, true, 4, true>(p, stream, what);
+        if (pf) return launch_scan<DK, true, 4, true, 2>(p, stream, what);
       }
       return launch_scan<DK <= 128 ? DK : 128, true, 4, false>(p, stream, what);
     }
