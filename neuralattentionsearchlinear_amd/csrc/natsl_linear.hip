@@ -37,6 +37,10 @@
 //
 // The Mamba form has no solve: its prep is mamba_scale_kernel (the scale vectors only; q and k are not read), and the
 // scan's data-movement waves form P from the k and q tiles of the stage.
+//
+// The delta rule has a second form of the pair for launches that fill the GPU and need no backward ("PF" below): the prep
+// reads k only and leaves no P (two more scale vectors in its place), and the scan forms P from the staged k and q tiles in
+// waves that do not hold the state; a second barrier in the middle of a step hands it to the compute waves.
 #include "natsl_device.h"
 #include "natsl_host.h"
 
