@@ -133,6 +133,7 @@ def test_gdn_and_mamba_scan_with_64_columns_per_workgroup():
     assert B * H * (V // 64) >= _cus()
     _gdn(B, 320, H, 16, 128, V, 64, 0.3, True, seed=26, h0=True)
     _gdn(B, 256, H, 4, 64, V, 128, 0.5, False, seed=27)
+    _gdn(B, 200, H, 8, 128, V, 64, 0.4, True, seed=29, intra=False)      # (this launch forms P in the scan and does not use it)
     _mamba(B, 256, H, 8, 128, V, 64, 0.3, True, seed=28, h0=True)
 
 
