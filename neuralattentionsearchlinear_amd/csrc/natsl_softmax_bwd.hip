@@ -7,7 +7,10 @@
 //                  block, and every later chunk when the block is typed attention), for every query head of the group:
 //                  S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS, dnats += sum dS over later blocks (attns.py:719-983)
 //                  The query tiles (Q, dO, lse, delta) arrive by DMA in a ring of three LDS slots, two steps ahead.
-//                  One persistent workgroup per CU takes units from per-XCD work queues.
+//                  One persistent workgroup per CU takes units from per-XCD work queues.  Eight waves in two roles:
+//                  four form S, P and dV, four form dP, dS and dK of the same (32 keys) x (32 queries) quarters; P
+//                  passes between the two in fp32 through LDS.  Each wave keeps one stationary operand and one
+//                  accumulator, so two waves fit a SIMD.
 //
 // Layouts follow the forward kernel: the stationary operand of a workgroup (Q, dO there; K, V here) sits in registers
 // as the B operand (lane = its row), the streamed tiles are row-major in LDS, the accumulators' own layout is the B
@@ -390,26 +393,52 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const SoftmaxBwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// dk/dv.  Eight waves = 2 roles x 2 key halves x 2 query halves; a wave and its partner of the other role (wave + 4, on
+// the same SIMD) work on the same 32 keys x 32 queries of every step:
+//   role 0: S = Q K^T, P = exp2(S c - lse) (masks, the clamp for blocks that only give dnats), dV^T += dO^T P
+//   role 1: dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS, dnats
+// P goes from role 0 to role 1 in fp32 through LDS (two buffers, written before the step's barrier and read after it).
+// Each wave holds one stationary operand (K or V rows) and one accumulator (dV or dK) of its 32 keys: under 256
+// registers, so two waves share a SIMD and one's exponentials run under the other's matrix instructions.
+struct DkdvShared {
+  int unit_pair, unit_jc, unit_seq;
+  float red[4];
+};
+
 template <int DK, int DV>
-__global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) {
-  constexpr int KS = DK / 16, VS = DV / 16, DT = DK / 32, VT = DV / 32;
-  extern __shared__ __align__(16) unsigned char smem[];
-  __shared__ float red[4];
+struct DkdvLds {
+  static constexpr int QROWB = DK * 2, DROWB = DV * 2;
+  static constexpr unsigned DOFF = 64 * QROWB, LOFF = DOFF + 64 * DROWB, SLOT = LOFF + 512;   // slot: Q [64][DK], dO [64][DV], lse [64], delta [64]
+  static constexpr unsigned XOFF = 3 * SLOT, XBUF = 4 * 4096;   // P exchange: [2][4 wave pairs][4][64 lanes] of 4 floats
+  static constexpr unsigned RING = XOFF + 2 * XBUF;
+  static constexpr unsigned RED = 2u * (DV / 32 + DK / 32) * 16 * 64 * sizeof(float);   // the unit's end: sums of the query halves
+  static constexpr unsigned TOTAL = RING > RED ? RING : RED;
+};
+
+template <int DK, int DV, int ROLE>
+NATSL_DEVICE void dkdv_role(const SoftmaxBwdParams& p, unsigned char* smem, DkdvShared& sh) {
+  typedef DkdvLds<DK, DV> L;
+  // the first product contracts over D1 against the rows of tile 1 (Q for role 0, dO for role 1); the second product
+  // gives D2 rows from tile 2 transposed (dO for role 0, Q for role 1)
+  constexpr int D1 = ROLE == 0 ? DK : DV, D2 = ROLE == 0 ? DV : DK;
+  constexpr int S1 = D1 / 16, T2 = D2 / 32, VT = DV / 32, DT = DK / 32;
+  constexpr int ROWB1 = D1 * 2, ROWB2 = D2 * 2;
+  constexpr unsigned OFF1 = ROLE == 0 ? 0u : L::DOFF, OFF2 = ROLE == 0 ? L::DOFF : 0u;
+  constexpr unsigned SLOT = L::SLOT, LOFF = L::LOFF;
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int quad = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);
   const int l32 = lane & 31, hf = lane >> 5;
-  const int kh = wave & 1, qh = wave >> 1;
+  const int kh = quad & 1, qh = quad >> 1;
   const bool packed = p.seqs != nullptr;
   const int n_pairs = p.B * p.HKV;
-  // ---- Persistent workgroups (one per CU; the kernel's registers and LDS admit no more) take units = (sequence, kv
-  // head, key chunk) from work queues: starting a workgroup per unit left the CUs idle a quarter of the time.
-  // Workgroups that run at the same time should stream the same queries, so every XCD (block index mod 8) has a queue
-  // of its own with the key chunks of one (sequence, kv head) after the other, earliest (heaviest) chunk first, and
-  // every unit walks the later query chunks from the last one down: units started together stay together in L2.  A
-  // workgroup whose queue is empty takes from the other XCDs' queues.
-  // Packed sequences: one queue, the units of a sequence (kv head after kv head) after those of the one before.
-  __shared__ int unit_pair, unit_jc, unit_seq;
+  // ---- Persistent workgroups (one per CU) take units = (sequence, kv head, key chunk) from work queues: starting a
+  // workgroup per unit left the CUs idle a quarter of the time.  Workgroups that run at the same time should stream the
+  // same queries, so every XCD (block index mod 8) has a queue of its own with the key chunks of one (sequence, kv
+  // head) after the other, earliest (heaviest) chunk first, and every unit walks the later query chunks from the last
+  // one down: units started together stay together in L2.  A workgroup whose queue is empty takes from the other
+  // XCDs' queues.  Packed sequences: one queue, the units of a sequence (kv head after kv head) after those of the one
+  // before.
   const int NT_reg = (p.T + 63) >> 6;
   const bool per_xcd = !packed && n_pairs % 8 == 0;
   const int n_queues = per_xcd ? 8 : 1;
@@ -429,7 +458,7 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
             const int r = i - p.seqs[sn].chunk_off * p.HKV, ntc = (p.seqs[sn].eos - p.seqs[sn].bos + 63) >> 6;
             pr = r / ntc;   // the kv head
             jj = r % ntc;
-            unit_seq = sn;
+            sh.unit_seq = sn;
           } else {
             pr = per_xcd ? (i / NT_reg) * 8 + x : i / NT_reg;
             jj = i % NT_reg;
@@ -438,405 +467,347 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const SoftmaxBwdParams p) 
         }
         ++q_probe;
       }
-      unit_pair = pr;
-      unit_jc = jj;
+      sh.unit_pair = pr;
+      sh.unit_jc = jj;
     }
     __syncthreads();
-    const int pair = unit_pair, jc = unit_jc, seq = packed ? unit_seq : 0;
+    const int pair = sh.unit_pair, jc = sh.unit_jc, seq = packed ? sh.unit_seq : 0;
     __syncthreads();   // (read before the next round's write)
     if (pair < 0) break;
-  const int n = packed ? seq : pair / p.HKV, hkv = packed ? pair : pair % p.HKV;
-  const int bos = packed ? p.seqs[n].bos : n * p.T, len = packed ? p.seqs[n].eos - bos : p.T;
-  const int bos_nats = packed ? p.seqs[n].bos_nats : n * p.TN;
-  const int NTc = (len + 63) >> 6;
-  const int Bs = p.block, per_blk = Bs >> 6;
-  const int G = p.HQ / p.HKV, GN = p.HQ / p.HN;
-  const int kb = (jc * 64) / Bs;
-  const int blk_end_chunk = min((kb + 1) * per_blk, NTc);    // one past the last chunk of the key block
+    const int n = packed ? seq : pair / p.HKV, hkv = packed ? pair : pair % p.HKV;
+    const int bos = packed ? p.seqs[n].bos : n * p.T, len = packed ? p.seqs[n].eos - bos : p.T;
+    const int bos_nats = packed ? p.seqs[n].bos_nats : n * p.TN;
+    const int NTc = (len + 63) >> 6;
+    const int Bs = p.block, per_blk = Bs >> 6;
+    const int G = p.HQ / p.HKV, GN = p.HQ / p.HN;
+    const int kb = (jc * 64) / Bs;
+    const int blk_end_chunk = min((kb + 1) * per_blk, NTc);   // one past the last chunk of the key block
 
-  // K and V of the wave's 32 keys as B operands (lane = key)
-  bf16x8 KB[KS], VB[VS];
-  {
-    const int ki = min(jc * 64 + 32 * kh + l32, len - 1);
-    const bf16_t* kr = p.k + ((size_t)(bos + ki) * p.HKV + hkv) * DK + 8 * hf;
+    // the stationary operand: K (role 0) or V (role 1) of the wave's 32 keys as B operands (lane = key)
+    bf16x8 XB[S1];
+    {
+      const int ki = min(jc * 64 + 32 * kh + l32, len - 1);
+      const bf16_t* xr = (ROLE == 0 ? p.k : p.v) + ((size_t)(bos + ki) * p.HKV + hkv) * D1 + 8 * hf;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) KB[s] = ld8(kr + 16 * s);
-    const bf16_t* vr = p.v + ((size_t)(bos + ki) * p.HKV + hkv) * DV + 8 * hf;
-#pragma unroll
-    for (int s = 0; s < VS; ++s) VB[s] = ld8(vr + 16 * s);
-  }
-  f32x16 dv[VT], dk[DT];
-#pragma unroll
-  for (int t = 0; t < VT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dv[t][r] = 0.f;
-#pragma unroll
-  for (int t = 0; t < DT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dk[t][r] = 0.f;
-
-  const float c = p.scale_log2;
-
-  // ---- the ring of query tiles.  Slot layout: Q [64][DK], dO [64][DV], lse [64], delta [64]; rows are unpadded and
-  // the 16-byte segment s of row r sits at position s ^ bwd_swizzle(r).  Tiles arrive by DMA (global -> LDS, no
-  // registers): each instruction fills 1 KiB of a tile, and the swizzle is applied on the global side.
-  constexpr int QROWB = DK * 2, DROWB = DV * 2;
-  constexpr unsigned DOFF = 64 * QROWB, LOFF = DOFF + 64 * DROWB, SLOT = LOFF + 512;
-  constexpr int QI = DK / 32, DI = DV / 32;              // DMA instructions per wave and tile
-  const unsigned lds0 = (unsigned)(size_t)smem;
-  unsigned q_row[QI], q_seg[QI], d_row[DI], d_seg[DI];   // per DMA instruction: the lane's tile row and global byte offset in the row
-#pragma unroll
-  for (int j = 0; j < QI; ++j) {
-    const int pos = lane % (DK / 8), row = (QI * wave + j) * (1024 / QROWB) + lane / (DK / 8);
-    q_row[j] = row;
-    q_seg[j] = 16u * (pos ^ bwd_swizzle<DK>(row));
-  }
-#pragma unroll
-  for (int j = 0; j < DI; ++j) {
-    const int pos = lane % (DV / 8), row = (DI * wave + j) * (1024 / DROWB) + lane / (DV / 8);
-    d_row[j] = row;
-    d_seg[j] = 16u * (pos ^ bwd_swizzle<DV>(row));
-  }
-  // waves 0 and 2 fetch lse, waves 1 and 3 delta (twice the same bytes: every wave then has the same number of requests)
-  const float* l_src = (wave & 1) ? p.delta : p.lse;
-  constexpr int NREQ = QI + DI + 1;   // requests per wave and tile
-  // request piece r of tile jq of head hq into a slot
-  auto piece = [&](const int r, const int hq, const int jq, const int slot, const void*& g, unsigned& voff, unsigned& dst) __attribute__((always_inline)) {
-    const unsigned sl = lds0 + slot * SLOT;
-    if (r < QI) {
-      g = p.q + ((size_t)bos * p.HQ + hq) * DK;
-      voff = (unsigned)min(jq * 64 + (int)q_row[r < QI ? r : 0], len - 1) * ((unsigned)p.HQ * QROWB) + q_seg[r < QI ? r : 0];
-      dst = sl + (QI * wave + r) * 1024;
-    } else if (r < QI + DI) {
-      const int j = r < QI ? 0 : (r < QI + DI ? r - QI : 0);
-      g = p.dout + ((size_t)bos * p.HQ + hq) * DV;
-      voff = (unsigned)min(jq * 64 + (int)d_row[j], len - 1) * ((unsigned)p.HQ * DROWB) + d_seg[j];
-      dst = sl + DOFF + (DI * wave + j) * 1024;
-    } else {
-      g = l_src + (size_t)bos * p.HQ + hq;
-      voff = (unsigned)min(jq * 64 + lane, len - 1) * (unsigned)(p.HQ * 4);
-      dst = sl + LOFF + 256 * (wave & 1);
+      for (int s = 0; s < S1; ++s) XB[s] = ld8(xr + 16 * s);
     }
-  };
-  auto request = [&](const int hq, const int jq, const int slot) __attribute__((always_inline)) {
+    f32x16 acc[T2];
 #pragma unroll
-    for (int r = 0; r < NREQ; ++r) {
+    for (int t = 0; t < T2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+
+    const float c = p.scale_log2;
+
+    // ---- the ring of query tiles.  Rows are unpadded and the 16-byte segment s of row r sits at position
+    // s ^ bwd_swizzle(r).  Tiles arrive by DMA (global -> LDS, no registers): each instruction fills 1 KiB of a tile, and
+    // the swizzle is applied on the global side.  A wave requests its share of its own role's first tile (role 0: Q and
+    // lse, role 1: dO and delta).
+    constexpr int I1 = D1 / 32;   // 1 KiB DMA instructions per wave and tile
+    constexpr int NREQ = I1 + 1;  // requests per wave and tile
+    const unsigned lds0 = (unsigned)(size_t)smem;
+    unsigned r_row[I1], r_seg[I1];   // per DMA instruction: the lane's tile row and global byte offset in the row
+#pragma unroll
+    for (int j = 0; j < I1; ++j) {
+      const int pos = lane % (D1 / 8), row = (I1 * quad + j) * (1024 / ROWB1) + lane / (D1 / 8);
+      r_row[j] = row;
+      r_seg[j] = 16u * (pos ^ bwd_swizzle<D1>(row));
+    }
+    const bf16_t* g_src = ROLE == 0 ? p.q : p.dout;
+    const float* l_src = ROLE == 0 ? p.lse : p.delta;
+    // request piece r of tile jq of head hq into a slot
+    auto piece = [&](const int r, const int hq, const int jq, const int slot, const void*& g, unsigned& voff, unsigned& dst) __attribute__((always_inline)) {
+      const unsigned sl = lds0 + slot * SLOT;
+      if (r < I1) {
+        g = g_src + ((size_t)bos * p.HQ + hq) * D1;
+        voff = (unsigned)min(jq * 64 + (int)r_row[r < I1 ? r : 0], len - 1) * ((unsigned)p.HQ * ROWB1) + r_seg[r < I1 ? r : 0];
+        dst = sl + OFF1 + (I1 * quad + r) * 1024;
+      } else {
+        g = l_src + (size_t)bos * p.HQ + hq;
+        voff = (unsigned)min(jq * 64 + lane, len - 1) * (unsigned)(p.HQ * 4);
+        dst = sl + LOFF + 256 * ROLE;   // (the four waves of a role bring the same 256 bytes)
+      }
+    };
+    auto request = [&](const int hq, const int jq, const int slot) __attribute__((always_inline)) {
+#pragma unroll
+      for (int r = 0; r < NREQ; ++r) {
+        const void* g;
+        unsigned voff, dst;
+        piece(r, hq, jq, slot, g, voff, dst);
+        if (r < I1) dma16(g, voff, dst);
+        else dma4(g, voff, dst);
+      }
+    };
+    auto request_piece_if = [&](const int r, const int hq, const int jq, const int slot, const unsigned on) __attribute__((always_inline)) {
       const void* g;
       unsigned voff, dst;
       piece(r, hq, jq, slot, g, voff, dst);
-      if (r < QI + DI) dma16(g, voff, dst);
-      else dma4(g, voff, dst);
-    }
-  };
-  auto request_piece_if = [&](const int r, const int hq, const int jq, const int slot, const unsigned on) __attribute__((always_inline)) {
-    const void* g;
-    unsigned voff, dst;
-    piece(r, hq, jq, slot, g, voff, dst);
-    if (r < QI + DI) dma16_if(g, voff, dst, on);
-    else dma4_if(g, voff, dst, on);
-  };
+      if (r < I1) dma16_if(g, voff, dst, on);
+      else dma4_if(g, voff, dst, on);
+    };
 
-  // ---- LDS byte offsets of the lane's operands inside a slot
-  typedef __attribute__((address_space(3))) const bf16x8* lds_op;
-  typedef __attribute__((address_space(3))) s16x4* lds_tr;
-  unsigned aq[KS], ad[VS];              // first two products: the lane's query row, k-step st
-  {
-    const int row = 32 * qh + l32;
+    // ---- LDS byte offsets of the lane's operands inside a slot
+    typedef __attribute__((address_space(3))) const bf16x8* lds_op;
+    typedef __attribute__((address_space(3))) s16x4* lds_tr;
+    typedef __attribute__((address_space(3))) f32x4* lds_f4;
+    unsigned a1[S1];   // first product: the lane's query row, k-step st
+    {
+      const int row = 32 * qh + l32;
 #pragma unroll
-    for (int st = 0; st < KS; ++st) aq[st] = row * QROWB + 16u * ((2 * st + hf) ^ bwd_swizzle<DK>(row));
-#pragma unroll
-    for (int st = 0; st < VS; ++st) ad[st] = DOFF + row * DROWB + 16u * ((2 * st + hf) ^ bwd_swizzle<DV>(row));
-  }
-  // last two products: transposing reads.  Within 16 lanes, lane i addresses 4 elements of row 4 hf + i/4 (+ 8 for the
-  // second read) at column 32 t + 16 (lane/16 % 2) + 4 (i % 4).
-  unsigned tq[2][DT][2], td[2][VT][2];
-  {
-    const int i16 = lane & 15;
-#pragma unroll
-    for (int ss = 0; ss < 2; ++ss)
-#pragma unroll
-      for (int rd = 0; rd < 2; ++rd) {
-        const int row = 32 * qh + 16 * ss + 8 * rd + 4 * hf + (i16 >> 2);
-        const int seg0 = 2 * ((lane >> 4) & 1) + ((i16 >> 1) & 1);
-#pragma unroll
-        for (int t = 0; t < DT; ++t) tq[ss][t][rd] = row * QROWB + 16u * ((4 * t + seg0) ^ bwd_swizzle<DK>(row)) + 8u * (i16 & 1);
-#pragma unroll
-        for (int t = 0; t < VT; ++t) td[ss][t][rd] = DOFF + row * DROWB + 16u * ((4 * t + seg0) ^ bwd_swizzle<DV>(row)) + 8u * (i16 & 1);
-      }
-  }
-
-  for (int g = 0; g < G; ++g) {
-    const int hq = hkv * G + g, hn = hq / GN;
-    const bool attn = bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + kb) * p.HN + hn) * 2);
-    const int n_same = p.same_block ? blk_end_chunk - jc : 0;
-    // a block that is not typed attention walks the later queries only when its dnats is asked for, and then for nothing else
-    const bool walk_later = attn || p.dnats_invalid != 0;
-    const int n_later = __builtin_amdgcn_readfirstlane(walk_later ? max(NTc - blk_end_chunk, 0) : 0);   // (the type was read by a vector load)
-    const bool attn_u = __builtin_amdgcn_readfirstlane(attn ? 1 : 0) != 0;
-    const int n_it = n_same + n_later;
-    float dn = 0.f;
-    auto chunk_of = [&](const int it) { return it < n_same ? jc + it : NTc - 1 - (it - n_same); };
-    if (n_it > 0) {
-      __syncthreads();   // the previous head's last reads of the ring are done
-      request(hq, chunk_of(0), 0);
-      if (n_it > 1) {
-        request(hq, chunk_of(1), 1);
-        __builtin_amdgcn_s_waitcnt(0x0f70 | NREQ);   // vmcnt: all but the newest tile's requests
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-      }
-      __syncthreads();
+      for (int st = 0; st < S1; ++st) a1[st] = OFF1 + row * ROWB1 + 16u * ((2 * st + hf) ^ bwd_swizzle<D1>(row));
     }
-    int slot = 0;
-    for (int it = 0; it < n_it; ++it) {
-      const int jq = chunk_of(it);
-      const unsigned sb = lds0 + slot * SLOT;
-      // ---- S^T = Q K^T and dP^T = dO V^T for (32 queries) x (32 keys): one stream of LDS operands, read ahead
-      constexpr int NOPS = KS + VS, AHEAD = 6;
-      constexpr int NPAIR = KS < VS ? KS : VS;
-      auto is_v = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? (j & 1) != 0 : VS > KS; };
-      auto step_of = [&](const int j) __attribute__((always_inline)) { return j < 2 * NPAIR ? j >> 1 : j - NPAIR; };
-      // (equal head dims: the dO tile has the Q tile's layout DOFF bytes further, an immediate offset of the read)
-      constexpr bool SAME = DK == DV;
-      unsigned cq[KS], cd[SAME ? 1 : VS];
+    // second product: transposing reads.  Within 16 lanes, lane i addresses 4 elements of row 4 hf + i/4 (+ 8 for the
+    // second read) at column 32 t + 16 (lane/16 % 2) + 4 (i % 4).
+    unsigned t2[2][T2][2];
+    {
+      const int i16 = lane & 15;
 #pragma unroll
-      for (int st = 0; st < KS; ++st) { cq[st] = sb + aq[st]; asm("" : "+v"(cq[st])); }
-      if constexpr (!SAME) {
+      for (int ss = 0; ss < 2; ++ss)
 #pragma unroll
-        for (int st = 0; st < VS; ++st) { cd[st] = sb + ad[st]; asm("" : "+v"(cd[st])); }
-      }
-      auto ld_op = [&](const int j) __attribute__((always_inline)) -> bf16x8 {
-        if constexpr (SAME) return *reinterpret_cast<lds_op>(cq[step_of(j)] + (is_v(j) ? DOFF : 0u));
-        else return *reinterpret_cast<lds_op>(is_v(j) ? cd[step_of(j)] : cq[step_of(j)]);
-      };
-      f32x16 s, dp;
+        for (int rd = 0; rd < 2; ++rd) {
+          const int row = 32 * qh + 16 * ss + 8 * rd + 4 * hf + (i16 >> 2);
+          const int seg0 = 2 * ((lane >> 4) & 1) + ((i16 >> 1) & 1);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
-      {
-        bf16x8 op[NOPS + AHEAD];
-#pragma unroll
-        for (int j = 0; j < AHEAD; ++j) op[j] = ld_op(j);
-#pragma unroll
-        for (int j = 0; j < NOPS; ++j) {
-          if (j + AHEAD < NOPS) op[j + AHEAD] = ld_op(j + AHEAD);
-          if (is_v(j)) dp = mfma32(op[j], VB[step_of(j)], dp);
-          else s = mfma32(op[j], KB[step_of(j)], s);
+          for (int t = 0; t < T2; ++t) t2[ss][t][rd] = OFF2 + row * ROWB2 + 16u * ((4 * t + seg0) ^ bwd_swizzle<D2>(row)) + 8u * (i16 & 1);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
-#pragma unroll
-        for (int j = 0; j < NOPS; ++j) {
-          if (j + AHEAD < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    const unsigned xlane = lds0 + L::XOFF + quad * 4096 + 16 * lane;   // the wave pair's exchange area, this lane's 16 bytes of group 0
+
+    for (int g = 0; g < G; ++g) {
+      const int hq = hkv * G + g, hn = hq / GN;
+      const bool attn = bwd_type_is_one(p.types, p.types_dtype, ((size_t)(bos_nats + kb) * p.HN + hn) * 2);
+      const int n_same = p.same_block ? blk_end_chunk - jc : 0;
+      // a block that is not typed attention walks the later queries only when its dnats is asked for, and then for nothing else
+      const bool walk_later = attn || p.dnats_invalid != 0;
+      const int n_later = __builtin_amdgcn_readfirstlane(walk_later ? max(NTc - blk_end_chunk, 0) : 0);   // (the type was read by a vector load)
+      const bool attn_u = __builtin_amdgcn_readfirstlane(attn ? 1 : 0) != 0;
+      const int n_it = n_same + n_later;
+      float dn = 0.f;
+      auto chunk_of = [&](const int it) { return it < n_same ? jc + it : NTc - 1 - (it - n_same); };
+      if (n_it > 0) {
+        __syncthreads();   // the previous head's last reads of the ring are done
+        request(hq, chunk_of(0), 0);
+        if (n_it > 1) {
+          request(hq, chunk_of(1), 1);
+          __builtin_amdgcn_s_waitcnt(0x0f70 | NREQ);   // vmcnt: all but the newest tile's requests
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
         }
+        __syncthreads();
       }
-      // ---- the tile of the next step has been requested a whole step ago: once every wave has seen its own requests
-      // land it is complete, and the slot of the previous step is free for the tile two steps ahead
-      __builtin_amdgcn_sched_barrier(0);   // (all matrix instructions are issued first: they drain while the wave waits)
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      __syncthreads();
-      const bool ask = it + 2 < n_it;   // the tile two steps ahead goes into the slot of the previous step
-      const int ask_jq = ask ? chunk_of(it + 2) : 0, ask_slot = slot == 0 ? 2 : slot - 1;
-      // no tile left to ask for: the requests run with no lane enabled (read through a lane so that it sits in scalar registers)
-      const unsigned ask_mask = __builtin_amdgcn_readfirstlane(ask ? 1u : 0u);
-      // ---- dV^T += dO^T P and dK^T += Q^T dS: 16 operands of two transposing reads each, read ahead.  The first of
-      // them and the rows' lse and delta are requested before the exponentials, which then run under the LDS latency.
-      constexpr int N2 = 2 * (VT + DT), A2 = 4;   // operand j: ss = j / (VT + DT); within it the VT value tiles, then the DT key-dim tiles
-      unsigned ct[SAME ? 2 * DT : N2][2];   // equal head dims: one address per (ss, tile) serves both tiles
-      if constexpr (SAME) {
+      int slot = 0;
+      for (int it = 0; it < n_it; ++it) {
+        const int jq = chunk_of(it);
+        const unsigned sb = lds0 + slot * SLOT;
+        const unsigned xb = xlane + (it & 1) * L::XBUF;
+        const bool own = jq == jc;
+        // keys the queries do not see: probabilities against the queries' lse, clamped to 1 as the reference does, enter
+        // dnats only (their dV, dK products run on zeros)
+        const bool only_dn = !attn_u && it >= n_same;
+        // ---- first product, (32 queries) x (32 keys): LDS operands read ahead
+        constexpr int AHEAD = 4;
+        unsigned c1[S1];
 #pragma unroll
-        for (int ss = 0; ss < 2; ++ss)
+        for (int st = 0; st < S1; ++st) { c1[st] = sb + a1[st]; asm("" : "+v"(c1[st])); }
+        f32x16 x;
 #pragma unroll
-          for (int t = 0; t < DT; ++t)
+        for (int r = 0; r < 16; ++r) x[r] = 0.f;
+        {
+          bf16x8 op[S1 + AHEAD];
 #pragma unroll
-            for (int rd = 0; rd < 2; ++rd) {
-              ct[ss * DT + t][rd] = sb + tq[ss][t][rd];
-              asm("" : "+v"(ct[ss * DT + t][rd]));
-            }
-      } else {
+          for (int j = 0; j < AHEAD; ++j) op[j] = *reinterpret_cast<lds_op>(c1[j]);
 #pragma unroll
-        for (int j = 0; j < N2; ++j) {
-          const int ss = j / (VT + DT), u = j % (VT + DT);
+          for (int j = 0; j < S1; ++j) {
+            if (j + AHEAD < S1) op[j + AHEAD] = *reinterpret_cast<lds_op>(c1[j + AHEAD]);
+            x = mfma32(op[j], XB[j], x);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+          for (int j = 0; j < S1; ++j) {
+            if (j + AHEAD < S1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
+        }
+        // the rows' lse (role 0) or delta (role 1)
+        const float* Lb = reinterpret_cast<const float*>(smem + slot * SLOT + LOFF) + 64 * ROLE;
+        f32x4 l4[4];
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) l4[rg] = *reinterpret_cast<const f32x4*>(Lb + 32 * qh + 8 * rg + 4 * hf);
+        // second product: operand j = (ss = j / T2, tile j % T2), two transposing reads each, read ahead; the first
+        // ones are asked for before the barrier (the tile has been complete since the last step)
+        constexpr int N2 = 2 * T2, A2 = 4 < N2 ? 4 : N2;
+        unsigned ct[N2][2];
+#pragma unroll
+        for (int j = 0; j < N2; ++j)
 #pragma unroll
           for (int rd = 0; rd < 2; ++rd) {
-            ct[j][rd] = sb + (u < VT ? td[ss][u < VT ? u : 0][rd] : tq[ss][u < VT ? 0 : u - VT][rd]);
+            ct[j][rd] = sb + t2[j / T2][j % T2][rd];
             asm("" : "+v"(ct[j][rd]));
           }
-        }
-      }
-      auto tr_read = [&](const int j, const int rd) __attribute__((always_inline)) -> s16x4 {
-        if constexpr (SAME) {
-          const int ss = j / (VT + DT), u = j % (VT + DT);
-          return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr>(ct[ss * DT + (u < VT ? u : u - VT)][rd] + (u < VT ? DOFF : 0u)));
-        } else {
+        auto tr_read = [&](const int j, const int rd) __attribute__((always_inline)) -> s16x4 {
           return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_tr>(ct[j][rd]));
+        };
+        s16x4 lo[N2 + A2], hi[N2 + A2];
+        bf16x8 PB[2];
+        float dsum = 0.f;
+        if constexpr (ROLE == 0) {
+          f32x16 pr;
+          if (!own && jq * 64 + 64 <= len) {   // every (query, key) pair of the tile is visible: no masks
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              float e = __builtin_amdgcn_exp2f(fmaf(x[r], c, -l4[r >> 2][r & 3]));
+              if (only_dn) e = fminf(e, 1.f);
+              pr[r] = e;
+            }
+          } else {
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int r = 4 * rg + j;
+                const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
+                const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
+                float e = vis ? __builtin_amdgcn_exp2f(fmaf(x[r], c, -l4[rg][j])) : 0.f;
+                if (only_dn) e = fminf(e, 1.f);
+                pr[r] = e;
+              }
+            }
+          }
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg)
+            *reinterpret_cast<lds_f4>(xb + 1024 * rg) = f32x4{pr[4 * rg], pr[4 * rg + 1], pr[4 * rg + 2], pr[4 * rg + 3]};
+#pragma unroll
+          for (int ss = 0; ss < 2; ++ss) PB[ss] = only_dn ? bf16x8{} : pack8(pr, ss);
         }
-      };
-      const float* Lb = reinterpret_cast<const float*>(smem + slot * SLOT + LOFF);
-      f32x4 l4[4], d4[4];
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        l4[rg] = *reinterpret_cast<const f32x4*>(Lb + 32 * qh + 8 * rg + 4 * hf);
-        d4[rg] = *reinterpret_cast<const f32x4*>(Lb + 64 + 32 * qh + 8 * rg + 4 * hf);
-      }
-      s16x4 lo[N2 + A2], hi[N2 + A2];
-#pragma unroll
-      for (int j = 0; j < A2; ++j) {
-        lo[j] = tr_read(j, 0);
-        hi[j] = tr_read(j, 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      f32x16 pr, ds;
-      const bool own = jq == jc;
-      // keys the queries do not see: probabilities against the queries' lse, clamped to 1 as the reference does, enter
-      // dnats only (their dV, dK products run on zeros)
-      const bool only_dn = !attn_u && it >= n_same;
-      float dsum = 0.f;
-      if (!own && jq * 64 + 64 <= len) {   // every (query, key) pair of the tile is visible: no masks
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float e = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[r >> 2][r & 3]));
-          if (only_dn) e = fminf(e, 1.f);
-          pr[r] = e;
-          ds[r] = e * (dp[r] - d4[r >> 2][r & 3]);
-          dsum += ds[r];
+        for (int j = 0; j < A2; ++j) {
+          lo[j] = tr_read(j, 0);
+          hi[j] = tr_read(j, 1);
         }
-      } else {
+        // ---- the tile of the next step has been requested a whole step ago: once every wave has seen its own requests
+        // land it is complete, and the slot of the previous step is free for the tile two steps ahead
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        const bool ask = it + 2 < n_it;   // the tile two steps ahead goes into the slot of the previous step
+        const int ask_jq = ask ? chunk_of(it + 2) : 0, ask_slot = slot == 0 ? 2 : slot - 1;
+        // no tile left to ask for: the requests run with no lane enabled (read through a lane so that it sits in scalar registers)
+        const unsigned ask_mask = __builtin_amdgcn_readfirstlane(ask ? 1u : 0u);
+        if constexpr (ROLE == 1) {
+          f32x4 p4[4];
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
+          for (int rg = 0; rg < 4; ++rg) p4[rg] = *reinterpret_cast<lds_f4>(xb + 1024 * rg);
+          f32x16 ds;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int r = 4 * rg + j;
-            const int qloc = 32 * qh + 8 * rg + 4 * hf + j;
-            const bool vis = jq * 64 + qloc < len && (!own || 32 * kh + l32 <= qloc);
-            float e = vis ? __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[rg][j])) : 0.f;
-            if (only_dn) e = fminf(e, 1.f);
-            pr[r] = e;
-            ds[r] = e * (dp[r] - d4[rg][j]);
+          for (int r = 0; r < 16; ++r) {
+            ds[r] = p4[r >> 2][r & 3] * (x[r] - l4[r >> 2][r & 3]);
             dsum += ds[r];
           }
+          if (it >= n_same && jc * 64 + 32 * kh + l32 < len) dn += dsum;
+#pragma unroll
+          for (int ss = 0; ss < 2; ++ss) PB[ss] = only_dn ? bf16x8{} : pack8(ds, ss);
         }
-      }
-      if (it >= n_same && jc * 64 + 32 * kh + l32 < len) dn += dsum;
-      bf16x8 PB[2][2];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ss = 0; ss < 2; ++ss) { PB[ss][0] = pack8(pr, ss); PB[ss][1] = pack8(ds, ss); }
-      if (only_dn) {
-#pragma unroll
-        for (int ss = 0; ss < 2; ++ss) PB[ss][0] = PB[ss][1] = bf16x8{};
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < N2; ++j) {
-        if (j + A2 < N2) {
-          lo[j + A2] = tr_read(j + A2, 0);
-          hi[j + A2] = tr_read(j + A2, 1);
+        for (int j = 0; j < N2; ++j) {
+          if (j + A2 < N2) {
+            lo[j + A2] = tr_read(j + A2, 0);
+            hi[j + A2] = tr_read(j + A2, 1);
+          }
+          acc[j % T2] = mfma32(join4(lo[j], hi[j]), PB[j / T2], acc[j % T2]);
+          if (j < NREQ) request_piece_if(j, hq, ask_jq, ask_slot, ask_mask);   // one request under each matrix instruction
         }
-        const int ss = j / (VT + DT), u = j % (VT + DT);
-        if (u < VT) dv[u < VT ? u : 0] = mfma32(join4(lo[j], hi[j]), PB[ss][0], dv[u < VT ? u : 0]);
-        else dk[u < VT ? 0 : u - VT] = mfma32(join4(lo[j], hi[j]), PB[ss][1], dk[u < VT ? 0 : u - VT]);
-        if (j < NREQ) request_piece_if(j, hq, ask_jq, ask_slot, ask_mask);   // one request under each matrix instruction
-      }
-      static_assert(NREQ <= N2, "requests are issued under the matrix instructions");
 #pragma unroll
-      for (int j = 0; j < N2; ++j) {
-        if (j + A2 < N2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-      slot = slot == 2 ? 0 : slot + 1;
-    }
-    // dnats of this (key block, query head): the four waves' sums
-    if (n_later > 0) {
+        for (int j = N2; j < NREQ; ++j) request_piece_if(j, hq, ask_jq, ask_slot, ask_mask);
 #pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) dn += __shfl_xor(dn, m);
-      if (lane == 0) red[wave] = dn;
-      __syncthreads();
-      if (tid == 0) atomicAdd(p.dnats + ((size_t)(bos_nats + kb)) * p.HQ + hq, red[0] + red[1] + red[2] + red[3]);
-      __syncthreads();
+        for (int j = 0; j < N2; ++j) {
+          if (j + A2 < N2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        slot = slot == 2 ? 0 : slot + 1;
+      }
+      // dnats of this (key block, query head): the sums of role 1's four waves
+      if (n_later > 0) {
+        if constexpr (ROLE == 1) {
+#pragma unroll
+          for (int m = 32; m >= 1; m >>= 1) dn += __shfl_xor(dn, m);
+          if (lane == 0) sh.red[quad] = dn;
+        }
+        __syncthreads();
+        if (ROLE == 1 && quad == 0 && lane == 0)
+          atomicAdd(p.dnats + ((size_t)(bos_nats + kb)) * p.HQ + hq, sh.red[0] + sh.red[1] + sh.red[2] + sh.red[3]);
+        __syncthreads();
+      }
     }
-  }
 
-  // ---- the two query halves of a key half are summed through LDS, then the tiles are transposed and stored
-  __syncthreads();
-  f32x4* Rs = reinterpret_cast<f32x4*>(smem);   // [2 key halves][(VT + DT) * 4 register groups][64 lanes] of 4 floats
-  if (qh == 1) {
-    f32x4* dst = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
+    // ---- the two query halves of a key half are summed through LDS, then the tiles are transposed and stored: role 0
+    // its dV tiles, role 1 its dK tiles
+    constexpr int TB = ROLE == 0 ? 0 : VT;   // this role's first tile in the order (dV tiles, dK tiles)
+    __syncthreads();
+    f32x4* Rs = reinterpret_cast<f32x4*>(smem);   // [2 key halves][(VT + DT) * 4 register groups][64 lanes] of 4 floats
+    if (qh == 1) {
+      f32x4* dst = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
+      for (int t = 0; t < T2; ++t)
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) dst[(t * 4 + rg) * 64] = f32x4{dv[t][4 * rg], dv[t][4 * rg + 1], dv[t][4 * rg + 2], dv[t][4 * rg + 3]};
+        for (int rg = 0; rg < 4; ++rg) dst[((TB + t) * 4 + rg) * 64] = f32x4{acc[t][4 * rg], acc[t][4 * rg + 1], acc[t][4 * rg + 2], acc[t][4 * rg + 3]};
+    }
+    __syncthreads();
+    if (qh == 0) {
+      // (all reads first, then the sums)
+      const f32x4* src = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
+      f32x4 xs[T2 * 4];
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+      for (int i = 0; i < T2 * 4; ++i) xs[i] = src[(TB * 4 + i) * 64];
+      const float mul = ROLE == 0 ? 1.f : p.scale;
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) dst[((VT + t) * 4 + rg) * 64] = f32x4{dk[t][4 * rg], dk[t][4 * rg + 1], dk[t][4 * rg + 2], dk[t][4 * rg + 3]};
-  }
-  __syncthreads();
-  if (qh == 0) {
-    // (all reads first, then the sums: a read-wait-add sequence per value took 5000 cycles)
-    const f32x4* src = Rs + (size_t)kh * (VT + DT) * 4 * 64 + lane;
-    f32x4 x[(VT + DT) * 4];
+      for (int t = 0; t < T2; ++t)
 #pragma unroll
-    for (int i = 0; i < (VT + DT) * 4; ++i) x[i] = src[i * 64];
+        for (int r = 0; r < 16; ++r) acc[t][r] = (acc[t][r] + xs[t * 4 + (r >> 2)][r & 3]) * mul;
+    }
+    __syncthreads();
+    if (qh == 0) {
+      // accumulators are [value or dim rows x key columns]: write [key][value|dim] rows to LDS, then coalesced stores
+      constexpr int OP = DV + DK + 8, CB = ROLE == 0 ? 0 : DV;
+      bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + kh * 32 * OP + CB;
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
+      for (int t = 0; t < T2; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dv[t][r] += x[t * 4 + (r >> 2)][r & 3];
+        for (int rg = 0; rg < 4; ++rg) {
+          u32x2 w;
+          w[0] = pack_bf16x2(acc[t][4 * rg], acc[t][4 * rg + 1]);
+          w[1] = pack_bf16x2(acc[t][4 * rg + 2], acc[t][4 * rg + 3]);
+          *reinterpret_cast<u32x2*>(Os + l32 * OP + 32 * t + 8 * rg + 4 * hf) = w;
+        }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+      // all LDS reads first, then the stores
+      constexpr int NS = 32 * (D2 / 8) / 64;
+      u32x4 w2[NS];
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dk[t][r] = (dk[t][r] + x[(VT + t) * 4 + (r >> 2)][r & 3]) * p.scale;
-  }
-  __syncthreads();
-  if (qh == 0) {
-    // accumulators are [value or dim rows x key columns]: write [key][value|dim] rows to LDS, then coalesced stores
-    constexpr int OP = DV + DK + 8;
-    bf16_t* Os = reinterpret_cast<bf16_t*>(smem) + kh * 32 * OP;
-#pragma unroll
-    for (int t = 0; t < VT; ++t)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 w;
-        w[0] = pack_bf16x2(dv[t][4 * rg], dv[t][4 * rg + 1]);
-        w[1] = pack_bf16x2(dv[t][4 * rg + 2], dv[t][4 * rg + 3]);
-        *reinterpret_cast<u32x2*>(Os + l32 * OP + 32 * t + 8 * rg + 4 * hf) = w;
+      for (int i = 0; i < NS; ++i) {
+        const int e = lane + 64 * i, row = e / (D2 / 8), seg = e % (D2 / 8);
+        w2[i] = *reinterpret_cast<const u32x4*>(Os + row * OP + seg * 8);
       }
+      const int t_base = jc * 64 + 32 * kh;
+      bf16_t* out = ROLE == 0 ? p.dv : p.dk;
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 w;
-        w[0] = pack_bf16x2(dk[t][4 * rg], dk[t][4 * rg + 1]);
-        w[1] = pack_bf16x2(dk[t][4 * rg + 2], dk[t][4 * rg + 3]);
-        *reinterpret_cast<u32x2*>(Os + l32 * OP + DV + 32 * t + 8 * rg + 4 * hf) = w;
+      for (int i = 0; i < NS; ++i) {
+        const int e = lane + 64 * i, row = e / (D2 / 8), seg = e % (D2 / 8);
+        if (t_base + row < len) *reinterpret_cast<u32x4*>(out + ((size_t)(bos + t_base + row) * p.HKV + hkv) * D2 + seg * 8) = w2[i];
       }
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    __builtin_amdgcn_wave_barrier();
-    // all LDS reads first, then the stores (a read-wait-store sequence per piece took 4000 cycles)
-    constexpr int NV = 32 * (DV / 8) / 64, NK = 32 * (DK / 8) / 64;
-    u32x4 wv[NV], wk[NK];
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int e = lane + 64 * i, row = e / (DV / 8), seg = e % (DV / 8);
-      wv[i] = *reinterpret_cast<const u32x4*>(Os + row * OP + seg * 8);
     }
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int e = lane + 64 * i, row = e / (DK / 8), seg = e % (DK / 8);
-      wk[i] = *reinterpret_cast<const u32x4*>(Os + row * OP + DV + seg * 8);
-    }
-    const int t_base = jc * 64 + 32 * kh;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int e = lane + 64 * i, row = e / (DV / 8), seg = e % (DV / 8);
-      if (t_base + row < len) *reinterpret_cast<u32x4*>(p.dv + ((size_t)(bos + t_base + row) * p.HKV + hkv) * DV + seg * 8) = wv[i];
-    }
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int e = lane + 64 * i, row = e / (DK / 8), seg = e % (DK / 8);
-      if (t_base + row < len) *reinterpret_cast<u32x4*>(p.dk + ((size_t)(bos + t_base + row) * p.HKV + hkv) * DK + seg * 8) = wk[i];
-    }
-  }
-  __syncthreads();   // the staging area is the next unit's tile ring
+    __syncthreads();   // the staging area is the next unit's tile ring
   }  // units
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(512, 1) void dkdv_kernel(const SoftmaxBwdParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ DkdvShared sh;
+  // (wave-uniform: each role runs the same sequence of workgroup barriers)
+  if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 8) == 0) dkdv_role<DK, DV, 0>(p, smem, sh);
+  else dkdv_role<DK, DV, 1>(p, smem, sh);
 }
 
 // number of CUs of the current device (one persistent dk/dv workgroup each)
@@ -867,16 +838,14 @@ static int launch_bwd(const SoftmaxBwdParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
   }
   {
-    size_t lds = (size_t)3 * (64 * (DK + DV) * sizeof(bf16_t) + 512);   // the ring of three query tiles
-    const size_t red = (size_t)2 * (DV / 32 + DK / 32) * 16 * 64 * sizeof(float);
-    if (red > lds) lds = red;
+    const size_t lds = DkdvLds<DK, DV>::TOTAL;   // the ring of three query tiles and the exchange buffers
     auto kern = dkdv_kernel<DK, DV>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(NATSL_ERR_LAUNCH, "softmax bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     const long long units = p.seqs ? (long long)p.total_chunks * p.HKV : (long long)p.B * p.HKV * ((p.T + 63) / 64);
     long long grid = (cu_count() + 7) / 8 * 8;   // whole groups of 8: block index mod 8 names the XCD and its queue
     if (grid > units) grid = units;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, p);
   }
   return check_launch("natsl_softmax_sparse_bwd");
 }
